@@ -1,0 +1,140 @@
+/*
+ * snd_scan.h — C ABI of the MI355X (gfx950) 2D-CrossScan selective scan, forward and backward.
+ *
+ * This is the drop-in boundary for the reference's one operator pair
+ *     fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay) -> [out, x, x_v, x_sd]
+ *     bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd)
+ *         -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
+ * (reference: kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:179-187,286-297,442-445).
+ *
+ * Plain pointers and sizes only.  The library never allocates device memory, never synchronises
+ * and never throws: every entry point returns an int status (0 = ok, negative = error) and
+ * enqueues its work on the HIP stream it is given.  The caller (the PyTorch extension, or any
+ * other host) validates ownership, allocates outputs / checkpoints / workspace and passes them in.
+ *
+ * Tensor layouts are the reference's (selective_scan_oflex.cpp:206-229):
+ *     u      [batch, dim, nrows, ncols]            input dtype, last dim contiguous
+ *     delta  [batch, delta_dim, nrows, ncols]      input dtype, last dim contiguous
+ *     A      [dim, dstate]                         fp32
+ *     B, C   [batch, n_groups, dstate, nrows, ncols] input dtype, last dim contiguous
+ *     D      [dim] fp32 (optional), delta_bias [delta_dim] fp32 (optional), A_decay [1] fp32 (optional)
+ *     out    [batch, dim, nrows, ncols]            fp32 or input dtype
+ * dim % n_groups == 0, dim % delta_dim == 0, dstate <= 16.  All strides are in ELEMENTS.
+ */
+#ifndef SND_SCAN_H
+#define SND_SCAN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SND_MAX_DSTATE 16          /* selective_scan_common.h:13 (MAX_DSTATE) */
+
+typedef void *snd_stream_t;        /* a hipStream_t, passed opaquely */
+
+typedef enum snd_dtype { SND_F32 = 0, SND_F16 = 1, SND_BF16 = 2 } snd_dtype;
+
+typedef enum snd_status {
+    SND_OK = 0,
+    SND_ERR_NULL = -1,             /* a required pointer is null */
+    SND_ERR_SHAPE = -2,            /* sizes violate the reference's checks (host.cpp:215-245) */
+    SND_ERR_DTYPE = -3,            /* unsupported dtype combination (host.cpp:190-195) */
+    SND_ERR_STRIDE = -4,           /* a stride is negative / zero where a dense walk is required */
+    SND_ERR_LAUNCH = -5,           /* hipLaunchKernel reported an error */
+    SND_ERR_WORKSPACE = -6,        /* checkpoint / workspace buffer missing or too small */
+    SND_ERR_ALIGN = -7             /* checkpoint / workspace pointer not 16-byte aligned */
+} snd_status;
+
+/* Problem sizes; replaces the size fields of SSMParamsBase
+ * (kernels/selective_nd_scan/include/cusoflex/selective_scan_oflex.h:4-20). */
+typedef struct snd_shape {
+    int32_t batch, dim, nrows, ncols, dstate, n_groups, delta_dim;
+    int32_t in_dtype;              /* snd_dtype of u, delta, B, C */
+} snd_shape;
+
+/* Sizes (in fp32 elements) of the opaque state that fwd hands to bwd and of bwd's scratch.
+ * Replaces the nChunksX / nChunksY arithmetic and the three torch::empty calls of
+ * selective_scan_oflex.cpp:247-258.  The tensors keep the reference's ranks so that call sites
+ * written for the reference still work:
+ *     x     [batch, dim, dstate, n_chunks_x, x_inner]     (h at the right edge of every column tile)
+ *     x_sd  [batch, dim, dstate, n_chunks_x, x_inner]     (row-only scan s at the same places)
+ *     x_v   [batch, dim, dstate, n_chunks_y, xv_inner]    (h at the last row of every row strip)
+ * Their contents are private to this library; bwd does NOT modify them (a second backward over
+ * the same saved state is valid, unlike the reference, bwd.cuh:489-491,614-619,725-727). */
+typedef struct snd_plan {
+    int32_t n_chunks_x, n_chunks_y;
+    int32_t x_inner, xv_inner;
+    int64_t x_elems, x_sd_elems, x_v_elems;    /* fp32 element counts of the three tensors */
+    int64_t bwd_workspace_bytes;               /* scratch bwd needs (16-byte aligned, uninitialised) */
+} snd_plan;
+
+/* Replaces SSMParamsBase (selective_scan_oflex.h:4-51); 64-bit strides instead of uint32. */
+typedef struct snd_fwd_params {
+    snd_shape shape;
+    int32_t out_dtype;             /* SND_F32 or shape.in_dtype (host.cpp:250, out_float) */
+    int32_t delta_softplus;        /* host.cpp:184 */
+    const void *u, *delta, *B, *C;
+    const float *A;
+    const float *D;                /* optional (null: D = 0, fwd.cuh:121-124) */
+    const float *delta_bias;       /* optional (null: 0, fwd.cuh:125-128) */
+    const float *A_decay;          /* optional, 1 element, must be > 0 (null: 1.0, fwd.cuh:131-134) */
+    void *out;
+    float *x, *x_v, *x_sd;         /* saved state sized by snd_make_plan, 16-byte aligned.  x_v is always
+                                      required (it also carries h from one row strip to the next);
+                                      x and x_sd may both be null = inference only (bwd impossible) */
+    int64_t u_batch_stride, u_d_stride, u_h_stride;
+    int64_t delta_batch_stride, delta_d_stride, delta_h_stride;
+    int64_t A_d_stride, A_dstate_stride;
+    int64_t B_batch_stride, B_group_stride, B_dstate_stride, B_h_stride;
+    int64_t C_batch_stride, C_group_stride, C_dstate_stride, C_h_stride;
+    int64_t out_batch_stride, out_d_stride, out_h_stride;
+} snd_fwd_params;
+
+/* Replaces SSMParamsBwd (selective_scan_oflex.h:53-86). Gradient buffers are dense (contiguous):
+ *     du      [batch, dim, nrows, ncols]          input dtype
+ *     ddelta  [batch, dim, nrows, ncols]          input dtype, PER CHANNEL (dim, not delta_dim):
+ *                                                 the caller sums channel groups when
+ *                                                 dim != delta_dim, as host.cpp:433-434 does
+ *     dA      [dim, dstate] fp32, accumulated with atomics: caller zero-fills (host.cpp:395)
+ *     dB, dC  [batch, n_groups, dstate, nrows, ncols] fp32, accumulated with atomics: caller
+ *                                                 zero-fills, then casts to the input dtype
+ *                                                 (host.cpp:398-399,432)
+ *     dD [dim], ddelta_bias [dim] (per channel, host.cpp:403), dA_decay [1]: fp32, optional,
+ *                                                 accumulated with atomics: caller zero-fills */
+typedef struct snd_bwd_params {
+    snd_fwd_params f;              /* inputs and saved state; f.out / f.out_dtype are ignored */
+    const void *dout;              /* [batch, dim, nrows, ncols], last dim contiguous */
+    int32_t dout_dtype;            /* SND_F32 or shape.in_dtype (host.cpp:303) */
+    int64_t dout_batch_stride, dout_d_stride, dout_h_stride;
+    void *du, *ddelta;
+    float *dA, *dB, *dC;
+    float *dD, *ddelta_bias, *dA_decay;
+    void *workspace;               /* plan.bwd_workspace_bytes bytes, 16-byte aligned */
+    int64_t workspace_bytes;
+} snd_bwd_params;
+
+/* Library / ABI version (major*100 + minor). */
+int snd_version(void);
+
+/* Human-readable text for a status code. */
+const char *snd_status_string(int status);
+
+/* Validate a shape the way selective_scan_oflex.cpp:215-217 does and size the saved state and
+ * backward scratch.  Returns SND_OK or SND_ERR_SHAPE / SND_ERR_DTYPE. */
+int snd_make_plan(const snd_shape *shape, snd_plan *plan);
+
+/* Forward: replaces selective_scan_fwd_cuda<input_t, weight_t, output_t>(params, stream)
+ * (selective_scan_oflex.cpp:31-32,275-281; kernel fwd.cuh:80-357).  Asynchronous on `stream`. */
+int snd_fwd(const snd_fwd_params *params, snd_stream_t stream);
+
+/* Backward: replaces selective_scan_bwd_cuda<input_t, weight_t, output_t>(params, stream)
+ * (selective_scan_oflex.cpp:34-35,424-430; kernel bwd.cuh:91-902).  Asynchronous on `stream`. */
+int snd_bwd(const snd_bwd_params *params, snd_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SND_SCAN_H */

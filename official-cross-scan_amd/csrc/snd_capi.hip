@@ -1,0 +1,105 @@
+// C ABI of the gfx950 selective_nd_scan library: validation, planning and dispatch.
+// Mirrors the checks of the reference host binding
+// (kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:188-245,298-361) as status codes.
+#include "snd_device.h"
+
+namespace snd {
+int launch_fwd(const snd_fwd_params &p, hipStream_t stream);
+int launch_bwd(const snd_bwd_params &p, hipStream_t stream);
+}  // namespace snd
+
+namespace {
+
+int check_shape(const snd_shape &s) {
+    if (s.batch <= 0 || s.dim <= 0 || s.nrows <= 0 || s.ncols <= 0 || s.dstate <= 0 || s.n_groups <= 0 ||
+        s.delta_dim <= 0)
+        return SND_ERR_SHAPE;
+    if (s.dim % s.n_groups != 0) return SND_ERR_SHAPE;      // host.cpp:215
+    if (s.dim % s.delta_dim != 0) return SND_ERR_SHAPE;     // host.cpp:216
+    if (s.dstate > SND_MAX_DSTATE) return SND_ERR_SHAPE;    // host.cpp:217
+    if (s.in_dtype != SND_F32 && s.in_dtype != SND_F16 && s.in_dtype != SND_BF16) return SND_ERR_DTYPE;
+    return SND_OK;
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+int check_fwd(const snd_fwd_params &p, bool need_state) {
+    int st = check_shape(p.shape);
+    if (st != SND_OK) return st;
+    if (!p.u || !p.delta || !p.A || !p.B || !p.C) return SND_ERR_NULL;
+    if (!p.x_v) return SND_ERR_WORKSPACE;
+    if ((p.x == nullptr) != (p.x_sd == nullptr)) return SND_ERR_WORKSPACE;
+    if (need_state && !p.x) return SND_ERR_WORKSPACE;
+    if (!aligned16(p.x_v) || !aligned16(p.x) || !aligned16(p.x_sd)) return SND_ERR_ALIGN;
+    if (p.u_h_stride < p.shape.ncols || p.delta_h_stride < p.shape.ncols || p.B_h_stride < p.shape.ncols ||
+        p.C_h_stride < p.shape.ncols)
+        if (p.shape.nrows > 1) return SND_ERR_STRIDE;
+    return SND_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int snd_version(void) { return 100; }
+
+const char *snd_status_string(int status) {
+    switch (status) {
+        case SND_OK: return "ok";
+        case SND_ERR_NULL: return "a required pointer is null";
+        case SND_ERR_SHAPE: return "bad shape: need dim % n_groups == 0, dim % delta_dim == 0, 1 <= dstate <= 16, all sizes > 0";
+        case SND_ERR_DTYPE: return "unsupported dtype combination (inputs fp32/fp16/bf16; out and dout fp32 or the input dtype)";
+        case SND_ERR_STRIDE: return "bad stride: rows must not overlap and the last dimension must be contiguous";
+        case SND_ERR_LAUNCH: return "kernel launch failed";
+        case SND_ERR_WORKSPACE: return "saved state (x, x_v, x_sd) or workspace missing or too small";
+        case SND_ERR_ALIGN: return "saved state / workspace pointers must be 16-byte aligned";
+        default: return "unknown status";
+    }
+}
+
+int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
+    if (!shape || !plan) return SND_ERR_NULL;
+    int st = check_shape(*shape);
+    if (st != SND_OK) return st;
+    const snd::Geo g = snd::make_geo(shape->nrows, shape->ncols);
+    const int64_t planes = (int64_t)shape->batch * shape->dim * shape->dstate;
+    plan->n_chunks_x = g.nCX;
+    plan->n_chunks_y = g.nCY;
+    plan->x_inner = g.Hp;
+    plan->xv_inner = g.Wp;
+    plan->x_elems = planes * g.nCX * g.Hp;
+    plan->x_sd_elems = plan->x_elems;
+    plan->x_v_elems = planes * g.nCY * g.Wp;
+    // backward scratch: one row of G = a*g per plane (the adjoint carried from the strip below)
+    plan->bwd_workspace_bytes = planes * (int64_t)(g.Wp + 8) * (int64_t)sizeof(float);
+    return SND_OK;
+}
+
+int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
+    if (!params) return SND_ERR_NULL;
+    int st = check_fwd(*params, false);
+    if (st != SND_OK) return st;
+    if (!params->out) return SND_ERR_NULL;
+    if (params->out_dtype != SND_F32 && params->out_dtype != params->shape.in_dtype) return SND_ERR_DTYPE;
+    return snd::launch_fwd(*params, (hipStream_t)stream);
+}
+
+int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
+    if (!params) return SND_ERR_NULL;
+    int st = check_fwd(params->f, true);
+    if (st != SND_OK) return st;
+    if (!params->dout || !params->du || !params->ddelta || !params->dA || !params->dB || !params->dC)
+        return SND_ERR_NULL;
+    if (params->dout_dtype != SND_F32 && params->dout_dtype != params->f.shape.in_dtype) return SND_ERR_DTYPE;
+    if ((params->f.D != nullptr) != (params->dD != nullptr)) return SND_ERR_NULL;
+    if ((params->f.delta_bias != nullptr) != (params->ddelta_bias != nullptr)) return SND_ERR_NULL;
+    if ((params->f.A_decay != nullptr) != (params->dA_decay != nullptr)) return SND_ERR_NULL;
+    snd_plan plan;
+    st = snd_make_plan(&params->f.shape, &plan);
+    if (st != SND_OK) return st;
+    if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
+    if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+    return snd::launch_bwd(*params, (hipStream_t)stream);
+}
+
+}  // extern "C"

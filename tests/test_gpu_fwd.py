@@ -1,0 +1,125 @@
+"""GPU parity of the HIP forward against the float64 oracle, through the C ABI.
+
+Tolerances are the ones the headline metric states: fp32 inputs max-rel <= 1e-4, bf16 inputs
+<= 1e-2 against the fp32 oracle, with rel = max|x - ref| / max|ref| per tensor.
+"""
+import numpy as np
+import pytest
+import torch
+
+import capi
+from oracle import snd_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def relerr(x, ref):
+    x = np.asarray(x, np.float64)
+    ref = np.asarray(ref, np.float64)
+    return float(np.abs(x - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def to_dev(d, dev, dtype=torch.float32):
+    out = {}
+    for k, v in d.items():
+        t = torch.from_numpy(v).to(dev)
+        if k in ("u", "delta", "B", "C"):
+            t = t.to(dtype)
+        out[k] = t
+    return out
+
+
+CASES = [
+    # Bt, Dm, H, W, N, K, Dd
+    (1, 64, 14, 14, 16, 4, None),      # config 0 of the benchmark list
+    (2, 8, 8, 8, 16, 2, None),         # exactly one tile
+    (1, 4, 1, 37, 16, 1, None),        # single row (1D scan)
+    (1, 4, 29, 1, 16, 1, None),        # single column
+    (2, 12, 19, 23, 16, 4, None),      # ragged strips and tiles, partial channel chunk
+    (1, 6, 17, 9, 5, 2, 3),            # dstate not a power of two, shared delta groups
+    (1, 40, 9, 10, 1, 2, None),        # d_state = 1 variant
+    (1, 20, 10, 12, 2, 1, None),
+    (1, 8, 11, 12, 4, 2, None),
+    (1, 8, 9, 20, 8, 1, 2),
+]
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,Dd", CASES)
+def test_fwd_fp32_matches_oracle(gpu_device, Bt, Dm, H, W, N, K, Dd):
+    print("case", Bt, Dm, H, W, N, K, Dd, flush=True)
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=H * 100 + W, Dd=Dd, with_dout=False)
+    ref = O.selective_nd_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True)
+    t = to_dev(d, gpu_device)
+    out, x, x_v, x_sd = capi.fwd(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"], True, True, None)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float32 and out.shape == t["u"].shape
+    e = relerr(out.cpu().numpy(), ref)
+    assert e <= 1e-4, e
+
+
+def test_fwd_no_optional_inputs_and_plain_delta(gpu_device):
+    d = O.make_inputs(2, 8, 10, 13, N=16, K=2, seed=5, with_dout=False)
+    delta = np.abs(d["delta"]) + 0.01
+    ref = O.selective_nd_scan_fwd(d["u"], delta, d["A"], d["B"], d["C"])
+    t = to_dev(dict(d, delta=delta), gpu_device)
+    out, *_ = capi.fwd(t["u"], t["delta"], t["A"], t["B"], t["C"], None, None, False, True, None, save=False)
+    assert relerr(out.cpu().numpy(), ref) <= 1e-4
+
+
+def test_fwd_a_decay(gpu_device):
+    d = O.make_inputs(1, 8, 9, 11, N=16, K=2, seed=6, with_dout=False)
+    dec = np.array([0.9], np.float32)
+    ref = O.selective_nd_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True, dec)
+    t = to_dev(d, gpu_device)
+    out, *_ = capi.fwd(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"], True, True,
+                       torch.from_numpy(dec).to(gpu_device))
+    assert relerr(out.cpu().numpy(), ref) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype,out_float", [(torch.bfloat16, True), (torch.bfloat16, False),
+                                             (torch.float16, True), (torch.float16, False)])
+def test_fwd_half_inputs(gpu_device, dtype, out_float):
+    d = O.make_inputs(2, 16, 14, 14, N=16, K=4, seed=7, with_dout=False)
+    t = to_dev(d, gpu_device, dtype)
+    # oracle on the un-rounded fp32 inputs: the headline tolerance for 16-bit inputs is 1e-2
+    ref = O.selective_nd_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True)
+    # oracle on the rounded inputs: isolates kernel error from input rounding
+    rd = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    ref_r = O.selective_nd_scan_fwd(rd["u"], rd["delta"], d["A"], rd["B"], rd["C"], d["D"], d["delta_bias"], True)
+    out, *_ = capi.fwd(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"], True, out_float, None)
+    assert out.dtype == (torch.float32 if out_float else dtype)
+    o = out.float().cpu().numpy()
+    tol16 = 1e-2 if dtype == torch.bfloat16 else 2e-3
+    assert relerr(o, ref) <= (1e-2 if dtype == torch.bfloat16 else 5e-3)
+    assert relerr(o, ref_r) <= (1e-4 if out_float else tol16)
+
+
+def test_fwd_strided_inputs(gpu_device):
+    """Only the last dimension has to be contiguous (selective_scan_oflex.cpp:203-204,227,229)."""
+    d = O.make_inputs(2, 8, 9, 12, N=16, K=2, seed=8, with_dout=False)
+    ref = O.selective_nd_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True)
+    t = to_dev(d, gpu_device)
+    pad = lambda x: torch.nn.functional.pad(x, (0, 5))[..., : x.shape[-1]]
+    u, dl, B, Cc = pad(t["u"]), pad(t["delta"]), pad(t["B"]), pad(t["C"])
+    assert not u.is_contiguous() and u.stride(-1) == 1
+    out, *_ = capi.fwd(u, dl, t["A"], B, Cc, t["D"], t["delta_bias"], True, True, None)
+    assert relerr(out.cpu().numpy(), ref) <= 1e-4
+
+
+def test_fwd_linearity_at_scale(gpu_device):
+    """Size-independent property at a shape the oracle cannot finish quickly: linear in u."""
+    torch.manual_seed(0)
+    Bt, Dm, H, W, N, K = 4, 96, 56, 56, 16, 4
+    dev = gpu_device
+    u1 = torch.randn(Bt, Dm, H, W, device=dev)
+    u2 = torch.randn(Bt, Dm, H, W, device=dev)
+    delta = 0.1 * torch.randn(Bt, Dm, H, W, device=dev)
+    bias = torch.log(torch.expm1(torch.exp(torch.empty(Dm, device=dev).uniform_(np.log(1e-3), np.log(1e-1)))))
+    A = -torch.arange(1, N + 1, device=dev, dtype=torch.float32).repeat(Dm, 1)
+    B = torch.randn(Bt, K, N, H, W, device=dev)
+    Cc = torch.randn(Bt, K, N, H, W, device=dev)
+    D = torch.ones(Dm, device=dev)
+    f = lambda uu: capi.fwd(uu, delta, A, B, Cc, D, bias, True, True, None)[0]
+    lhs = f(2.0 * u1 - 3.0 * u2)
+    rhs = 2.0 * f(u1) - 3.0 * f(u2)
+    assert relerr(lhs.cpu().numpy(), rhs.cpu().numpy()) <= 1e-4
