@@ -21,7 +21,7 @@ LIB = os.path.join(HERE, "libsnd_scan.so")
 
 HIP_SOURCES = ["snd_fwd.hip", "snd_bwd.hip", "snd_capi.hip"]
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
     # packed-FP32 VALU forms are switched off for every device function
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-I", INC, "-I", CSRC,

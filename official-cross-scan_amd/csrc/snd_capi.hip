@@ -71,7 +71,7 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->x_sd_elems = plan->x_elems;
     plan->x_v_elems = planes * g.nCY * g.Wp;
     // backward scratch: one row of G = a*g per plane (the adjoint carried from the strip below)
-    plan->bwd_workspace_bytes = planes * (int64_t)(g.Wp + 8) * (int64_t)sizeof(float);
+    plan->bwd_workspace_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);
     return SND_OK;
 }
 

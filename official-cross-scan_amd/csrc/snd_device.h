@@ -8,13 +8,17 @@ namespace snd {
 
 constexpr int kWave = 64;          // CDNA wavefront
 constexpr int kRows = 8;           // rows per strip == row-checkpoint spacing
-constexpr int kCkX = 8;            // column-checkpoint spacing == backward tile width
+constexpr int kCkX = 8;            // column-checkpoint spacing == tile width
+constexpr int kTile = kRows * kCkX;
+constexpr int kWPB = 4;            // waves per block
+constexpr int kThreads = kWave * kWPB;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
 
 // Geometry of the opaque saved state (see snd_plan in snd_scan.h).
 struct Geo {
     int nCX, nCY;                  // column tiles of kCkX, row strips of kRows
-    int Hp, Wp;                    // padded inner extents: nCY*kRows, round_up(W, 4) (+4 slack)
+    int Hp, Wp;                    // padded inner extents nCY*kRows, nCX*kCkX
 };
 __host__ __device__ inline Geo make_geo(int H, int W) {
     Geo g;
@@ -29,28 +33,43 @@ __host__ __device__ inline Geo make_geo(int H, int W) {
 struct bf16_t { uint16_t v; };
 typedef _Float16 f16_t;
 
-__device__ __forceinline__ float to_f32(float x) { return x; }
-__device__ __forceinline__ float to_f32(f16_t x) { return (float)x; }
-__device__ __forceinline__ float to_f32(bf16_t x) { return __builtin_bit_cast(float, (uint32_t)x.v << 16); }
-
-template <typename T> __device__ __forceinline__ T from_f32(float x);
-template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
-template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float x) { return (f16_t)x; }
-template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
+__device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
-    bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { r.v = (uint16_t)((u >> 16) | 0x40u); return r; }   // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                                         // RNE
-    r.v = (uint16_t)(u >> 16);
-    return r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                            // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+
+// Element access with the dtype chosen at run time (wave-uniform branch): the tile staging is the
+// only code that touches caller tensors, everything after it is fp32.
+__device__ __forceinline__ float ld_f32(const void *base, int64_t i, int dt) {
+    if (dt == SND_F32) return ((const float *)base)[i];
+    if (dt == SND_BF16) return bf16_to_f32(((const uint16_t *)base)[i]);
+    return (float)((const f16_t *)base)[i];
+}
+__device__ __forceinline__ void st_f32(void *base, int64_t i, int dt, float v) {
+    if (dt == SND_F32) ((float *)base)[i] = v;
+    else if (dt == SND_BF16) ((uint16_t *)base)[i] = f32_to_bf16(v);
+    else ((f16_t *)base)[i] = (f16_t)v;
 }
 
 // ---------------------------------------------------------------- math
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// softplus with the reference's threshold (fwd.cuh:223); log1pf keeps relative accuracy for
-// the small deltas (1e-3) the operator is used with.
-__device__ __forceinline__ float softplus20(float x) { return x <= 20.f ? log1pf(__expf(x)) : x; }
+// softplus with the reference's threshold (fwd.cuh:223): log1p(e) = log(1+e) * e / ((1+e) - 1)
+// keeps full relative accuracy for the tiny e = exp(x) that small time steps produce, using the
+// hardware exp2/log2/rcp (about 1 ulp each).  Also returns the derivative sigmoid(x) (bwd.cuh:792).
+__device__ __forceinline__ float softplus20(float x, float &dsp) {
+    const float e = fast_exp2(x * kLog2e);
+    const float w = 1.f + e;
+    const float d = w - 1.f;
+    const float rw = __builtin_amdgcn_rcpf(w);
+    float sp = (d == 0.f) ? e : __builtin_amdgcn_logf(w) * kLn2 * (e * __builtin_amdgcn_rcpf(d));
+    dsp = e * rw;
+    if (x > 20.f) { sp = x; dsp = 1.f; }
+    return sp;
+}
 
 // ---------------------------------------------------------------- cross-lane sums (DPP)
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
@@ -75,5 +94,18 @@ __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &p
     return pair < nPairs;
 }
 __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8) * 8 * nChunks; }
+
+// ---------------------------------------------------------------- shared tile staging
+// Thread <-> element maps used by both kernels (NP lanes per channel, kThreads threads):
+//   state tiles (B, C, dB, dC): element k of thread t is state (t/64 + kWPB*k), pixel t%64
+//   pixel tiles (delta', u, ...): thread t belongs to channel t/NP (the channel its lane computes)
+//                                 and owns pixels (t%NP) + NP*k, k < 64/NP
+template <int NP> struct Map {
+    static constexpr int CPW = kWave / NP;          // channels per wave
+    static constexpr int CB = CPW * kWPB;           // channels per block
+    static constexpr int NBC = NP * kTile / kThreads;   // B/C elements per thread per tile
+    static constexpr int NPX = kTile / NP;          // pixels per thread per tile
+    static constexpr int NSTR = kTile + 4;          // per-state LDS pitch: lane n hits banks 4n..4n+3
+};
 
 }  // namespace snd

@@ -9,11 +9,15 @@
 //     s[i,j] = a*s[i,j-1] + bu                                          (:306-327)
 //     out    = D*u + sum_n C*(h - s + 0.25*bu)                          (:226-228,301,334)
 // but is organised for CDNA4 rather than translated:
-//   * one lane owns one (channel, state) plane and walks it tile by tile in plain row-major
+//   * one lane owns one (channel, state) plane and walks it in 8x8 tiles in plain row-major
 //     order, so the recurrence needs no block scans, shuffles or barriers in its dependency
 //     chain; a wave holds 64/NP channels x NP states of one (batch, group);
-//   * the block (4 waves) stages each B/C tile once in LDS for all of its channels, and the
-//     per-pixel work (softplus, delta*u) is done once per pixel while staging, not per state;
+//   * the block stages each B/C tile once in LDS for its 16 channels; the per-pixel work
+//     (softplus, delta*u) is done once per pixel while staging, not once per state;
+//   * the next tile's global loads are issued before the current tile is computed;
+//   * tiles are always computed in full on zero-padded staging: cells outside the plane only
+//     feed cells further right/down, so they never reach a stored value and the inner loops
+//     carry no bounds checks;
 //   * the sum over states is a DPP reduction inside aligned lane groups;
 //   * h at strip bottoms (x_v) doubles as the carry to the next strip and as the backward's row
 //     checkpoint; h and s at tile right edges (x, x_sd) are the backward's column checkpoints.
@@ -21,24 +25,23 @@
 
 namespace snd {
 
-template <typename T, typename TO, int NP, int WPB, int TC, bool SAVE>
-__global__ __launch_bounds__(WPB * kWave) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
-    constexpr int R = kRows;
-    constexpr int CPW = kWave / NP;                 // channels per wave
-    constexpr int CB = CPW * WPB;                   // channels per block
-    constexpr int kThreads = WPB * kWave;
-    constexpr int NSTR = R * TC + 4;                // per-state pitch: lane n hits banks 4n..4n+3
-    constexpr int NG = TC / kCkX;                   // column-checkpoint groups per tile
-    static_assert(TC % kCkX == 0, "tile width must be a multiple of the checkpoint spacing");
+template <int NP, bool SAVE>
+__global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
+    constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
+    constexpr int CB = 16;                          // channels per block
+    constexpr int NSTR = kTile + 4;                 // per-state pitch: lane n hits banks 4n..4n+3
+    constexpr int NBC = 4;                          // B/C elements per thread per tile
+    constexpr int NPX = kTile / NP;                 // pixels per thread per tile
+    constexpr int DLP = kTile + kCkX;               // delta' tile with one halo row above
 
     __shared__ __align__(16) float sB[NP * NSTR];
     __shared__ __align__(16) float sC[NP * NSTR];
-    __shared__ __align__(16) float sDl[CB * (R + 1) * TC];   // delta' with one halo row above
-    __shared__ __align__(16) float sDu[CB * R * TC];         // delta' * u
-    __shared__ __align__(16) float sY[CB * R * TC];          // sum_n C*(h - s + bu/4)
+    __shared__ __align__(16) float sDl[CB * DLP];
+    __shared__ __align__(16) float sDu[CB * kTile];  // delta' * u
+    __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s + bu/4)
 
     const snd_shape &sh = p.shape;
-    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
+    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups, dt = sh.in_dtype;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
@@ -46,226 +49,206 @@ __global__ __launch_bounds__(WPB * kWave) void fwd_kernel(const snd_fwd_params p
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
 
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int n = lane % NP, cl = wave * CPW + lane / NP;
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const int n = tid % NP, cl = tid / NP;          // state and block-local channel of this lane
     const int c = cbase + cl;
     const bool cvalid = c < cend;
     const bool lvalid = cvalid && n < N;
     const int cc = cvalid ? c : cend - 1, nn = n < N ? n : N - 1;
+    const int px = tid & 63, pr = px >> 3, pj = px & 7;   // this thread's pixel in B/C staging
 
     const float A2 = lvalid ? p.A[(int64_t)cc * p.A_d_stride + (int64_t)nn * p.A_dstate_stride] * kLog2e : 0.f;
     const float ld = p.A_decay ? __log2f(p.A_decay[0]) : 0.f;
+    const float Dv = p.D ? p.D[cc] : 0.f;
+    const float bias = p.delta_bias ? p.delta_bias[cc / rd] : 0.f;
+    const bool softplus = p.delta_softplus != 0;
 
-    const T *Bp = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
-    const T *Cp = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
-    const T *up = (const T *)p.u + (int64_t)b * p.u_batch_stride;
-    const T *dp = (const T *)p.delta + (int64_t)b * p.delta_batch_stride;
-    TO *op = (TO *)p.out + (int64_t)b * p.out_batch_stride;
+    const int64_t offB = (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
+    const int64_t offC = (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
+    const int64_t offU = (int64_t)b * p.u_batch_stride + (int64_t)cc * p.u_d_stride;
+    const int64_t offD = (int64_t)b * p.delta_batch_stride + (int64_t)(cc / rd) * p.delta_d_stride;
+    const int64_t offO = (int64_t)b * p.out_batch_stride + (int64_t)cc * p.out_d_stride;
 
     const int64_t plane = ((int64_t)b * Dm + cc) * N + nn;
     float *xv = p.x_v + plane * geo.nCY * geo.Wp;
     float *xh = SAVE ? p.x + plane * geo.nCX * geo.Hp : nullptr;
     float *xs = SAVE ? p.x_sd + plane * geo.nCX * geo.Hp : nullptr;
 
-    const int nJ = (W + TC - 1) / TC;
-    const float *myDl = sDl + cl * (R + 1) * TC;
-    const float *myDu = sDu + cl * R * TC;
+    const float *myDl = sDl + cl * DLP;
+    const float *myDu = sDu + cl * kTile;
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
 
-    for (int I = 0; I < geo.nCY; ++I) {
-        const int r0 = I * R;
-        const int rn = min(R, H - r0);
-        float hl[R], sl[R], al[R];                  // h, s, a at the column left of the tile
+    // raw values of one tile, held in registers between their global load and their LDS commit
+    float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo = 0.f;
+    auto prefetch = [&](int I, int J) {
+        const int r0 = I * kRows, j0 = J * kCkX;
+        {
+            const int row = r0 + pr, col = j0 + pj;
+            const bool in = row < H && col < W;
 #pragma unroll
-        for (int r = 0; r < R; ++r) { hl[r] = 0.f; sl[r] = 0.f; al[r] = 0.f; }
-
-        for (int J = 0; J < nJ; ++J) {
-            const int j0 = J * TC;
-            const int tcn = min(TC, W - j0);
-
-            // ---- stage B, C (all states, this tile) : zero outside the plane and for n >= N
-            for (int idx = tid; idx < NP * R * TC; idx += kThreads) {
-                const int sn = idx / (R * TC), rem = idx - sn * (R * TC);
-                const int r = rem / TC, j = rem - r * TC;
-                float vb = 0.f, vc = 0.f;
-                if (sn < N && r < rn && j < tcn) {
-                    const int64_t off = (int64_t)(r0 + r) * p.B_h_stride + (j0 + j);
-                    vb = to_f32(Bp[(int64_t)sn * p.B_dstate_stride + off]);
-                    const int64_t offc = (int64_t)(r0 + r) * p.C_h_stride + (j0 + j);
-                    vc = to_f32(Cp[(int64_t)sn * p.C_dstate_stride + offc]);
-                }
-                sB[sn * NSTR + rem] = vb;
-                sC[sn * NSTR + rem] = vc;
+            for (int k = 0; k < NBC; ++k) {
+                const int sn = wave + WPB * k;
+                const bool ok = in && sn < N;
+                qb[k] = ok ? ld_f32(p.B, offB + (int64_t)sn * p.B_dstate_stride + (int64_t)row * p.B_h_stride + col, dt) : 0.f;
+                qc[k] = ok ? ld_f32(p.C, offC + (int64_t)sn * p.C_dstate_stride + (int64_t)row * p.C_h_stride + col, dt) : 0.f;
             }
-            // ---- stage delta' (rows r0-1 .. r0+R-1) and delta'*u : once per pixel, not per state
-            for (int idx = tid; idx < CB * (R + 1) * TC; idx += kThreads) {
-                const int scl = idx / ((R + 1) * TC), rem = idx - scl * ((R + 1) * TC);
-                const int rr = rem / TC, j = rem - rr * TC;
-                const int sc = cbase + scl, row = r0 - 1 + rr, col = j0 + j;
-                float dl = 0.f, du = 0.f;
-                if (sc < cend && row >= 0 && row < H && col < W) {
-                    const int dgi = sc / rd;
-                    float raw = to_f32(dp[(int64_t)dgi * p.delta_d_stride + (int64_t)row * p.delta_h_stride + col]);
-                    if (p.delta_bias) raw += p.delta_bias[dgi];
-                    dl = p.delta_softplus ? softplus20(raw) : raw;
-                    if (rr > 0) du = dl * to_f32(up[(int64_t)sc * p.u_d_stride + (int64_t)row * p.u_h_stride + col]);
-                }
-                sDl[idx] = dl;
-                if (rr > 0) sDu[scl * R * TC + (rr - 1) * TC + j] = du;
-            }
+        }
+#pragma unroll
+        for (int k = 0; k < NPX; ++k) {
+            const int pp = n + NP * k;
+            const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
+            const bool ok = cvalid && row < H && col < W;
+            qdl[k] = ok ? ld_f32(p.delta, offD + (int64_t)row * p.delta_h_stride + col, dt) : 0.f;
+            qu[k] = ok ? ld_f32(p.u, offU + (int64_t)row * p.u_h_stride + col, dt) : 0.f;
+        }
+        if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
+            const int row = r0 - 1, col = j0 + n;
+            qhalo = (cvalid && row >= 0 && col < W) ? ld_f32(p.delta, offD + (int64_t)row * p.delta_h_stride + col, dt) : 0.f;
+        }
+    };
+    float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
+    auto commit = [&]() {
+#pragma unroll
+        for (int k = 0; k < NBC; ++k) {
+            const int sn = wave + WPB * k;
+            sB[sn * NSTR + px] = qb[k];
+            sC[sn * NSTR + px] = qc[k];
+        }
+        float dsp;
+#pragma unroll
+        for (int k = 0; k < NPX; ++k) {
+            const int pp = n + NP * k;
+            const float raw = qdl[k] + bias;
+            const float dl = softplus ? softplus20(raw, dsp) : raw;
+            sDl[cl * DLP + kCkX + pp] = dl;
+            sDu[cl * kTile + pp] = dl * qu[k];
+            dukeep[k] = Dv * qu[k];
+        }
+        if (n < kCkX) {
+            const float raw = qhalo + bias;
+            sDl[cl * DLP + n] = softplus ? softplus20(raw, dsp) : raw;
+        }
+    };
+
+    prefetch(0, 0);
+    for (int I = 0; I < geo.nCY; ++I) {
+        const int r0 = I * kRows;
+        float hl[kRows], sl[kRows], al[kRows];      // h, s, a at the column left of the tile
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) { hl[r] = 0.f; sl[r] = 0.f; al[r] = 0.f; }
+
+        for (int J = 0; J < geo.nCX; ++J) {
+            const int j0 = J * kCkX;
+            commit();
             __syncthreads();
+            {   // issue the next tile's loads now; they complete while this tile is computed
+                int In = I, Jn = J + 1;
+                if (Jn == geo.nCX) { Jn = 0; In = I + 1; }
+                if (In < geo.nCY) prefetch(In, Jn);
+            }
 
             // ---- per-lane tile walk
-            float hup[TC], aup[TC];                 // row above the current one
+            float hup[kCkX], aup[kCkX];             // row above the current one
             float corner = 0.f;                     // h[r0-1][j0-1]
             if (I > 0) {
                 const float4 *src = (const float4 *)(xv + (int64_t)(I - 1) * geo.Wp + j0);
+                const float4 v0 = src[0], v1 = src[1];
+                hup[0] = v0.x; hup[1] = v0.y; hup[2] = v0.z; hup[3] = v0.w;
+                hup[4] = v1.x; hup[5] = v1.y; hup[6] = v1.z; hup[7] = v1.w;
 #pragma unroll
-                for (int k = 0; k < TC / 4; ++k) {
-                    const float4 v = src[k];
-                    hup[4 * k + 0] = v.x; hup[4 * k + 1] = v.y; hup[4 * k + 2] = v.z; hup[4 * k + 3] = v.w;
-                }
-#pragma unroll
-                for (int j = 0; j < TC; ++j) {
-                    hup[j] = lvalid ? hup[j] : 0.f;
-                    aup[j] = fast_exp2(fmaf(myDl[j], A2, ld));
-                }
-                if (J > 0) corner = lvalid ? xv[(int64_t)(I - 1) * geo.Wp + j0 - 1] : 0.f;
+                for (int j = 0; j < kCkX; ++j) aup[j] = fast_exp2(fmaf(myDl[j], A2, ld));
+                if (J > 0) corner = xv[(int64_t)(I - 1) * geo.Wp + j0 - 1];
             } else {
 #pragma unroll
-                for (int j = 0; j < TC; ++j) { hup[j] = 0.f; aup[j] = 0.f; }
+                for (int j = 0; j < kCkX; ++j) { hup[j] = 0.f; aup[j] = 0.f; }
             }
 
-            float xe[NG][R], xse[NG][R];            // h, s at checkpoint columns
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (r < rn) {
-                    float left = hl[r], sleft = sl[r], aleft = al[r];
-                    float diag = corner;
-                    corner = hl[r];                 // h[r0+r][j0-1] is the next row's corner
-                    float y[TC];
+            for (int r = 0; r < kRows; ++r) {
+                float left = hl[r], sleft = sl[r], aleft = al[r];
+                float diag = corner;
+                corner = hl[r];                     // h[r0+r][j0-1] is the next row's corner
+                float y[kCkX];
 #pragma unroll
-                    for (int j4 = 0; j4 < TC; j4 += 4) {
-                        const float4 vdl = *(const float4 *)(myDl + (r + 1) * TC + j4);
-                        const float4 vdu = *(const float4 *)(myDu + r * TC + j4);
-                        const float4 vb = *(const float4 *)(myB + r * TC + j4);
-                        const float4 vc = *(const float4 *)(myC + r * TC + j4);
-                        const float adl[4] = {vdl.x, vdl.y, vdl.z, vdl.w};
-                        const float adu[4] = {vdu.x, vdu.y, vdu.z, vdu.w};
-                        const float ab[4] = {vb.x, vb.y, vb.z, vb.w};
-                        const float ac[4] = {vc.x, vc.y, vc.z, vc.w};
+                for (int j4 = 0; j4 < kCkX; j4 += 4) {
+                    const float4 vdl = *(const float4 *)(myDl + (r + 1) * kCkX + j4);
+                    const float4 vdu = *(const float4 *)(myDu + r * kCkX + j4);
+                    const float4 vb = *(const float4 *)(myB + r * kCkX + j4);
+                    const float4 vc = *(const float4 *)(myC + r * kCkX + j4);
+                    const float adl[4] = {vdl.x, vdl.y, vdl.z, vdl.w};
+                    const float adu[4] = {vdu.x, vdu.y, vdu.z, vdu.w};
+                    const float ab[4] = {vb.x, vb.y, vb.z, vb.w};
+                    const float ac[4] = {vc.x, vc.y, vc.z, vc.w};
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const int j = j4 + q;
-                            if (j < tcn) {
-                                const float a = fast_exp2(fmaf(adl[q], A2, ld));
-                                const float bu = ab[q] * adu[q];
-                                const float X = fmaf(-0.5f * (aup[j] + aleft), diag, hup[j]);
-                                const float h = fmaf(a, left + X, bu);
-                                const float s = fmaf(a, sleft, bu);
-                                y[j] = ac[q] * fmaf(0.25f, bu, h - s);
-                                diag = hup[j];
-                                hup[j] = h; aup[j] = a;
-                                left = h; aleft = a; sleft = s;
-                                if ((j & (kCkX - 1)) == kCkX - 1) { xe[j / kCkX][r] = h; xse[j / kCkX][r] = s; }
-                            } else {
-                                y[j] = 0.f;
-                            }
-                        }
+                    for (int q = 0; q < 4; ++q) {
+                        const int j = j4 + q;
+                        const float a = fast_exp2(fmaf(adl[q], A2, ld));
+                        const float bu = ab[q] * adu[q];
+                        const float X = fmaf(-0.5f * (aup[j] + aleft), diag, hup[j]);
+                        const float h = fmaf(a, left + X, bu);
+                        const float s = fmaf(a, sleft, bu);
+                        y[j] = ac[q] * fmaf(0.25f, bu, h - s);
+                        diag = hup[j];
+                        hup[j] = h; aup[j] = a;
+                        left = h; aleft = a; sleft = s;
                     }
-                    hl[r] = left; sl[r] = sleft; al[r] = aleft;
+                }
+                hl[r] = left; sl[r] = sleft; al[r] = aleft;
 #pragma unroll
-                    for (int j = 0; j < TC; ++j) y[j] = group_sum<NP>(y[j]);
-                    if (n == 0) {
-                        float4 *dst = (float4 *)(sY + cl * R * TC + r * TC);
-#pragma unroll
-                        for (int k = 0; k < TC / 4; ++k) dst[k] = make_float4(y[4 * k], y[4 * k + 1], y[4 * k + 2], y[4 * k + 3]);
-                    }
-                } else {
-#pragma unroll
-                    for (int gi = 0; gi < NG; ++gi) { xe[gi][r] = 0.f; xse[gi][r] = 0.f; }
+                for (int j = 0; j < kCkX; ++j) y[j] = group_sum<NP>(y[j]);
+                if (n == 0) {
+                    float4 *dst = (float4 *)(sY + cl * kTile + r * kCkX);
+                    dst[0] = make_float4(y[0], y[1], y[2], y[3]);
+                    dst[1] = make_float4(y[4], y[5], y[6], y[7]);
                 }
             }
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float4 *dst = (float4 *)(xv + (int64_t)I * geo.Wp + j0);
-#pragma unroll
-                for (int k = 0; k < TC / 4; ++k) dst[k] = make_float4(hup[4 * k], hup[4 * k + 1], hup[4 * k + 2], hup[4 * k + 3]);
-                if (SAVE) {
-#pragma unroll
-                    for (int gi = 0; gi < NG; ++gi) {
-                        if (gi * kCkX + kCkX <= tcn) {
-                            const int Jb = (j0 + gi * kCkX) / kCkX;
-                            float4 *dh = (float4 *)(xh + (int64_t)Jb * geo.Hp + r0);
-                            float4 *ds = (float4 *)(xs + (int64_t)Jb * geo.Hp + r0);
-#pragma unroll
-                            for (int k = 0; k < R / 4; ++k) {
-                                dh[k] = make_float4(xe[gi][4 * k], xe[gi][4 * k + 1], xe[gi][4 * k + 2], xe[gi][4 * k + 3]);
-                                ds[k] = make_float4(xse[gi][4 * k], xse[gi][4 * k + 1], xse[gi][4 * k + 2], xse[gi][4 * k + 3]);
-                            }
-                        }
-                    }
+                dst[0] = make_float4(hup[0], hup[1], hup[2], hup[3]);
+                dst[1] = make_float4(hup[4], hup[5], hup[6], hup[7]);
+                if (SAVE && J + 1 < geo.nCX) {      // column checkpoints: only if a tile follows
+                    float4 *dh = (float4 *)(xh + (int64_t)J * geo.Hp + r0);
+                    float4 *ds = (float4 *)(xs + (int64_t)J * geo.Hp + r0);
+                    dh[0] = make_float4(hl[0], hl[1], hl[2], hl[3]);
+                    dh[1] = make_float4(hl[4], hl[5], hl[6], hl[7]);
+                    ds[0] = make_float4(sl[0], sl[1], sl[2], sl[3]);
+                    ds[1] = make_float4(sl[4], sl[5], sl[6], sl[7]);
                 }
             }
             __syncthreads();
 
-            // ---- out = D*u + y, written by the whole block, coalesced along the row
-            for (int idx = tid; idx < CB * R * TC; idx += kThreads) {
-                const int scl = idx / (R * TC), rem = idx - scl * (R * TC);
-                const int r = rem / TC, j = rem - r * TC;
-                const int sc = cbase + scl;
-                if (sc < cend && r < rn && j < tcn) {
-                    const int row = r0 + r, col = j0 + j;
-                    float v = sY[idx];
-                    if (p.D) v = fmaf(p.D[sc], to_f32(up[(int64_t)sc * p.u_d_stride + (int64_t)row * p.u_h_stride + col]), v);
-                    op[(int64_t)sc * p.out_d_stride + (int64_t)row * p.out_h_stride + col] = from_f32<TO>(v);
-                }
+            // ---- out = D*u + y, written by the thread that staged the pixel
+#pragma unroll
+            for (int k = 0; k < NPX; ++k) {
+                const int pp = n + NP * k;
+                const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
+                if (cvalid && row < H && col < W)
+                    st_f32(p.out, offO + (int64_t)row * p.out_h_stride + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
-            // the next tile's staging does not touch sY, and its first barrier orders the
-            // sY reads above against the next tile's sY writes
+            // the next commit() does not touch sY; its barrier orders these sY reads against the
+            // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
         }
     }
 }
 
-template <typename T, typename TO, int NP>
+template <int NP>
 static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
-    constexpr int TC = 8;
-    // waves per block: keep channels per block (and with it the per-channel LDS tiles) bounded
-    constexpr int WPB = NP >= 8 ? 4 : (NP == 4 ? 2 : 1);
-    constexpr int CB = (kWave / NP) * WPB;
-    constexpr int kThreads = WPB * kWave;
     const snd_shape &sh = p.shape;
     const Geo geo = make_geo(sh.nrows, sh.ncols);
     const int rg = sh.dim / sh.n_groups;
-    const int nChunks = (rg + CB - 1) / CB;
+    const int nChunks = (rg + 15) / 16;
     const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
-    const bool save = p.x != nullptr;
-    if (save)
-        hipLaunchKernelGGL((fwd_kernel<T, TO, NP, WPB, TC, true>), dim3(grid), dim3(kThreads), 0, stream, p, geo);
+    if (p.x != nullptr)
+        hipLaunchKernelGGL((fwd_kernel<NP, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     else
-        hipLaunchKernelGGL((fwd_kernel<T, TO, NP, WPB, TC, false>), dim3(grid), dim3(kThreads), 0, stream, p, geo);
+        hipLaunchKernelGGL((fwd_kernel<NP, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
-template <typename T, typename TO>
-static int launch_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
-    const int N = p.shape.dstate;
-    if (N > 8) return launch_fwd_np<T, TO, 16>(p, stream);
-    if (N > 4) return launch_fwd_np<T, TO, 8>(p, stream);
-    if (N > 2) return launch_fwd_np<T, TO, 4>(p, stream);
-    if (N > 1) return launch_fwd_np<T, TO, 2>(p, stream);
-    return launch_fwd_np<T, TO, 1>(p, stream);
-}
-
 int launch_fwd(const snd_fwd_params &p, hipStream_t stream) {
-    const int it = p.shape.in_dtype, ot = p.out_dtype;
-    if (it == SND_F32 && ot == SND_F32) return launch_fwd_t<float, float>(p, stream);
-    if (it == SND_BF16 && ot == SND_F32) return launch_fwd_t<bf16_t, float>(p, stream);
-    if (it == SND_BF16 && ot == SND_BF16) return launch_fwd_t<bf16_t, bf16_t>(p, stream);
-    if (it == SND_F16 && ot == SND_F32) return launch_fwd_t<f16_t, float>(p, stream);
-    if (it == SND_F16 && ot == SND_F16) return launch_fwd_t<f16_t, f16_t>(p, stream);
-    return SND_ERR_DTYPE;
+    return p.shape.dstate > 8 ? launch_fwd_np<16>(p, stream) : launch_fwd_np<8>(p, stream);
 }
 
 }  // namespace snd
