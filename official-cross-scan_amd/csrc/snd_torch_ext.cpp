@@ -1,0 +1,215 @@
+// Thin PyTorch-ROCm extension over the C ABI in include/snd_scan.h.
+//
+// Exports the reference's operator pair with the reference's argument and return lists
+// (kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:179-187,282 and :286-297,432-438,
+// pybind :442-445):
+//     fwd(u, delta, A, B, C, D?, delta_bias?, delta_softplus, out_float, A_decay?) -> [out, x, x_v, x_sd]
+//     bwd(u, delta, A, B, C, D?, delta_bias?, dout, x?, x_v?, delta_softplus, A_decay?, x_sd?)
+//         -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
+// It does what a host binding has to do and nothing else: the reference's TORCH_CHECKs
+// (:188-245, :298-391), allocation of outputs / saved state / scratch, device guard, current-stream
+// lookup, and mapping of a non-zero library status to a c10::Error (Python RuntimeError).
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/extension.h>
+
+#include <vector>
+
+#include "snd_scan.h"
+
+namespace {
+
+#define CHECK_SHAPE(x, ...) \
+    TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
+
+int dtype_code(at::ScalarType t) {
+    switch (t) {
+        case at::ScalarType::Float: return SND_F32;
+        case at::ScalarType::Half: return SND_F16;
+        case at::ScalarType::BFloat16: return SND_BF16;
+        default: TORCH_CHECK(false, "selective_nd_scan: unsupported dtype ", toString(t)); return -1;
+    }
+}
+
+void check_status(int st, const char *what) {
+    TORCH_CHECK(st == SND_OK, "selective_nd_scan ", what, " failed: ", snd_status_string(st), " (status ", st, ")");
+}
+
+struct Checked {
+    int batch, dim, nrows, ncols, dstate, n_groups, delta_dim;
+    snd_shape shape;
+    snd_plan plan;
+};
+
+// The checks of selective_scan_oflex.cpp:188-245 (shared by fwd and bwd).
+Checked check_inputs(const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A, const at::Tensor &B,
+                     const at::Tensor &C, const c10::optional<at::Tensor> &D_,
+                     const c10::optional<at::Tensor> &delta_bias_, const c10::optional<at::Tensor> &A_decay_) {
+    auto input_type = u.scalar_type();
+    TORCH_CHECK(input_type == at::ScalarType::Float || input_type == at::ScalarType::Half ||
+                input_type == at::ScalarType::BFloat16, "u must be float32, float16 or bfloat16");
+    TORCH_CHECK(A.scalar_type() == at::ScalarType::Float, "A must be float32");
+    TORCH_CHECK(delta.scalar_type() == input_type && B.scalar_type() == input_type && C.scalar_type() == input_type,
+                "u, delta, B, C must share one dtype");
+    TORCH_CHECK(u.is_cuda() && delta.is_cuda() && A.is_cuda() && B.is_cuda() && C.is_cuda(),
+                "all tensors must be on the GPU");
+    TORCH_CHECK(u.dim() == 4 && delta.dim() == 4 && A.dim() == 2 && B.dim() == 5 && C.dim() == 5,
+                "expected u, delta 4-D; A 2-D; B, C 5-D");
+    TORCH_CHECK(u.stride(-1) == 1 || u.size(-1) == 1, "u must be contiguous in its last dimension");
+    TORCH_CHECK(delta.stride(-1) == 1 || delta.size(-1) == 1, "delta must be contiguous in its last dimension");
+
+    Checked c;
+    c.batch = u.size(0); c.dim = u.size(1); c.nrows = u.size(2); c.ncols = u.size(3);
+    c.dstate = A.size(1); c.n_groups = B.size(1); c.delta_dim = delta.size(1);
+    TORCH_CHECK(c.dim % c.n_groups == 0, "dims should be dividable by n_groups");
+    TORCH_CHECK(c.dim % c.delta_dim == 0, "dims should be dividable by delta_dim");
+    TORCH_CHECK(c.dstate <= SND_MAX_DSTATE, "selective_scan only supports state dimension <= 16");
+    const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate,
+              n_groups = c.n_groups, delta_dim = c.delta_dim;
+    CHECK_SHAPE(u, batch_size, dim, nrows, ncols);
+    CHECK_SHAPE(delta, batch_size, delta_dim, nrows, ncols);
+    CHECK_SHAPE(A, dim, dstate);
+    CHECK_SHAPE(B, batch_size, n_groups, dstate, nrows, ncols);
+    TORCH_CHECK(B.stride(-1) == 1 || B.size(-1) == 1, "B must be contiguous in its last dimension");
+    CHECK_SHAPE(C, batch_size, n_groups, dstate, nrows, ncols);
+    TORCH_CHECK(C.stride(-1) == 1 || C.size(-1) == 1, "C must be contiguous in its last dimension");
+    if (A_decay_.has_value()) {
+        const auto &A_decay = A_decay_.value();
+        TORCH_CHECK(A_decay.scalar_type() == at::ScalarType::Float && A_decay.is_cuda());
+        CHECK_SHAPE(A_decay, 1);
+    }
+    if (D_.has_value()) {
+        const auto &D = D_.value();
+        TORCH_CHECK(D.scalar_type() == at::ScalarType::Float && D.is_cuda());
+        TORCH_CHECK(D.stride(-1) == 1 || D.size(-1) == 1);
+        CHECK_SHAPE(D, dim);
+    }
+    if (delta_bias_.has_value()) {
+        const auto &delta_bias = delta_bias_.value();
+        TORCH_CHECK(delta_bias.scalar_type() == at::ScalarType::Float && delta_bias.is_cuda());
+        TORCH_CHECK(delta_bias.stride(-1) == 1 || delta_bias.size(-1) == 1);
+        CHECK_SHAPE(delta_bias, delta_dim);
+    }
+    c.shape = snd_shape{c.batch, c.dim, c.nrows, c.ncols, c.dstate, c.n_groups, c.delta_dim, dtype_code(input_type)};
+    check_status(snd_make_plan(&c.shape, &c.plan), "plan");
+    return c;
+}
+
+void fill_fwd(snd_fwd_params &p, const Checked &c, const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
+              const at::Tensor &B, const at::Tensor &C, const c10::optional<at::Tensor> &D_,
+              const c10::optional<at::Tensor> &delta_bias_, const c10::optional<at::Tensor> &A_decay_,
+              bool delta_softplus) {
+    memset(&p, 0, sizeof(p));
+    p.shape = c.shape;
+    p.delta_softplus = delta_softplus ? 1 : 0;
+    p.u = u.data_ptr(); p.delta = delta.data_ptr(); p.B = B.data_ptr(); p.C = C.data_ptr();
+    p.A = A.data_ptr<float>();
+    p.D = D_.has_value() ? D_.value().data_ptr<float>() : nullptr;
+    p.delta_bias = delta_bias_.has_value() ? delta_bias_.value().data_ptr<float>() : nullptr;
+    p.A_decay = A_decay_.has_value() ? A_decay_.value().data_ptr<float>() : nullptr;
+    p.u_batch_stride = u.stride(0); p.u_d_stride = u.stride(1); p.u_h_stride = u.stride(2);
+    p.delta_batch_stride = delta.stride(0); p.delta_d_stride = delta.stride(1); p.delta_h_stride = delta.stride(2);
+    p.A_d_stride = A.stride(0); p.A_dstate_stride = A.stride(1);
+    p.B_batch_stride = B.stride(0); p.B_group_stride = B.stride(1); p.B_dstate_stride = B.stride(2); p.B_h_stride = B.stride(3);
+    p.C_batch_stride = C.stride(0); p.C_group_stride = C.stride(1); p.C_dstate_stride = C.stride(2); p.C_h_stride = C.stride(3);
+}
+
+std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
+                                           const at::Tensor &B, const at::Tensor &C,
+                                           const c10::optional<at::Tensor> &D_,
+                                           const c10::optional<at::Tensor> &delta_bias_, bool delta_softplus,
+                                           bool out_float, const c10::optional<at::Tensor> &A_decay_) {
+    const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
+    at::hip::HIPGuardMasqueradingAsCUDA device_guard{u.device()};
+    const auto f32 = u.options().dtype(at::ScalarType::Float);
+    at::Tensor out = torch::empty({c.batch, c.dim, c.nrows, c.ncols},
+                                  u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
+    at::Tensor x = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
+    at::Tensor x_v = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_y, c.plan.xv_inner}, f32);
+    at::Tensor x_sd = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
+
+    snd_fwd_params p;
+    fill_fwd(p, c, u, delta, A, B, C, D_, delta_bias_, A_decay_, delta_softplus);
+    p.out = out.data_ptr();
+    p.out_dtype = dtype_code(out.scalar_type());
+    p.out_batch_stride = out.stride(0); p.out_d_stride = out.stride(1); p.out_h_stride = out.stride(2);
+    p.x = x.data_ptr<float>(); p.x_v = x_v.data_ptr<float>(); p.x_sd = x_sd.data_ptr<float>();
+    auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");
+    return {out, x, x_v, x_sd};
+}
+
+std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
+                                           const at::Tensor &B, const at::Tensor &C,
+                                           const c10::optional<at::Tensor> &D_,
+                                           const c10::optional<at::Tensor> &delta_bias_, const at::Tensor &dout,
+                                           const c10::optional<at::Tensor> &x_, const c10::optional<at::Tensor> &x_v_,
+                                           bool delta_softplus, const c10::optional<at::Tensor> &A_decay_,
+                                           const c10::optional<at::Tensor> &x_sd_) {
+    const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
+    const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate;
+    TORCH_CHECK(dout.scalar_type() == u.scalar_type() || dout.scalar_type() == at::ScalarType::Float,
+                "dout must be float32 or the input dtype");
+    TORCH_CHECK(dout.is_cuda());
+    TORCH_CHECK(dout.stride(-1) == 1 || dout.size(-1) == 1, "dout must be contiguous in its last dimension");
+    CHECK_SHAPE(dout, batch_size, dim, nrows, ncols);
+    // the saved state is required: gradients computed without it would belong to another function
+    TORCH_CHECK(x_.has_value() && x_v_.has_value() && x_sd_.has_value(),
+                "bwd needs the x, x_v and x_sd tensors returned by fwd");
+    const auto &x = x_.value(), &x_v = x_v_.value(), &x_sd = x_sd_.value();
+    const int nChunksX = c.plan.n_chunks_x, nChunksY = c.plan.n_chunks_y, x_inner = c.plan.x_inner,
+              xv_inner = c.plan.xv_inner;
+    for (const at::Tensor *t : {&x, &x_v, &x_sd}) {
+        TORCH_CHECK(t->scalar_type() == at::ScalarType::Float && t->is_cuda() && t->is_contiguous(),
+                    "saved state must be contiguous float32 GPU tensors");
+    }
+    CHECK_SHAPE(x, batch_size, dim, dstate, nChunksX, x_inner);
+    CHECK_SHAPE(x_sd, batch_size, dim, dstate, nChunksX, x_inner);
+    CHECK_SHAPE(x_v, batch_size, dim, dstate, nChunksY, xv_inner);
+
+    at::hip::HIPGuardMasqueradingAsCUDA device_guard{u.device()};
+    const auto f32 = u.options().dtype(at::ScalarType::Float);
+    at::Tensor du = torch::empty({batch_size, dim, nrows, ncols}, u.options());
+    at::Tensor ddelta = torch::empty({batch_size, dim, nrows, ncols}, u.options());
+    at::Tensor dA = torch::zeros({dim, dstate}, f32);
+    at::Tensor dB = torch::zeros(B.sizes(), f32);
+    at::Tensor dC = torch::zeros(C.sizes(), f32);
+    at::Tensor dD, ddelta_bias, dA_decay;
+    if (D_.has_value()) dD = torch::zeros({dim}, f32);
+    if (delta_bias_.has_value()) ddelta_bias = torch::zeros({dim}, f32);
+    if (A_decay_.has_value()) dA_decay = torch::zeros({1}, f32);
+    at::Tensor ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
+
+    snd_bwd_params p;
+    memset(&p, 0, sizeof(p));
+    fill_fwd(p.f, c, u, delta, A, B, C, D_, delta_bias_, A_decay_, delta_softplus);
+    p.f.x = x.data_ptr<float>(); p.f.x_v = x_v.data_ptr<float>(); p.f.x_sd = x_sd.data_ptr<float>();
+    p.dout = dout.data_ptr();
+    p.dout_dtype = dtype_code(dout.scalar_type());
+    p.dout_batch_stride = dout.stride(0); p.dout_d_stride = dout.stride(1); p.dout_h_stride = dout.stride(2);
+    p.du = du.data_ptr(); p.ddelta = ddelta.data_ptr();
+    p.dA = dA.data_ptr<float>(); p.dB = dB.data_ptr<float>(); p.dC = dC.data_ptr<float>();
+    p.dD = dD.defined() ? dD.data_ptr<float>() : nullptr;
+    p.ddelta_bias = ddelta_bias.defined() ? ddelta_bias.data_ptr<float>() : nullptr;
+    p.dA_decay = dA_decay.defined() ? dA_decay.data_ptr<float>() : nullptr;
+    p.workspace = ws.data_ptr();
+    p.workspace_bytes = c.plan.bwd_workspace_bytes;
+    auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
+
+    // host.cpp:432-438: cast dB/dC to the input dtype, fold channel groups that share a delta
+    std::vector<at::Tensor> result = {du, ddelta, dA, dB.to(B.dtype()), dC.to(C.dtype()), dD, ddelta_bias, dA_decay};
+    if (dim != c.delta_dim) {
+        const int rep = dim / c.delta_dim;
+        result[1] = ddelta.view({batch_size, c.delta_dim, rep, nrows, ncols}).sum(2);
+        if (delta_bias_.has_value()) result[6] = ddelta_bias.view({c.delta_dim, rep}).sum(1);
+    }
+    return result;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)");
+    m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)");
+}

@@ -1,0 +1,69 @@
+"""Python face of the 2D-CrossScan selective scan on MI355X.
+
+The reference ships only the pybind pair `fwd` / `bwd`
+(kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:442-445); the Python function and
+autograd.Function that backbones call are authored here on top of the same pair, with the argument
+order of those bindings (selective_scan_oflex.cpp:179-187).
+
+    out = selective_nd_scan(u, delta, A, B, C, D=None, delta_bias=None,
+                            delta_softplus=False, out_float=True, A_decay=None)
+
+    u      [B, D, H, W]        fp32 / fp16 / bf16
+    delta  [B, Dd, H, W]       same dtype, D % Dd == 0
+    A      [D, N]              fp32, N <= 16
+    B, C   [B, G, N, H, W]     same dtype as u, D % G == 0
+    D      [D] fp32, delta_bias [Dd] fp32, A_decay [1] fp32 (all optional)
+    out    [B, D, H, W]        fp32 if out_float else u.dtype
+
+Every group is scanned from the top-left corner, as the reference kernel does
+(selective_scan_fwd_kernel_oflex.cuh:140); the four corner directions are made by the caller
+(see cross_scan.py).
+"""
+import torch
+
+from ._ext import ext
+
+
+def fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None):
+    """Reference binding `fwd` -> [out, x, x_v, x_sd] (selective_scan_oflex.cpp:179-187,282)."""
+    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)
+
+
+def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd):
+    """Reference binding `bwd` -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
+    (selective_scan_oflex.cpp:286-297,432-438)."""
+    return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd)
+
+
+def _last_dim_contiguous(t):
+    return t if (t is None or t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
+
+
+class SelectiveNdScanFn(torch.autograd.Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
+                A_decay=None):
+        u, delta, B, C = map(_last_dim_contiguous, (u, delta, B, C))
+        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)
+        ctx.delta_softplus = delta_softplus
+        ctx.has = (D is not None, delta_bias is not None, A_decay is not None)
+        ctx.save_for_backward(u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd)
+        return out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dout):
+        u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd = ctx.saved_tensors
+        dout = _last_dim_contiguous(dout)
+        du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay = bwd(
+            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd)
+        has_D, has_bias, has_decay = ctx.has
+        return (du, ddelta, dA, dB, dC, dD if has_D else None, ddelta_bias if has_bias else None,
+                None, None, dA_decay if has_decay else None)
+
+
+def selective_nd_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
+                      A_decay=None):
+    """Differentiable 2D-CrossScan selective scan (forward and backward run on the HIP kernels)."""
+    return SelectiveNdScanFn.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)

@@ -1,0 +1,83 @@
+"""CPU-only checks of the boundary: the C-ABI library loads, exports every symbol the header
+declares, plans and validates like the reference's host code, and fails loudly without a GPU path."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import capi
+
+
+def test_library_exports_every_declared_symbol():
+    names = capi.declared_symbols()
+    assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd"}
+    lib = capi.lib()
+    for n in names:
+        assert getattr(lib, n) is not None, n
+    assert lib.snd_version() >= 100
+
+
+def test_struct_layouts_match_header_sizes():
+    # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
+    assert C.sizeof(capi.Shape) == 32
+    assert C.sizeof(capi.Plan) == 48
+    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8
+    assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8
+
+
+@pytest.mark.parametrize("H,W,ncx,ncy", [(56, 56, 7, 7), (14, 14, 2, 2), (200, 336, 42, 25), (1, 37, 5, 1), (512, 512, 64, 64)])
+def test_plan_geometry(H, W, ncx, ncy):
+    st, plan = capi.make_plan(capi.Shape(2, 8, H, W, 16, 4, 8, capi.SND_F32))
+    assert st == 0
+    assert (plan.n_chunks_x, plan.n_chunks_y) == (ncx, ncy)
+    assert plan.x_inner == ncy * 8 and plan.xv_inner == ncx * 8
+    planes = 2 * 8 * 16
+    assert plan.x_elems == planes * ncx * plan.x_inner == plan.x_sd_elems
+    assert plan.x_v_elems == planes * ncy * plan.xv_inner
+    assert plan.bwd_workspace_bytes == planes * plan.xv_inner * 4
+
+
+@pytest.mark.parametrize("shape,code", [
+    ((1, 6, 4, 4, 16, 4, 6, 0), -2),     # dim % n_groups != 0      (selective_scan_oflex.cpp:215)
+    ((1, 8, 4, 4, 16, 4, 3, 0), -2),     # dim % delta_dim != 0     (:216)
+    ((1, 8, 4, 4, 17, 4, 8, 0), -2),     # dstate > MAX_DSTATE      (:217)
+    ((0, 8, 4, 4, 16, 4, 8, 0), -2),
+    ((1, 8, 4, 4, 16, 4, 8, 7), -3),     # unknown dtype            (:190)
+])
+def test_plan_rejects_what_the_reference_rejects(shape, code):
+    st, _ = capi.make_plan(capi.Shape(*shape))
+    assert st == code
+    assert len(capi.lib().snd_status_string(st)) > 0
+
+
+def test_entry_points_validate_before_touching_the_gpu():
+    lib = capi.lib()
+    assert lib.snd_fwd(None, None) == -1
+    assert lib.snd_bwd(None, None) == -1
+    fp = capi.FwdParams()
+    fp.shape = capi.Shape(1, 8, 4, 4, 16, 4, 8, capi.SND_F32)
+    assert lib.snd_fwd(C.byref(fp), None) == -1            # null tensors
+    fp.u = fp.delta = fp.A = fp.B = fp.C = 16
+    assert lib.snd_fwd(C.byref(fp), None) == -6            # saved state missing
+    fp.x_v = 24                                            # not 16-byte aligned
+    assert lib.snd_fwd(C.byref(fp), None) == -7
+    assert b"16-byte" in lib.snd_status_string(-7)
+
+
+def test_python_operator_has_no_cpu_fallback():
+    torch = pytest.importorskip("torch")
+    import selective_nd_scan as s
+    with pytest.raises(RuntimeError, match="GPU"):
+        s.selective_nd_scan(torch.zeros(1, 4, 3, 4), torch.zeros(1, 4, 3, 4), torch.zeros(4, 2),
+                            torch.zeros(1, 1, 2, 3, 4), torch.zeros(1, 1, 2, 3, 4))
+
+
+def test_extension_checks_mirror_reference_messages():
+    torch = pytest.importorskip("torch")
+    import selective_nd_scan as s
+    z = torch.zeros
+    with pytest.raises(RuntimeError):                       # A must be fp32 (:191)
+        s.fwd(z(1, 4, 3, 4), z(1, 4, 3, 4), z(4, 2, dtype=torch.float16), z(1, 1, 2, 3, 4), z(1, 1, 2, 3, 4))
+    with pytest.raises(RuntimeError):                       # dtype mismatch (:193)
+        s.fwd(z(1, 4, 3, 4), z(1, 4, 3, 4, dtype=torch.float16), z(4, 2), z(1, 1, 2, 3, 4), z(1, 1, 2, 3, 4))
