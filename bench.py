@@ -1,0 +1,185 @@
+"""Benchmark of the 2D-CrossScan selective scan (selective_nd_scan fwd + bwd) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c4n1] [--no-cpu]
+
+One step = one forward + one backward of the operator through the PyTorch extension (output,
+saved-state and gradient allocations, zero-fills and dtype casts included, as a caller of the
+reference's fwd/bwd bindings would pay them) on synthetic inputs already resident in HBM.
+Prints ONE JSON line.  `value` is the algorithmic HBM rate of the whole step:
+    bytes = (2eP + 2eQ + 4P) + (4eP + 4eQ + 4P),  P = B*D*H*W, Q = B*K*N*H*W, e = input bytes
+(compulsory tensor I/O only) divided by the mean step time.  `roofline` is the same figure for the
+dominant kernel alone (the backward), from HIP events around its launches on the launch stream;
+`cpu_baseline` times the C restatement of the reference recurrence (oracle/) on the host cores on
+a bounded sample of the same workload.
+"""
+import argparse
+import json
+import math
+import os
+import re
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "official-cross-scan_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+METRIC = "fwd+bwd 2D-scan ms/iter & HBM GB/s (% peak), B64 D192 56x56 N16 K4"
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published peak
+WORKLOADS = {                   # name: (B, D, H, W, N, K, input dtype)
+    "c1": (64, 192, 56, 56, 16, 4, "float32"),
+    "c2": (64, 768, 14, 14, 16, 4, "bfloat16"),
+    "c3": (2, 192, 200, 336, 16, 4, "float32"),
+    "c4": (1, 256, 512, 512, 16, 4, "bfloat16"),
+    "c4n1": (1, 256, 512, 512, 1, 4, "bfloat16"),
+}
+
+
+def algorithmic_bytes(Bt, Dm, H, W, N, K, e):
+    P, Q = Bt * Dm * H * W, Bt * K * N * H * W
+    return 2 * e * P + 2 * e * Q + 4 * P, 4 * e * P + 4 * e * Q + 4 * P
+
+
+def make_inputs(torch, Bt, Dm, H, W, N, K, dtype, dev):
+    """Value distributions of the headline metric, generated on the device, seed 0."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    u = rn(Bt, Dm, H, W).to(dtype)
+    delta = (0.1 * rn(Bt, Dm, H, W)).to(dtype)
+    dt = torch.exp(torch.empty(Dm, device=dev).uniform_(math.log(1e-3), math.log(1e-1), generator=g))
+    bias = torch.log(torch.expm1(dt))
+    A = -torch.arange(1, N + 1, device=dev, dtype=torch.float32).repeat(Dm, 1).contiguous()
+    B = rn(Bt, K, N, H, W).to(dtype)
+    C = rn(Bt, K, N, H, W).to(dtype)
+    D = torch.ones(Dm, device=dev)
+    dout = rn(Bt, Dm, H, W)
+    return u, delta, A, B, C, D, bias, dout
+
+
+def cpu_baseline(workload, budget_s=20.0):
+    """C restatement of the reference recurrence (fp32 state) on the host cores, fwd + bwd, on a
+    slice of the batch sized to take roughly `budget_s` seconds of CPU work."""
+    import numpy as np
+    from oracle import snd_oracle as O
+    from oracle import snd_oracle_c as OC
+    Bt, Dm, H, W, N, K, dtn = WORKLOADS[workload]
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    cores = int(env) if env.isdigit() and int(env) > 0 else (os.cpu_count() or 1)
+
+    def run(sb, sd):
+        d = O.make_inputs(sb, sd, H, W, N=N, K=K, seed=0)
+        a = (d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"])
+        t0 = time.perf_counter()
+        OC.fwd(*a, True, None, nthreads=cores)
+        OC.bwd(*a, d["dout"], True, None, nthreads=cores)
+        return time.perf_counter() - t0
+
+    # planes are independent, so a slice of the batch (of the channels when B == 1) is the same work
+    # per element; grow the slice until one fwd+bwd takes about budget_s of wall time
+    if Bt > 1:
+        sb, sd = min(Bt, max(1, (cores + K - 1) // K)), Dm
+    else:
+        sb, sd = 1, min(Dm, K * max(1, cores // K))
+    t = run(sb, sd)
+    if t < 0.5 * budget_s:
+        grow = budget_s / max(t, 1e-6)
+        if Bt > 1:
+            sb = int(max(sb, min(Bt, sb * grow)))
+        else:
+            sd = int(max(sd, min(Dm, (int(sd * grow) // K) * K)))
+        t = run(sb, sd)
+    fb, bb = algorithmic_bytes(sb, sd, H, W, N, K, 4)
+    return {"value": round((fb + bb) / t / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "%s slice B=%d D=%d (fp32 I/O, fp32 state), fwd+bwd once, %.1f s wall, %.3f ms per (b,c) plane set"
+                      % (workload, sb, sd, t, 1e3 * t / (sb * sd)),
+            "ms_per_step_extrapolated": round(1e3 * t * (Bt * Dm) / (sb * sd), 1)}
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary."""
+    path = os.path.join(ROOT, "profiles", "bwd_kernel_%s_pmc.txt" % workload)
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read())
+    return float(m.group(1)) if m else None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this operator is measured on ONE GPU (every (batch, channel, state) plane is an "
+                 "independent recurrence; multi-GPU is plain batch sharding and is not part of this build). "
+                 "Run with --gpus 1.")
+
+    import torch
+    import selective_nd_scan as snd
+    from selective_nd_scan import capi
+
+    dev = torch.device("cuda:0")
+    Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
+    dtype = getattr(torch, dtn)
+    u, delta, A, B, C, D, bias, dout = make_inputs(torch, Bt, Dm, H, W, N, K, dtype, dev)
+    fb, bb = algorithmic_bytes(Bt, Dm, H, W, N, K, u.element_size())
+
+    def step():
+        out, x, x_v, x_sd = snd.fwd(u, delta, A, B, C, D, bias, True, True, None)
+        return snd.bwd(u, delta, A, B, C, D, bias, dout, x, x_v, True, None, x_sd)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # kernel-only durations: HIP events on the launch stream around each launch through the C ABI
+    fcall = capi.FwdCall(u, delta, A, B, C, D, bias, True, True, None)
+    fcall.launch()
+    bcall = capi.BwdCall(u, delta, A, B, C, D, bias, dout, fcall.x, fcall.x_v, True, None, fcall.x_sd)
+    stream = torch.cuda.current_stream()
+    kf, kb = [], []
+    for i in range(args.warmup + args.steps):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        bcall.zero()
+        e[0].record(stream); fcall.launch(); e[1].record(stream)
+        e[2].record(stream); bcall.launch_kernel_only(); e[3].record(stream)
+        torch.cuda.synchronize()
+        if i >= args.warmup:
+            kf.append(e[0].elapsed_time(e[1]))
+            kb.append(e[2].elapsed_time(e[3]))
+    kf_ms, kb_ms = sum(kf) / len(kf), sum(kb) / len(kb)
+
+    value = (fb + bb) / (ms * 1e-3) / 1e9
+    achieved = bb / (kb_ms * 1e-3) / 1e9
+    rec = {
+        "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: selective_nd_scan fwd+bwd, B=%d D=%d H=%d W=%d N=%d K=%d, %s inputs, fp32 state"
+                               % (args.workload, Bt, Dm, H, W, N, K, dtn),
+                   "algorithmic_bytes": fb + bb, "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+                   "pixels_per_s": round(Bt * Dm * H * W / (ms * 1e-3), 1),
+                   "state_cells_per_s": round(Bt * Dm * H * W * N / (ms * 1e-3), 1),
+                   "kernel_ms": {"fwd": round(kf_ms, 4), "bwd": round(kb_ms, 4)},
+                   "kernel_only_GBs": round((fb + bb) / ((kf_ms + kb_ms) * 1e-3) / 1e9, 2)},
+        "roofline": {"bound": "hbm", "kernel": "snd::bwd_kernel", "achieved": round(achieved, 2),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(args.workload), "algorithmic_bytes_per_launch": bb},
+    }
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

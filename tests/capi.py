@@ -1,162 +1,4 @@
-"""ctypes binding of include/snd_scan.h used by the tests (and by nothing in the shipped package).
-
-It drives libsnd_scan.so exactly as a foreign host would: plain pointers, sizes and a stream.
-torch is used only to own device memory.
-"""
-import ctypes as C
-import os
-import re
-
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(ROOT, "official-cross-scan_amd", "libsnd_scan.so")
-HEADER = os.path.join(ROOT, "include", "snd_scan.h")
-
-SND_F32, SND_F16, SND_BF16 = 0, 1, 2
-i32, i64, vp = C.c_int32, C.c_int64, C.c_void_p
-
-
-class Shape(C.Structure):
-    _fields_ = [(n, i32) for n in ("batch", "dim", "nrows", "ncols", "dstate", "n_groups", "delta_dim", "in_dtype")]
-
-
-class Plan(C.Structure):
-    _fields_ = [("n_chunks_x", i32), ("n_chunks_y", i32), ("x_inner", i32), ("xv_inner", i32),
-                ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64)]
-
-
-class FwdParams(C.Structure):
-    _fields_ = ([("shape", Shape), ("out_dtype", i32), ("delta_softplus", i32)] +
-                [(n, vp) for n in ("u", "delta", "B", "C", "A", "D", "delta_bias", "A_decay", "out", "x", "x_v", "x_sd")] +
-                [(n, i64) for n in ("u_batch_stride", "u_d_stride", "u_h_stride",
-                                    "delta_batch_stride", "delta_d_stride", "delta_h_stride",
-                                    "A_d_stride", "A_dstate_stride",
-                                    "B_batch_stride", "B_group_stride", "B_dstate_stride", "B_h_stride",
-                                    "C_batch_stride", "C_group_stride", "C_dstate_stride", "C_h_stride",
-                                    "out_batch_stride", "out_d_stride", "out_h_stride")])
-
-
-class BwdParams(C.Structure):
-    _fields_ = ([("f", FwdParams), ("dout", vp), ("dout_dtype", i32)] +
-                [(n, i64) for n in ("dout_batch_stride", "dout_d_stride", "dout_h_stride")] +
-                [(n, vp) for n in ("du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias", "dA_decay", "workspace")] +
-                [("workspace_bytes", i64)])
-
-
-def declared_symbols():
-    """Every function include/snd_scan.h declares."""
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(snd_[a-z_]+)\s*\(", text)))
-
-
-_lib = None
-
-
-def lib():
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError("libsnd_scan.so is not built: run python official-cross-scan_amd/build.py")
-        _lib = C.CDLL(LIB_PATH)
-        _lib.snd_version.restype = C.c_int
-        _lib.snd_status_string.restype = C.c_char_p
-        _lib.snd_status_string.argtypes = [C.c_int]
-        _lib.snd_make_plan.argtypes = [C.POINTER(Shape), C.POINTER(Plan)]
-        _lib.snd_fwd.argtypes = [C.POINTER(FwdParams), vp]
-        _lib.snd_bwd.argtypes = [C.POINTER(BwdParams), vp]
-    return _lib
-
-
-def _dt(t):
-    import torch
-    return {torch.float32: SND_F32, torch.float16: SND_F16, torch.bfloat16: SND_BF16}[t.dtype]
-
-
-def make_shape(u, delta, A, B):
-    return Shape(u.shape[0], u.shape[1], u.shape[2], u.shape[3], A.shape[1], B.shape[1], delta.shape[1], _dt(u))
-
-
-def make_plan(shape):
-    plan = Plan()
-    st = lib().snd_make_plan(C.byref(shape), C.byref(plan))
-    return st, plan
-
-
-def _ptr(t):
-    return None if t is None else t.data_ptr()
-
-
-def _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, out, x, x_v, x_sd):
-    fp.shape = shape
-    fp.out_dtype = _dt(out) if out is not None else SND_F32
-    fp.delta_softplus = int(bool(delta_softplus))
-    fp.u, fp.delta, fp.B, fp.C, fp.A = _ptr(u), _ptr(delta), _ptr(B), _ptr(Cc), _ptr(A)
-    fp.D, fp.delta_bias, fp.A_decay = _ptr(D), _ptr(delta_bias), _ptr(A_decay)
-    fp.out, fp.x, fp.x_v, fp.x_sd = _ptr(out), _ptr(x), _ptr(x_v), _ptr(x_sd)
-    fp.u_batch_stride, fp.u_d_stride, fp.u_h_stride = u.stride(0), u.stride(1), u.stride(2)
-    fp.delta_batch_stride, fp.delta_d_stride, fp.delta_h_stride = delta.stride(0), delta.stride(1), delta.stride(2)
-    fp.A_d_stride, fp.A_dstate_stride = A.stride(0), A.stride(1)
-    fp.B_batch_stride, fp.B_group_stride, fp.B_dstate_stride, fp.B_h_stride = B.stride()[:4]
-    fp.C_batch_stride, fp.C_group_stride, fp.C_dstate_stride, fp.C_h_stride = Cc.stride()[:4]
-    if out is not None:
-        fp.out_batch_stride, fp.out_d_stride, fp.out_h_stride = out.stride(0), out.stride(1), out.stride(2)
-
-
-def check(st):
-    if st != 0:
-        raise RuntimeError("snd status %d: %s" % (st, lib().snd_status_string(st).decode()))
-
-
-def fwd(u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
-        save=True, stream=None):
-    """Reference operator `fwd` (selective_scan_oflex.cpp:179-187) through the C ABI."""
-    import torch
-    shape = make_shape(u, delta, A, B)
-    st, plan = make_plan(shape)
-    check(st)
-    Bt, Dm, N = u.shape[0], u.shape[1], A.shape[1]
-    f32 = dict(device=u.device, dtype=torch.float32)
-    out = torch.empty(u.shape, device=u.device, dtype=torch.float32 if out_float else u.dtype)
-    x_v = torch.empty((Bt, Dm, N, plan.n_chunks_y, plan.xv_inner), **f32)
-    x = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
-    x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
-    fp = FwdParams()
-    _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, out, x, x_v, x_sd)
-    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
-    check(lib().snd_fwd(C.byref(fp), s))
-    return out, x, x_v, x_sd
-
-
-def bwd(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, stream=None):
-    """Reference operator `bwd` (selective_scan_oflex.cpp:286-297, return list :432-438)."""
-    import torch
-    shape = make_shape(u, delta, A, B)
-    st, plan = make_plan(shape)
-    check(st)
-    Bt, Dm, H, W = u.shape
-    Dd = delta.shape[1]
-    f32 = dict(device=u.device, dtype=torch.float32)
-    du = torch.empty_like(u)
-    ddelta = torch.empty_like(u)
-    dA = torch.zeros_like(A)
-    dB = torch.zeros(B.shape, **f32)
-    dC = torch.zeros(Cc.shape, **f32)
-    dD = torch.zeros_like(D) if D is not None else None
-    dbias = torch.zeros(Dm, **f32) if delta_bias is not None else None
-    ddec = torch.zeros_like(A_decay) if A_decay is not None else None
-    ws = torch.empty(plan.bwd_workspace_bytes // 4 + 4, **f32)
-    bp = BwdParams()
-    _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd)
-    bp.dout, bp.dout_dtype = dout.data_ptr(), _dt(dout)
-    bp.dout_batch_stride, bp.dout_d_stride, bp.dout_h_stride = dout.stride(0), dout.stride(1), dout.stride(2)
-    bp.du, bp.ddelta, bp.dA, bp.dB, bp.dC = du.data_ptr(), ddelta.data_ptr(), dA.data_ptr(), dB.data_ptr(), dC.data_ptr()
-    bp.dD, bp.ddelta_bias, bp.dA_decay = _ptr(dD), _ptr(dbias), _ptr(ddec)
-    bp.workspace, bp.workspace_bytes = ws.data_ptr(), plan.bwd_workspace_bytes
-    s = torch.cuda.current_stream().cuda_stream if stream is None else stream
-    check(lib().snd_bwd(C.byref(bp), s))
-    dB, dC = dB.to(B.dtype), dC.to(Cc.dtype)
-    if Dd != Dm:
-        ddelta = ddelta.view(Bt, Dd, Dm // Dd, H, W).sum(2)
-        if dbias is not None:
-            dbias = dbias.view(Dd, Dm // Dd).sum(1)
-    return du, ddelta, dA, dB, dC, dD, dbias, ddec
+"""The tests drive the C ABI through the package's ctypes binding."""
+from selective_nd_scan.capi import *  # noqa: F401,F403
+from selective_nd_scan.capi import (BwdParams, FwdParams, Plan, Shape, bwd, check, declared_symbols, fwd, lib,  # noqa: F401
+                                    make_plan, make_shape)
