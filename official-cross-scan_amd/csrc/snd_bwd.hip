@@ -35,6 +35,25 @@ __device__ __forceinline__ void glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// v_permlane32_swap: upper 32 lanes of a <-> lower 32 lanes of b.  v_permlane16_swap: odd 16-lane
+// rows of a <-> even rows of b.  After either swap, a + b is the pair-sum of the value the lane keeps.
+__device__ __forceinline__ void swap32(float &a, float &b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap16(float &a, float &b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+// Sum v[0..7] over the four 16-lane rows of a wave (= its four channels when a row holds the 16
+// states of one channel).  Row q of the wave ends up with the totals of v[2q] and v[2q+1]:
+// a reduce-scatter, 12 swaps + 12 adds for 8 values instead of 16 for a broadcast sum.
+__device__ __forceinline__ void rows_reduce8(const float (&v)[8], float &w0, float &w1) {
+    float t[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { float a = v[k], b = v[k + 4]; swap32(a, b); t[k] = a + b; }
+    { float a = t[0], b = t[2]; swap16(a, b); w0 = a + b; }
+    { float a = t[1], b = t[3]; swap16(a, b); w1 = a + b; }
+}
+
 template <int NP>
 __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4;                     // waves per block
@@ -45,18 +64,22 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     constexpr int HG = 10, DLP = HG * HG;           // delta' on the tile plus a one-cell halo
     constexpr int NHALO = 36, NHK = (NHALO + NP - 1) / NP;
 
-    __shared__ __align__(16) float sB[NP * NSTR];
-    __shared__ __align__(16) float sC[NP * NSTR];
-    __shared__ __align__(16) float sdB[NP * NSTR];
-    __shared__ __align__(16) float sdC[NP * NSTR];
-    __shared__ __align__(16) float sDl[CB * DLP];
-    __shared__ __align__(16) float sDu[CB * kTile];   // delta' * u
-    __shared__ __align__(16) float sU[CB * kTile];
-    __shared__ __align__(16) float sDo[CB * kTile];   // dout
-    __shared__ __align__(16) float sSg[CB * kTile];   // d softplus / d raw
-    __shared__ __align__(16) float sQ[CB * kTile];    // sum_n dbu*B
-    __shared__ __align__(16) float sP[CB * kTile];    // sum_n A*da*a
-    __shared__ float sRed[WPB];
+    // NP == 16: a wave's four channels are reduced in registers (rows_reduce8) and every wave owns
+    // a partial dB/dC tile, written with plain stores.  NP == 8: one shared tile, LDS atomics.
+    constexpr int NPART = (NP == 16) ? WPB : 1;
+    extern __shared__ __align__(16) float smem[];
+    float *sB = smem;                               // [NP][NSTR]
+    float *sC = sB + NP * NSTR;
+    float *sdB = sC + NP * NSTR;                    // [NPART][NP][NSTR]
+    float *sdC = sdB + NPART * NP * NSTR;
+    float *sDl = sdC + NPART * NP * NSTR;           // [CB][DLP]
+    float *sDu = sDl + CB * DLP;                    // [CB][kTile] delta' * u
+    float *sU = sDu + CB * kTile;
+    float *sDo = sU + CB * kTile;                   // dout
+    float *sSg = sDo + CB * kTile;                  // d softplus / d raw
+    float *sQ = sSg + CB * kTile;                   // sum_n dbu*B
+    float *sP = sQ + CB * kTile;                    // sum_n A*da*a
+    float *sRed = sP + CB * kTile;                  // [WPB]
 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
@@ -92,21 +115,26 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;            // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
 
-    const int64_t plane = ((int64_t)b * Dm + cc) * N + nn;
-    const float *xv = f.x_v + plane * geo.nCY * geo.Wp;
-    const float *xh = f.x + plane * geo.nCX * geo.Hp;
-    const float *xs = f.x_sd + plane * geo.nCX * geo.Hp;
-    float *gdown = (float *)p.workspace + plane * geo.Wp;
+    // saved state and scratch, (channel, state) innermost (same layouts as the forward writes):
+    //   x_v [b][strip][col][c][n]   x, x_sd [b][col tile][row][c][n]   scratch G row [b][col][c][n]
+    const int64_t DN = (int64_t)Dm * N;
+    const int64_t lane_off = (int64_t)cc * N + nn;
+    const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.Wp * DN + lane_off;
+    const float *xh = f.x + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off;
+    const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off;
+    float *gdown = (float *)p.workspace + (int64_t)b * geo.Wp * DN + lane_off;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
     const float *myDo = sDo + cl * kTile;
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
-    float *mydB = sdB + n * NSTR;
-    float *mydC = sdC + n * NSTR;
+    float *mydB = sdB + (NP == 16 ? wave * NP * NSTR : 0) + n * NSTR;
+    float *mydC = sdC + (NP == 16 ? wave * NP * NSTR : 0) + n * NSTR;
+    const int qrow = (tid & 63) >> 4;               // 16-lane row of this lane inside its wave
 
-    for (int i = tid; i < NP * NSTR; i += 16 * NP) { sdB[i] = 0.f; sdC[i] = 0.f; }
+    if (NP != 16)
+        for (int i = tid; i < NP * NSTR; i += 16 * NP) { sdB[i] = 0.f; sdC[i] = 0.f; }
 
     // ---- register staging of one tile's raw inputs (global loads issued one tile ahead)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
@@ -205,32 +233,27 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;
             float Gd[kCkX];
             if (I > 0) {
-                const float4 *src = (const float4 *)(xv + (int64_t)(I - 1) * geo.Wp + j0);
-                const float4 v0 = src[0], v1 = src[1];
-                hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
-                hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
-                if (J > 0) hc = xv[(int64_t)(I - 1) * geo.Wp + j0 - 1];
+                const float *src = xv + ((int64_t)(I - 1) * geo.Wp + j0) * DN;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) hu[j] = src[j * DN];
+                if (J > 0) hc = src[-DN];
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
             if (J > 0) {
-                const float4 *sh_ = (const float4 *)(xh + (int64_t)(J - 1) * geo.Hp + r0);
-                const float4 *ss_ = (const float4 *)(xs + (int64_t)(J - 1) * geo.Hp + r0);
-                const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
-                hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
-                hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
-                slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
-                slft[4] = s1.x; slft[5] = s1.y; slft[6] = s1.z; slft[7] = s1.w;
+                const float *sh_ = xh + ((int64_t)(J - 1) * geo.Hp + r0) * DN;
+                const float *ss_ = xs + ((int64_t)(J - 1) * geo.Hp + r0) * DN;
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) { hlft[r] = sh_[r * DN]; slft[r] = ss_[r * DN]; }
             } else {
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
             }
             if (I + 1 < geo.nCY && lvalid) {
-                const float4 *src = (const float4 *)(gdown + j0);
-                const float4 v0 = src[0], v1 = src[1];
-                Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
-                Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
+                const float *src = gdown + (int64_t)j0 * DN;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) Gd[j] = src[j * DN];
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
@@ -281,7 +304,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                     }
                 }
                 float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
-                float q[kCkX], pp_[kCkX];
+                float q[kCkX], pp_[kCkX], vB[kCkX], vC[kCkX];
 #pragma unroll
                 for (int j = kCkX - 1; j >= 0; --j) {
                     const float dov = myDo[r * kCkX + j];
@@ -292,9 +315,9 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                     const float gs = Gsr - dyC;
                     const float dbu = fmaf(0.25f, dyC, g_ + gs);
                     q[j] = dbu * Bv;
-                    lds_add(mydB + r * kCkX + j, dbu * myDu[r * kCkX + j]);
+                    vB[j] = dbu * myDu[r * kCkX + j];
                     const float hb = hT[r][j] - bu[j], sb = s[j] - bu[j];
-                    lds_add(mydC + r * kCkX + j, dov * fmaf(0.25f, bu[j], hb - sb));
+                    vC[j] = dov * fmaf(0.25f, bu[j], hb - sb);
                     const float h_l = (j == 0) ? hlft[r] : hT[r][j - 1 < 0 ? 0 : j - 1];
                     const float h_u = (r == 0) ? hu[j] : hT[r - 1 < 0 ? 0 : r - 1][j];
                     const float cross = fmaf(Gd[j], h_l, Gr * h_u);
@@ -313,6 +336,16 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                 GsR[r] = Gsr;
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) adn[j] = arow[j];
+                if (NP == 16) {                     // sum over the wave's 4 channels, then one plain store
+                    float b0, b1, c0, c1;
+                    rows_reduce8(vB, b0, b1);
+                    rows_reduce8(vC, c0, c1);
+                    *(float2 *)(mydB + r * kCkX + 2 * qrow) = make_float2(b0, b1);
+                    *(float2 *)(mydC + r * kCkX + 2 * qrow) = make_float2(c0, c1);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kCkX; ++j) { lds_add(mydB + r * kCkX + j, vB[j]); lds_add(mydC + r * kCkX + j, vC[j]); }
+                }
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) { q[j] = group_sum<NP>(q[j]); pp_[j] = group_sum<NP>(pp_[j]); }
                 if (n == 0) {
@@ -326,9 +359,9 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             }
             GRc = gd_old0;
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
-                float4 *dst = (float4 *)(gdown + j0);
-                dst[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
-                dst[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
+                float *dst = gdown + (int64_t)j0 * DN;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) dst[j * DN] = Gd[j];
             }
             __syncthreads();
 
@@ -356,13 +389,18 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
 #pragma unroll
                 for (int k = 0; k < NBC; ++k) {
                     const int sn = wave + WPB * k;
+                    float tb = 0.f, tc = 0.f;
+#pragma unroll
+                    for (int w = 0; w < NPART; ++w) {
+                        tb += sdB[w * NP * NSTR + sn * NSTR + px];
+                        tc += sdC[w * NP * NSTR + sn * NSTR + px];
+                    }
                     if (in && sn < N) {
                         const int64_t o = (int64_t)sn * H * W + (int64_t)row * W + col;
-                        glb_add(dBg + o, sdB[sn * NSTR + px]);
-                        glb_add(dCg + o, sdC[sn * NSTR + px]);
+                        glb_add(dBg + o, tb);
+                        glb_add(dCg + o, tc);
                     }
-                    sdB[sn * NSTR + px] = 0.f;
-                    sdC[sn * NSTR + px] = 0.f;
+                    if (NP != 16) { sdB[sn * NSTR + px] = 0.f; sdC[sn * NSTR + px] = 0.f; }
                 }
             }
         }
@@ -400,7 +438,15 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
-    hipLaunchKernelGGL((bwd_kernel<NP>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+    constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = (NP == 16) ? WPB : 1;
+    constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void *)bwd_kernel<NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+            return SND_ERR_LAUNCH;
+        configured = true;
+    }
+    hipLaunchKernelGGL((bwd_kernel<NP>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 

@@ -69,10 +69,13 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
     const int64_t offD = (int64_t)b * p.delta_batch_stride + (int64_t)(cc / rd) * p.delta_d_stride;
     const int64_t offO = (int64_t)b * p.out_batch_stride + (int64_t)cc * p.out_d_stride;
 
-    const int64_t plane = ((int64_t)b * Dm + cc) * N + nn;
-    float *xv = p.x_v + plane * geo.nCY * geo.Wp;
-    float *xh = SAVE ? p.x + plane * geo.nCX * geo.Hp : nullptr;
-    float *xs = SAVE ? p.x_sd + plane * geo.nCX * geo.Hp : nullptr;
+    // saved state, (channel, state) innermost so that a wave's 64 planes touch one contiguous run:
+    //   x_v  [b][strip I][col][c][n]      x, x_sd  [b][col tile J][row][c][n]
+    const int64_t DN = (int64_t)Dm * N;
+    const int64_t lane_off = (int64_t)cc * N + nn;
+    float *xv = p.x_v + (int64_t)b * geo.nCY * geo.Wp * DN + lane_off;
+    float *xh = SAVE ? p.x + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off : nullptr;
+    float *xs = SAVE ? p.x_sd + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off : nullptr;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
@@ -81,8 +84,15 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
 
     // raw values of one tile, held in registers between their global load and their LDS commit
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo = 0.f;
+    float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto prefetch = [&](int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
+        if (I > 0 && geo.nCX > 1) {                 // with one column tile the row comes from registers
+            const float *src = xv + ((int64_t)(I - 1) * geo.Wp + j0) * DN;
+#pragma unroll
+            for (int j = 0; j < kCkX; ++j) qxv[j] = src[j * DN];
+            qcorner = J > 0 ? src[-DN] : 0.f;
+        }
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
@@ -141,6 +151,11 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
         for (int J = 0; J < geo.nCX; ++J) {
             const int j0 = J * kCkX;
             commit();
+            // row above this tile: fetched one tile ahead (or handed over in registers)
+            float hup[kCkX], aup[kCkX];
+            float corner = (I > 0) ? qcorner : 0.f; // h[r0-1][j0-1]
+#pragma unroll
+            for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
             __syncthreads();
             {   // issue the next tile's loads now; they complete while this tile is computed
                 int In = I, Jn = J + 1;
@@ -149,20 +164,8 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
             }
 
             // ---- per-lane tile walk
-            float hup[kCkX], aup[kCkX];             // row above the current one
-            float corner = 0.f;                     // h[r0-1][j0-1]
-            if (I > 0) {
-                const float4 *src = (const float4 *)(xv + (int64_t)(I - 1) * geo.Wp + j0);
-                const float4 v0 = src[0], v1 = src[1];
-                hup[0] = v0.x; hup[1] = v0.y; hup[2] = v0.z; hup[3] = v0.w;
-                hup[4] = v1.x; hup[5] = v1.y; hup[6] = v1.z; hup[7] = v1.w;
 #pragma unroll
-                for (int j = 0; j < kCkX; ++j) aup[j] = fast_exp2(fmaf(myDl[j], A2, ld));
-                if (J > 0) corner = xv[(int64_t)(I - 1) * geo.Wp + j0 - 1];
-            } else {
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) { hup[j] = 0.f; aup[j] = 0.f; }
-            }
+            for (int j = 0; j < kCkX; ++j) aup[j] = (I > 0) ? fast_exp2(fmaf(myDl[j], A2, ld)) : 0.f;
 
 #pragma unroll
             for (int r = 0; r < kRows; ++r) {
@@ -203,18 +206,21 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
                     dst[1] = make_float4(y[4], y[5], y[6], y[7]);
                 }
             }
+            if (geo.nCX == 1) {                     // the next strip's row above is this tile's last row
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];
+                qcorner = 0.f;
+            }
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
-                float4 *dst = (float4 *)(xv + (int64_t)I * geo.Wp + j0);
-                dst[0] = make_float4(hup[0], hup[1], hup[2], hup[3]);
-                dst[1] = make_float4(hup[4], hup[5], hup[6], hup[7]);
+                float *dst = xv + ((int64_t)I * geo.Wp + j0) * DN;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) dst[j * DN] = hup[j];
                 if (SAVE && J + 1 < geo.nCX) {      // column checkpoints: only if a tile follows
-                    float4 *dh = (float4 *)(xh + (int64_t)J * geo.Hp + r0);
-                    float4 *ds = (float4 *)(xs + (int64_t)J * geo.Hp + r0);
-                    dh[0] = make_float4(hl[0], hl[1], hl[2], hl[3]);
-                    dh[1] = make_float4(hl[4], hl[5], hl[6], hl[7]);
-                    ds[0] = make_float4(sl[0], sl[1], sl[2], sl[3]);
-                    ds[1] = make_float4(sl[4], sl[5], sl[6], sl[7]);
+                    float *dh = xh + ((int64_t)J * geo.Hp + r0) * DN;
+                    float *ds = xs + ((int64_t)J * geo.Hp + r0) * DN;
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r) { dh[r * DN] = hl[r]; ds[r * DN] = sl[r]; }
                 }
             }
             __syncthreads();
