@@ -24,6 +24,7 @@
 // du/ddelta are reduced over states by DPP and finished once per pixel by the thread that staged it.
 // As in the forward, tiles are computed in full on zero-padded staging (dout = B = C = 0 outside
 // the plane makes every adjoint there exactly zero), so the inner loops have no bounds checks.
+#pragma once
 #include "snd_device.h"
 
 namespace snd {
@@ -54,7 +55,20 @@ __device__ __forceinline__ void rows_reduce8(const float (&v)[8], float &w0, flo
     { float a = t[1], b = t[3]; swap16(a, b); w1 = a + b; }
 }
 
-template <int NP>
+// Explicit use of the accumulation half of the unified register file as storage.
+#ifdef SND_TILE_IN_AGPR
+__device__ __forceinline__ void acc_put(float &slot, float v) { asm("v_accvgpr_write_b32 %0, %1" : "=a"(slot) : "v"(v)); }
+__device__ __forceinline__ float acc_get(const float &slot) {
+    float v;
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(slot));
+    return v;
+}
+#else
+__device__ __forceinline__ void acc_put(float &slot, float v) { slot = v; }
+__device__ __forceinline__ float acc_get(const float &slot) { return slot; }
+#endif
+
+template <typename T, int NP>
 __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
@@ -83,7 +97,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
-    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups, dt = sh.in_dtype;
+    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
@@ -106,23 +120,30 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     const float bias = f.delta_bias ? f.delta_bias[cc / rd] : 0.f;
     const bool softplus = f.delta_softplus != 0;
 
-    const int64_t offB = (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
-    const int64_t offC = (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
-    const int64_t offU = (int64_t)b * f.u_batch_stride + (int64_t)cc * f.u_d_stride;
-    const int64_t offD = (int64_t)b * f.delta_batch_stride + (int64_t)(cc / rd) * f.delta_d_stride;
-    const int64_t offDo = (int64_t)b * p.dout_batch_stride + (int64_t)cc * p.dout_d_stride;
-    const int64_t offG = ((int64_t)b * Dm + cc) * H * W;             // du, ddelta: dense [b, c, H, W]
+    // per-batch-image base pointers (uniform) and 32-bit offsets inside the image
+    const T *Bb = (const T *)f.B + (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
+    const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
+    const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride;
+    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride;
+    const int esz_do = p.dout_dtype == SND_F32 ? 4 : 2;
+    const void *dob = (const char *)p.dout + (int64_t)b * p.dout_batch_stride * esz_do;
+    T *dub = (T *)p.du + (int64_t)b * Dm * H * W;                    // du, ddelta: dense [b, c, H, W]
+    T *ddb = (T *)p.ddelta + (int64_t)b * Dm * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;            // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
+    const int cU = cc * (int)f.u_d_stride, cD = (cc / rd) * (int)f.delta_d_stride, cDo = cc * (int)p.dout_d_stride;
+    const int cG = cc * H * W;
+    const int Bh = (int)f.B_h_stride, Ch = (int)f.C_h_stride, Uh = (int)f.u_h_stride, Dh = (int)f.delta_h_stride;
+    const int Bs = (int)f.B_dstate_stride, Cs = (int)f.C_dstate_stride, Doh = (int)p.dout_h_stride;
 
-    // saved state and scratch, (channel, state) innermost (same layouts as the forward writes):
-    //   x_v [b][strip][col][c][n]   x, x_sd [b][col tile][row][c][n]   scratch G row [b][col][c][n]
-    const int64_t DN = (int64_t)Dm * N;
-    const int64_t lane_off = (int64_t)cc * N + nn;
-    const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.Wp * DN + lane_off;
-    const float *xh = f.x + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off;
-    const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off;
-    float *gdown = (float *)p.workspace + (int64_t)b * geo.Wp * DN + lane_off;
+    // saved state and scratch, tile-major with the lane's 8 values innermost (as the forward writes):
+    //   x_v [b][I][J][c][n][8 cols]   x, x_sd [b][J][I][c][n][8 rows]   scratch G row [b][J][c][n][8 cols]
+    const int64_t DN8 = (int64_t)Dm * N * 8;
+    const int64_t lane_off = ((int64_t)cc * N + nn) * 8;
+    const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
+    const float *xh = f.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
+    const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
+    float *gdown = (float *)p.workspace + (int64_t)b * geo.nCX * DN8 + lane_off;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
@@ -140,15 +161,18 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
+        // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
+            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int ob = rc * Bh + cx, oc = rc * Ch + cx;
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
-                const int sn = wave + WPB * k;
-                const bool ok = in && sn < N;
-                qb[k] = ok ? ld_f32(f.B, offB + (int64_t)sn * f.B_dstate_stride + (int64_t)row * f.B_h_stride + col, dt) : 0.f;
-                qc[k] = ok ? ld_f32(f.C, offC + (int64_t)sn * f.C_dstate_stride + (int64_t)row * f.C_h_stride + col, dt) : 0.f;
+                const int sn = wave + WPB * k, sc = min(sn, N - 1);
+                const float vb = ldg(Bb, sc * Bs + ob), vc = ldg(Cb, sc * Cs + oc);
+                qb[k] = (in && sn < N) ? vb : 0.f;
+                qc[k] = (in && sn < N) ? vc : 0.f;
             }
         }
 #pragma unroll
@@ -156,9 +180,12 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            qdl[k] = ok ? ld_f32(f.delta, offD + (int64_t)row * f.delta_h_stride + col, dt) : 0.f;
-            qu[k] = ok ? ld_f32(f.u, offU + (int64_t)row * f.u_h_stride + col, dt) : 0.f;
-            qdo[k] = ok ? ld_f32(p.dout, offDo + (int64_t)row * p.dout_h_stride + col, p.dout_dtype) : 0.f;
+            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
+            const float vo = ld_f32(dob, cDo + rc * Doh + cx, p.dout_dtype);
+            qdl[k] = ok ? vd : 0.f;
+            qu[k] = ok ? vu : 0.f;
+            qdo[k] = ok ? vo : 0.f;
         }
 #pragma unroll
         for (int k = 0; k < NHK; ++k) {   // the 36 halo cells of the 10x10 delta' grid
@@ -169,8 +196,9 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             else if (hidx < 28) { rr = hidx - 19; jj = 0; }
             else { rr = hidx - 27; jj = 9; }
             const int row = r0 - 1 + rr, col = j0 - 1 + jj;
-            const bool ok = hidx < NHALO && cvalid && row >= 0 && row < H && col >= 0 && col < W;
-            qh[k] = ok ? ld_f32(f.delta, offD + (int64_t)row * f.delta_h_stride + col, dt) : 0.f;
+            const bool ok = cvalid && row >= 0 && row < H && col >= 0 && col < W;
+            const float vd = ldg(db, cD + min(max(row, 0), H - 1) * Dh + min(max(col, 0), W - 1));
+            qh[k] = ok ? vd : 0.f;
         }
     };
     auto commit = [&]() {
@@ -230,30 +258,71 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             }
 
             // ---- checkpoints and carried adjoints of this tile
-            float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;
+            // h on the tile and its upper/left halo lives in 81 accumulation registers (AGPRs):
+            // HA(r, j), r, j in -1..7.  Rows are moved to VGPRs only while they are being used.
+            float hA[kRows + 1][kCkX + 1];
+#define HA(r, j) hA[(r) + 1][(j) + 1]
+            float slft[kRows];
             float Gd[kCkX];
-            if (I > 0) {
-                const float *src = xv + ((int64_t)(I - 1) * geo.Wp + j0) * DN;
+            {
+                float hu[kCkX], hlft[kRows], hc = 0.f;
+                if (I > 0) {
+                    const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+                    const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                    hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
+                    hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
+                    if (J > 0) hc = src[7 - DN8];
+                } else {
 #pragma unroll
-                for (int j = 0; j < kCkX; ++j) hu[j] = src[j * DN];
-                if (J > 0) hc = src[-DN];
-            } else {
+                    for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
+                }
+                if (J > 0) {
+                    const float4 *sh_ = (const float4 *)(xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
+                    const float4 *ss_ = (const float4 *)(xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
+                    const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
+                    hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
+                    hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
+                    slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
+                    slft[4] = s1.x; slft[5] = s1.y; slft[6] = s1.z; slft[7] = s1.w;
+                } else {
 #pragma unroll
-                for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
-            }
-            if (J > 0) {
-                const float *sh_ = xh + ((int64_t)(J - 1) * geo.Hp + r0) * DN;
-                const float *ss_ = xs + ((int64_t)(J - 1) * geo.Hp + r0) * DN;
+                    for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
+                }
+                acc_put(HA(-1, -1), hc);
 #pragma unroll
-                for (int r = 0; r < kRows; ++r) { hlft[r] = sh_[r * DN]; slft[r] = ss_[r * DN]; }
-            } else {
+                for (int j = 0; j < kCkX; ++j) acc_put(HA(-1, j), hu[j]);
 #pragma unroll
-                for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
+                for (int r = 0; r < kRows; ++r) acc_put(HA(r, -1), hlft[r]);
+
+                // ---- recompute h on the tile (row r-1 stays in VGPRs as the "up" row)
+                float aprev[kCkX], hprev[kCkX];
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) { aprev[j] = AEXP(-1, j); hprev[j] = hu[j]; }
+                float diag0 = hc;                   // h[r-1][-1]
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    float al = AEXP(r, -1);
+                    float left = hlft[r];
+                    float diag = diag0;
+                    diag0 = hlft[r];
+#pragma unroll
+                    for (int j = 0; j < kCkX; ++j) {
+                        const float a = AEXP(r, j);
+                        const float bu = myB[r * kCkX + j] * myDu[r * kCkX + j];
+                        const float up = hprev[j];
+                        const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
+                        const float h = fmaf(a, left + X, bu);
+                        acc_put(HA(r, j), h);
+                        hprev[j] = h;
+                        diag = up; left = h; al = a; aprev[j] = a;
+                    }
+                }
             }
             if (I + 1 < geo.nCY && lvalid) {
-                const float *src = gdown + (int64_t)j0 * DN;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) Gd[j] = src[j * DN];
+                const float4 *src = (const float4 *)(gdown + (int64_t)J * DN8);
+                const float4 v0 = src[0], v1 = src[1];
+                Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
+                Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
@@ -261,68 +330,45 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
             const float gd_old0 = Gd[0];            // G[r0+8][j0]: the corner of the tile on the left
             float Gd8 = GRc;
 
-            // ---- recompute h on the tile
-            float hT[kRows][kCkX];
-            {
-                float aprev[kCkX];
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) aprev[j] = AEXP(-1, j);
-#pragma unroll
-                for (int r = 0; r < kRows; ++r) {
-                    float al = AEXP(r, -1);
-                    float left = hlft[r];
-                    float diag = (r == 0) ? hc : hlft[r - 1 < 0 ? 0 : r - 1];
-#pragma unroll
-                    for (int j = 0; j < kCkX; ++j) {
-                        const float a = AEXP(r, j);
-                        const float bu = myB[r * kCkX + j] * myDu[r * kCkX + j];
-                        const float up = (r == 0) ? hu[j] : hT[r - 1 < 0 ? 0 : r - 1][j];
-                        const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
-                        const float h = fmaf(a, left + X, bu);
-                        hT[r][j] = h;
-                        diag = up; left = h; al = a; aprev[j] = a;
-                    }
-                }
-            }
-
             // ---- reverse sweep
             float adn[kCkX];
+            float hcur[kCkX + 1], hupr[kCkX];       // h rows r (with left halo) and r-1, in VGPRs
 #pragma unroll
             for (int j = 0; j < kCkX; ++j) adn[j] = AEXP(kRows, j);
 #pragma unroll
+            for (int j = -1; j < kCkX; ++j) hcur[j + 1] = acc_get(HA(kRows - 1, j));
+#pragma unroll
             for (int r = kRows - 1; r >= 0; --r) {
-                float arow[kCkX + 1], bu[kCkX], s[kCkX];
+                __builtin_amdgcn_sched_barrier(0);
+                float arow[kCkX + 1], s[kCkX];
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) hupr[j] = acc_get(HA(r - 1, j));
 #pragma unroll
                 for (int j = 0; j <= kCkX; ++j) arow[j] = AEXP(r, j);
                 {
                     float sp = slft[r];
 #pragma unroll
                     for (int j = 0; j < kCkX; ++j) {
-                        bu[j] = myB[r * kCkX + j] * myDu[r * kCkX + j];
-                        sp = fmaf(arow[j], sp, bu[j]);
+                        sp = fmaf(arow[j], sp, myB[r * kCkX + j] * myDu[r * kCkX + j]);
                         s[j] = sp;
                     }
                 }
                 float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
-                float q[kCkX], pp_[kCkX], vB[kCkX], vC[kCkX];
+                float q[4], pp_[4], vB[4], vC[4], tB[4], tC[4];
 #pragma unroll
                 for (int j = kCkX - 1; j >= 0; --j) {
                     const float dov = myDo[r * kCkX + j];
                     const float Bv = myB[r * kCkX + j], Cv = myC[r * kCkX + j];
+                    const float duv = myDu[r * kCkX + j];
+                    const float bu = Bv * duv;
                     const float dyC = dov * Cv;
                     const float a = arow[j];
                     const float g_ = fmaf(-0.5f * (arow[j + 1] + adn[j]), Gdiag, dyC + Gr + Gd[j]);
                     const float gs = Gsr - dyC;
                     const float dbu = fmaf(0.25f, dyC, g_ + gs);
-                    q[j] = dbu * Bv;
-                    vB[j] = dbu * myDu[r * kCkX + j];
-                    const float hb = hT[r][j] - bu[j], sb = s[j] - bu[j];
-                    vC[j] = dov * fmaf(0.25f, bu[j], hb - sb);
-                    const float h_l = (j == 0) ? hlft[r] : hT[r][j - 1 < 0 ? 0 : j - 1];
-                    const float h_u = (r == 0) ? hu[j] : hT[r - 1 < 0 ? 0 : r - 1][j];
-                    const float cross = fmaf(Gd[j], h_l, Gr * h_u);
+                    const float hb = hcur[j + 1] - bu, sb = s[j] - bu;
+                    const float cross = fmaf(Gd[j], hcur[j], Gr * hupr[j]);
                     const float da = fmaf(-0.5f * a, cross, fmaf(g_, hb, gs * sb));
-                    pp_[j] = Av * da;
                     dA_acc = fmaf(DL(r, j), da, dA_acc);
                     dec_acc += da;
                     const float Gn = a * g_;
@@ -330,38 +376,48 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                     Gd[j] = Gn;
                     Gr = Gn;
                     Gsr = a * gs;
+                    // per-pixel sums over states, flushed per half row
+                    q[j & 3] = group_sum<NP>(dbu * Bv);
+                    pp_[j & 3] = group_sum<NP>(Av * da);
+                    if ((j & 3) == 0 && n == 0) {
+                        *(float4 *)(sQ + cl * kTile + r * kCkX + j) = make_float4(q[0], q[1], q[2], q[3]);
+                        *(float4 *)(sP + cl * kTile + r * kCkX + j) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
+                    }
+                    // dB, dC contributions: summed over the wave's channels pair by pair (j, j+4)
+                    const float vb = dbu * duv, vc = dov * fmaf(0.25f, bu, hb - sb);
+                    if (NP == 16) {
+                        if (j >= 4) { vB[j - 4] = vb; vC[j - 4] = vc; }
+                        else {
+                            float a0 = vb, a1 = vB[j]; swap32(a0, a1); tB[j] = a0 + a1;
+                            float c0 = vc, c1 = vC[j]; swap32(c0, c1); tC[j] = c0 + c1;
+                        }
+                    } else {
+                        lds_add(mydB + r * kCkX + j, vb);
+                        lds_add(mydC + r * kCkX + j, vc);
+                    }
+                }
+                if (NP == 16) {
+                    float b0, b1, c0, c1;
+                    { float x0 = tB[0], x1 = tB[2]; swap16(x0, x1); b0 = x0 + x1; }
+                    { float x0 = tB[1], x1 = tB[3]; swap16(x0, x1); b1 = x0 + x1; }
+                    { float x0 = tC[0], x1 = tC[2]; swap16(x0, x1); c0 = x0 + x1; }
+                    { float x0 = tC[1], x1 = tC[3]; swap16(x0, x1); c1 = x0 + x1; }
+                    *(float2 *)(mydB + r * kCkX + 2 * qrow) = make_float2(b0, b1);
+                    *(float2 *)(mydC + r * kCkX + 2 * qrow) = make_float2(c0, c1);
                 }
                 Gd8 = GR[r];                        // G[r][j0+8]: diagonal neighbour for the row above
                 GR[r] = Gr;                         // G[r][j0]: right neighbour for the tile on the left
                 GsR[r] = Gsr;
 #pragma unroll
-                for (int j = 0; j < kCkX; ++j) adn[j] = arow[j];
-                if (NP == 16) {                     // sum over the wave's 4 channels, then one plain store
-                    float b0, b1, c0, c1;
-                    rows_reduce8(vB, b0, b1);
-                    rows_reduce8(vC, c0, c1);
-                    *(float2 *)(mydB + r * kCkX + 2 * qrow) = make_float2(b0, b1);
-                    *(float2 *)(mydC + r * kCkX + 2 * qrow) = make_float2(c0, c1);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < kCkX; ++j) { lds_add(mydB + r * kCkX + j, vB[j]); lds_add(mydC + r * kCkX + j, vC[j]); }
-                }
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) { q[j] = group_sum<NP>(q[j]); pp_[j] = group_sum<NP>(pp_[j]); }
-                if (n == 0) {
-                    float4 *dq = (float4 *)(sQ + cl * kTile + r * kCkX);
-                    float4 *dp = (float4 *)(sP + cl * kTile + r * kCkX);
-                    dq[0] = make_float4(q[0], q[1], q[2], q[3]);
-                    dq[1] = make_float4(q[4], q[5], q[6], q[7]);
-                    dp[0] = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
-                    dp[1] = make_float4(pp_[4], pp_[5], pp_[6], pp_[7]);
-                }
+                for (int j = 0; j < kCkX; ++j) { adn[j] = arow[j]; hcur[j + 1] = hupr[j]; }
+                hcur[0] = acc_get(HA(r - 1, -1));
             }
+#undef HA
             GRc = gd_old0;
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
-                float *dst = gdown + (int64_t)j0 * DN;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) dst[j * DN] = Gd[j];
+                float4 *dst = (float4 *)(gdown + (int64_t)J * DN8);
+                dst[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
+                dst[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
             }
             __syncthreads();
 
@@ -378,8 +434,8 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                 dD_acc = fmaf(dov, uv, dD_acc);
                 dbias_acc += ddl;
                 if (cvalid && row < H && col < W) {
-                    st_f32(p.du, offG + (int64_t)row * W + col, dt, duv);
-                    st_f32(p.ddelta, offG + (int64_t)row * W + col, dt, ddl);
+                    stg(dub, cG + row * W + col, duv);
+                    stg(ddb, cG + row * W + col, ddl);
                 }
             }
             // ---- dB, dC of this tile leave the block (summed over its channels)
@@ -396,7 +452,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                         tc += sdC[w * NP * NSTR + sn * NSTR + px];
                     }
                     if (in && sn < N) {
-                        const int64_t o = (int64_t)sn * H * W + (int64_t)row * W + col;
+                        const int o = (sn * H + row) * W + col;
                         glb_add(dBg + o, tb);
                         glb_add(dCg + o, tc);
                     }
@@ -431,7 +487,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     }
 }
 
-template <int NP>
+template <typename T, int NP>
 static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const Geo geo = make_geo(sh.nrows, sh.ncols);
@@ -442,16 +498,18 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void *)bwd_kernel<NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void *)bwd_kernel<T, NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return SND_ERR_LAUNCH;
         configured = true;
     }
-    hipLaunchKernelGGL((bwd_kernel<NP>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
+    hipLaunchKernelGGL((bwd_kernel<T, NP>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
-int launch_bwd(const snd_bwd_params &p, hipStream_t stream) {
-    return p.f.shape.dstate > 8 ? launch_bwd_np<16>(p, stream) : launch_bwd_np<8>(p, stream);
+// One instantiation per input dtype, each in its own translation unit.
+template <typename T>
+int launch_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
+    return p.f.shape.dstate > 8 ? launch_bwd_np<T, 16>(p, stream) : launch_bwd_np<T, 8>(p, stream);
 }
 
 }  // namespace snd

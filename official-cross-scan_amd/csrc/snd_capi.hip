@@ -4,8 +4,12 @@
 #include "snd_device.h"
 
 namespace snd {
-int launch_fwd(const snd_fwd_params &p, hipStream_t stream);
-int launch_bwd(const snd_bwd_params &p, hipStream_t stream);
+int launch_fwd_f32(const snd_fwd_params &p, hipStream_t stream);
+int launch_fwd_bf16(const snd_fwd_params &p, hipStream_t stream);
+int launch_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
+int launch_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
+int launch_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
+int launch_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
 }  // namespace snd
 
 namespace {
@@ -23,6 +27,12 @@ int check_shape(const snd_shape &s) {
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+// The kernels address inside one batch image with 32-bit offsets.
+bool fits32(int64_t a_count, int64_t a_stride, int64_t b_count, int64_t b_stride, int64_t tail) {
+    if (a_stride < 0 || b_stride < 0) return false;
+    return (a_count - 1) * a_stride + (b_count - 1) * b_stride + tail < ((int64_t)1 << 31);
+}
+
 int check_fwd(const snd_fwd_params &p, bool need_state) {
     int st = check_shape(p.shape);
     if (st != SND_OK) return st;
@@ -34,6 +44,13 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
     if (p.u_h_stride < p.shape.ncols || p.delta_h_stride < p.shape.ncols || p.B_h_stride < p.shape.ncols ||
         p.C_h_stride < p.shape.ncols)
         if (p.shape.nrows > 1) return SND_ERR_STRIDE;
+    const snd_shape &s = p.shape;
+    if (!fits32(s.dim, p.u_d_stride, s.nrows, p.u_h_stride, s.ncols) ||
+        !fits32(s.delta_dim, p.delta_d_stride, s.nrows, p.delta_h_stride, s.ncols) ||
+        !fits32(s.dstate, p.B_dstate_stride, s.nrows, p.B_h_stride, s.ncols) ||
+        !fits32(s.dstate, p.C_dstate_stride, s.nrows, p.C_h_stride, s.ncols) ||
+        (int64_t)s.dim * s.nrows * s.ncols >= ((int64_t)1 << 31))
+        return SND_ERR_STRIDE;
     return SND_OK;
 }
 
@@ -49,7 +66,7 @@ const char *snd_status_string(int status) {
         case SND_ERR_NULL: return "a required pointer is null";
         case SND_ERR_SHAPE: return "bad shape: need dim % n_groups == 0, dim % delta_dim == 0, 1 <= dstate <= 16, all sizes > 0";
         case SND_ERR_DTYPE: return "unsupported dtype combination (inputs fp32/fp16/bf16; out and dout fp32 or the input dtype)";
-        case SND_ERR_STRIDE: return "bad stride: rows must not overlap and the last dimension must be contiguous";
+        case SND_ERR_STRIDE: return "bad stride: rows must not overlap, the last dimension must be contiguous and one batch image must span fewer than 2^31 elements";
         case SND_ERR_LAUNCH: return "kernel launch failed";
         case SND_ERR_WORKSPACE: return "saved state (x, x_v, x_sd) or workspace missing or too small";
         case SND_ERR_ALIGN: return "saved state / workspace pointers must be 16-byte aligned";
@@ -81,7 +98,13 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->out) return SND_ERR_NULL;
     if (params->out_dtype != SND_F32 && params->out_dtype != params->shape.in_dtype) return SND_ERR_DTYPE;
-    return snd::launch_fwd(*params, (hipStream_t)stream);
+    if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols))
+        return SND_ERR_STRIDE;
+    switch (params->shape.in_dtype) {
+        case SND_F32: return snd::launch_fwd_f32(*params, (hipStream_t)stream);
+        case SND_BF16: return snd::launch_fwd_bf16(*params, (hipStream_t)stream);
+        default: return snd::launch_fwd_f16(*params, (hipStream_t)stream);
+    }
 }
 
 int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
@@ -99,7 +122,14 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
     if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
-    return snd::launch_bwd(*params, (hipStream_t)stream);
+    if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
+                params->f.shape.ncols))
+        return SND_ERR_STRIDE;
+    switch (params->f.shape.in_dtype) {
+        case SND_F32: return snd::launch_bwd_f32(*params, (hipStream_t)stream);
+        case SND_BF16: return snd::launch_bwd_bf16(*params, (hipStream_t)stream);
+        default: return snd::launch_bwd_f16(*params, (hipStream_t)stream);
+    }
 }
 
 }  // extern "C"

@@ -10,8 +10,6 @@ constexpr int kWave = 64;          // CDNA wavefront
 constexpr int kRows = 8;           // rows per strip == row-checkpoint spacing
 constexpr int kCkX = 8;            // column-checkpoint spacing == tile width
 constexpr int kTile = kRows * kCkX;
-constexpr int kWPB = 4;            // waves per block
-constexpr int kThreads = kWave * kWPB;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -41,14 +39,22 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
     return (uint16_t)(u >> 16);
 }
 
-// Element access with the dtype chosen at run time (wave-uniform branch): the tile staging is the
-// only code that touches caller tensors, everything after it is fp32.
-__device__ __forceinline__ float ld_f32(const void *base, int64_t i, int dt) {
+// Typed element access.  The tile staging is the only code that touches caller tensors; everything
+// after it is fp32.  Offsets inside one batch image are 32-bit (checked by the host entry points).
+__device__ __forceinline__ float ldg(const float *base, int i) { return base[i]; }
+__device__ __forceinline__ float ldg(const bf16_t *base, int i) { return bf16_to_f32(base[i].v); }
+__device__ __forceinline__ float ldg(const f16_t *base, int i) { return (float)base[i]; }
+__device__ __forceinline__ void stg(float *base, int i, float v) { base[i] = v; }
+__device__ __forceinline__ void stg(bf16_t *base, int i, float v) { base[i].v = f32_to_bf16(v); }
+__device__ __forceinline__ void stg(f16_t *base, int i, float v) { base[i] = (f16_t)v; }
+// Same with the dtype chosen at run time (wave-uniform branch): used for out / dout, whose dtype
+// may differ from the inputs' (fp32 or the input dtype).
+__device__ __forceinline__ float ld_f32(const void *base, int i, int dt) {
     if (dt == SND_F32) return ((const float *)base)[i];
     if (dt == SND_BF16) return bf16_to_f32(((const uint16_t *)base)[i]);
     return (float)((const f16_t *)base)[i];
 }
-__device__ __forceinline__ void st_f32(void *base, int64_t i, int dt, float v) {
+__device__ __forceinline__ void st_f32(void *base, int i, int dt, float v) {
     if (dt == SND_F32) ((float *)base)[i] = v;
     else if (dt == SND_BF16) ((uint16_t *)base)[i] = f32_to_bf16(v);
     else ((f16_t *)base)[i] = (f16_t)v;
@@ -95,17 +101,5 @@ __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &p
 }
 __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8) * 8 * nChunks; }
 
-// ---------------------------------------------------------------- shared tile staging
-// Thread <-> element maps used by both kernels (NP lanes per channel, kThreads threads):
-//   state tiles (B, C, dB, dC): element k of thread t is state (t/64 + kWPB*k), pixel t%64
-//   pixel tiles (delta', u, ...): thread t belongs to channel t/NP (the channel its lane computes)
-//                                 and owns pixels (t%NP) + NP*k, k < 64/NP
-template <int NP> struct Map {
-    static constexpr int CPW = kWave / NP;          // channels per wave
-    static constexpr int CB = CPW * kWPB;           // channels per block
-    static constexpr int NBC = NP * kTile / kThreads;   // B/C elements per thread per tile
-    static constexpr int NPX = kTile / NP;          // pixels per thread per tile
-    static constexpr int NSTR = kTile + 4;          // per-state LDS pitch: lane n hits banks 4n..4n+3
-};
 
 }  // namespace snd

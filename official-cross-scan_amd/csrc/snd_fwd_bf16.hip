@@ -1,0 +1,5 @@
+// Forward kernel instantiation for bf16 inputs.
+#include "snd_fwd_kernel.h"
+namespace snd {
+int launch_fwd_bf16(const snd_fwd_params &p, hipStream_t stream) { return launch_fwd_t<bf16_t>(p, stream); }
+}  // namespace snd

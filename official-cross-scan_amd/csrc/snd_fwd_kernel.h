@@ -21,12 +21,13 @@
 //   * the sum over states is a DPP reduction inside aligned lane groups;
 //   * h at strip bottoms (x_v) doubles as the carry to the next strip and as the backward's row
 //     checkpoint; h and s at tile right edges (x, x_sd) are the backward's column checkpoints.
+#pragma once
 #include "snd_device.h"
 
 namespace snd {
 
-template <int NP, bool SAVE>
-__global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
+template <typename T, int NP, bool SAVE>
+__global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;                 // per-state pitch: lane n hits banks 4n..4n+3
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
     __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s + bu/4)
 
     const snd_shape &sh = p.shape;
-    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups, dt = sh.in_dtype;
+    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
@@ -63,19 +64,25 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
     const float bias = p.delta_bias ? p.delta_bias[cc / rd] : 0.f;
     const bool softplus = p.delta_softplus != 0;
 
-    const int64_t offB = (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
-    const int64_t offC = (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
-    const int64_t offU = (int64_t)b * p.u_batch_stride + (int64_t)cc * p.u_d_stride;
-    const int64_t offD = (int64_t)b * p.delta_batch_stride + (int64_t)(cc / rd) * p.delta_d_stride;
-    const int64_t offO = (int64_t)b * p.out_batch_stride + (int64_t)cc * p.out_d_stride;
+    // per-batch-image base pointers (uniform) and 32-bit offsets inside the image
+    const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
+    const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
+    const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride;
+    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride;
+    const int esz_out = p.out_dtype == SND_F32 ? 4 : 2;
+    void *outb = (char *)p.out + (int64_t)b * p.out_batch_stride * esz_out;
+    const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride, cO = cc * (int)p.out_d_stride;
+    const int Bh = (int)p.B_h_stride, Ch = (int)p.C_h_stride, Uh = (int)p.u_h_stride, Dh = (int)p.delta_h_stride;
+    const int Bs = (int)p.B_dstate_stride, Cs = (int)p.C_dstate_stride, Oh = (int)p.out_h_stride;
 
-    // saved state, (channel, state) innermost so that a wave's 64 planes touch one contiguous run:
-    //   x_v  [b][strip I][col][c][n]      x, x_sd  [b][col tile J][row][c][n]
-    const int64_t DN = (int64_t)Dm * N;
-    const int64_t lane_off = (int64_t)cc * N + nn;
-    float *xv = p.x_v + (int64_t)b * geo.nCY * geo.Wp * DN + lane_off;
-    float *xh = SAVE ? p.x + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off : nullptr;
-    float *xs = SAVE ? p.x_sd + (int64_t)b * geo.nCX * geo.Hp * DN + lane_off : nullptr;
+    // saved state, tile-major with the lane's 8 values innermost, so that each lane moves 32
+    // contiguous bytes and a wave's 64 planes one contiguous 2 KB run:
+    //   x_v  [b][strip I][col tile J][c][n][8 cols]     x, x_sd  [b][J][I][c][n][8 rows]
+    const int64_t DN8 = (int64_t)Dm * N * 8;
+    const int64_t lane_off = ((int64_t)cc * N + nn) * 8;
+    float *xv = p.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
+    float *xh = SAVE ? p.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off : nullptr;
+    float *xs = SAVE ? p.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off : nullptr;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
@@ -88,20 +95,24 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
     auto prefetch = [&](int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
         if (I > 0 && geo.nCX > 1) {                 // with one column tile the row comes from registers
-            const float *src = xv + ((int64_t)(I - 1) * geo.Wp + j0) * DN;
-#pragma unroll
-            for (int j = 0; j < kCkX; ++j) qxv[j] = src[j * DN];
-            qcorner = J > 0 ? src[-DN] : 0.f;
+            const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+            const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+            qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
+            qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
+            qcorner = J > 0 ? src[7 - DN8] : 0.f;
         }
+        // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
+            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int ob = rc * Bh + cx, oc = rc * Ch + cx;
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
-                const int sn = wave + WPB * k;
-                const bool ok = in && sn < N;
-                qb[k] = ok ? ld_f32(p.B, offB + (int64_t)sn * p.B_dstate_stride + (int64_t)row * p.B_h_stride + col, dt) : 0.f;
-                qc[k] = ok ? ld_f32(p.C, offC + (int64_t)sn * p.C_dstate_stride + (int64_t)row * p.C_h_stride + col, dt) : 0.f;
+                const int sn = wave + WPB * k, sc = min(sn, N - 1);
+                const float vb = ldg(Bb, sc * Bs + ob), vc = ldg(Cb, sc * Cs + oc);
+                qb[k] = (in && sn < N) ? vb : 0.f;
+                qc[k] = (in && sn < N) ? vc : 0.f;
             }
         }
 #pragma unroll
@@ -109,12 +120,15 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            qdl[k] = ok ? ld_f32(p.delta, offD + (int64_t)row * p.delta_h_stride + col, dt) : 0.f;
-            qu[k] = ok ? ld_f32(p.u, offU + (int64_t)row * p.u_h_stride + col, dt) : 0.f;
+            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
+            qdl[k] = ok ? vd : 0.f;
+            qu[k] = ok ? vu : 0.f;
         }
         if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
             const int row = r0 - 1, col = j0 + n;
-            qhalo = (cvalid && row >= 0 && col < W) ? ld_f32(p.delta, offD + (int64_t)row * p.delta_h_stride + col, dt) : 0.f;
+            const float vd = ldg(db, cD + max(row, 0) * Dh + min(col, W - 1));
+            qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
         }
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
@@ -213,14 +227,16 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
             }
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
-                float *dst = xv + ((int64_t)I * geo.Wp + j0) * DN;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) dst[j * DN] = hup[j];
+                float4 *dst = (float4 *)(xv + ((int64_t)I * geo.nCX + J) * DN8);
+                dst[0] = make_float4(hup[0], hup[1], hup[2], hup[3]);
+                dst[1] = make_float4(hup[4], hup[5], hup[6], hup[7]);
                 if (SAVE && J + 1 < geo.nCX) {      // column checkpoints: only if a tile follows
-                    float *dh = xh + ((int64_t)J * geo.Hp + r0) * DN;
-                    float *ds = xs + ((int64_t)J * geo.Hp + r0) * DN;
-#pragma unroll
-                    for (int r = 0; r < kRows; ++r) { dh[r * DN] = hl[r]; ds[r * DN] = sl[r]; }
+                    float4 *dh = (float4 *)(xh + ((int64_t)J * geo.nCY + I) * DN8);
+                    float4 *ds = (float4 *)(xs + ((int64_t)J * geo.nCY + I) * DN8);
+                    dh[0] = make_float4(hl[0], hl[1], hl[2], hl[3]);
+                    dh[1] = make_float4(hl[4], hl[5], hl[6], hl[7]);
+                    ds[0] = make_float4(sl[0], sl[1], sl[2], sl[3]);
+                    ds[1] = make_float4(sl[4], sl[5], sl[6], sl[7]);
                 }
             }
             __syncthreads();
@@ -231,7 +247,7 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                 if (cvalid && row < H && col < W)
-                    st_f32(p.out, offO + (int64_t)row * p.out_h_stride + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                    st_f32(outb, cO + row * Oh + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
@@ -239,7 +255,7 @@ __global__ __launch_bounds__(16 * NP) void fwd_kernel(const snd_fwd_params p, co
     }
 }
 
-template <int NP>
+template <typename T, int NP>
 static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const Geo geo = make_geo(sh.nrows, sh.ncols);
@@ -247,14 +263,16 @@ static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
     const int nChunks = (rg + 15) / 16;
     const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
     if (p.x != nullptr)
-        hipLaunchKernelGGL((fwd_kernel<NP, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+        hipLaunchKernelGGL((fwd_kernel<T, NP, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     else
-        hipLaunchKernelGGL((fwd_kernel<NP, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+        hipLaunchKernelGGL((fwd_kernel<T, NP, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
-int launch_fwd(const snd_fwd_params &p, hipStream_t stream) {
-    return p.shape.dstate > 8 ? launch_fwd_np<16>(p, stream) : launch_fwd_np<8>(p, stream);
+// One instantiation per input dtype, each in its own translation unit.
+template <typename T>
+int launch_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
+    return p.shape.dstate > 8 ? launch_fwd_np<T, 16>(p, stream) : launch_fwd_np<T, 8>(p, stream);
 }
 
 }  // namespace snd
