@@ -39,6 +39,7 @@ def run(cmd):
 
 def build_capi(extra=()):
     os.makedirs(OBJ, exist_ok=True)
+    extra = list(extra) + os.environ.get("SND_EXTRA_FLAGS", "").split()
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
     def one(src):

@@ -25,6 +25,7 @@
 // As in the forward, tiles are computed in full on zero-padded staging (dout = B = C = 0 outside
 // the plane makes every adjoint there exactly zero), so the inner loops have no bounds checks.
 #pragma once
+#include <type_traits>
 #include "snd_device.h"
 
 namespace snd {
@@ -68,8 +69,16 @@ __device__ __forceinline__ void acc_put(float &slot, float v) { slot = v; }
 __device__ __forceinline__ float acc_get(const float &slot) { return slot; }
 #endif
 
+#ifndef SND_BWD_WAVES
+#define SND_BWD_WAVES 2
+#endif
+#ifdef SND_X_NOBAR
+#define SND_SYNC() __builtin_amdgcn_wave_barrier()
+#else
+#define SND_SYNC() __syncthreads()
+#endif
 template <typename T, int NP>
-__global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
+__global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD_WAVES, SND_BWD_WAVES))) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;
@@ -132,7 +141,6 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;            // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
     const int cU = cc * (int)f.u_d_stride, cD = (cc / rd) * (int)f.delta_d_stride, cDo = cc * (int)p.dout_d_stride;
-    const int cG = cc * H * W;
     const int Bh = (int)f.B_h_stride, Ch = (int)f.C_h_stride, Uh = (int)f.u_h_stride, Dh = (int)f.delta_h_stride;
     const int Bs = (int)f.B_dstate_stride, Cs = (int)f.C_dstate_stride, Doh = (int)p.dout_h_stride;
 
@@ -160,7 +168,19 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     // ---- register staging of one tile's raw inputs (global loads issued one tile ahead)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
+#ifdef SND_X_NOLOAD
+        for (int k = 0; k < NBC; ++k) { qb[k] = 0.1f; qc[k] = 0.2f; }
+        for (int k = 0; k < NPX; ++k) { qdl[k] = 0.01f; qu[k] = 0.3f; qdo[k] = 0.4f; }
+        for (int k = 0; k < NHK; ++k) qh[k] = 0.01f;
+        (void)I; (void)J;
+        return;
+#endif
         const int r0 = I * kRows, j0 = J * kCkX;
+        // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
+        // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
+        SND_THREAD_MAPS(NP);
+        const int cU = cc * (int)f.u_d_stride, cD = (cc / rd) * (int)f.delta_d_stride;
+        const int cDo = cc * (int)p.dout_d_stride;
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
@@ -202,6 +222,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
         }
     };
     auto commit = [&]() {
+        SND_THREAD_MAPS(NP);
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
             const int sn = wave + WPB * k;
@@ -239,7 +260,9 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
     float dA_acc = 0.f, dec_acc = 0.f;              // per lane: sum delta'*da*a, sum da*a
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
 
+#ifdef SND_BWD_PREFETCH
     prefetch(geo.nCY - 1, geo.nCX - 1);
+#endif
     for (int I = geo.nCY - 1; I >= 0; --I) {
         const int r0 = I * kRows;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
@@ -249,76 +272,50 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
 
         for (int J = geo.nCX - 1; J >= 0; --J) {
             const int j0 = J * kCkX;
+#ifndef SND_BWD_PREFETCH
+            prefetch(I, J);                         // no loads in flight across the register-hungry sweep
+#endif
             commit();
-            __syncthreads();
-            {
-                int In = I, Jn = J - 1;
-                if (Jn < 0) { Jn = geo.nCX - 1; In = I - 1; }
-                if (In >= 0) prefetch(In, Jn);
-            }
+            SND_SYNC();
 
             // ---- checkpoints and carried adjoints of this tile
-            // h on the tile and its upper/left halo lives in 81 accumulation registers (AGPRs):
-            // HA(r, j), r, j in -1..7.  Rows are moved to VGPRs only while they are being used.
-            float hA[kRows + 1][kCkX + 1];
-#define HA(r, j) hA[(r) + 1][(j) + 1]
-            float slft[kRows];
-            float Gd[kCkX];
-            {
-                float hu[kCkX], hlft[kRows], hc = 0.f;
-                if (I > 0) {
-                    const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
-                    const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
-                    hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
-                    hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
-                    if (J > 0) hc = src[7 - DN8];
-                } else {
+            float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
+            float Gd[kCkX];                                        // G of the row below
+#ifdef SND_X_NOCKPT
+            if (false) {
+#else
+            if (I > 0) {
+#endif
+                const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+                const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
+                hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
+                if (J > 0) hc = src[7 - DN8];
+            } else {
 #pragma unroll
-                    for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
-                }
-                if (J > 0) {
-                    const float4 *sh_ = (const float4 *)(xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
-                    const float4 *ss_ = (const float4 *)(xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
-                    const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
-                    hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
-                    hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
-                    slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
-                    slft[4] = s1.x; slft[5] = s1.y; slft[6] = s1.z; slft[7] = s1.w;
-                } else {
-#pragma unroll
-                    for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
-                }
-                acc_put(HA(-1, -1), hc);
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) acc_put(HA(-1, j), hu[j]);
-#pragma unroll
-                for (int r = 0; r < kRows; ++r) acc_put(HA(r, -1), hlft[r]);
-
-                // ---- recompute h on the tile (row r-1 stays in VGPRs as the "up" row)
-                float aprev[kCkX], hprev[kCkX];
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) { aprev[j] = AEXP(-1, j); hprev[j] = hu[j]; }
-                float diag0 = hc;                   // h[r-1][-1]
-#pragma unroll
-                for (int r = 0; r < kRows; ++r) {
-                    float al = AEXP(r, -1);
-                    float left = hlft[r];
-                    float diag = diag0;
-                    diag0 = hlft[r];
-#pragma unroll
-                    for (int j = 0; j < kCkX; ++j) {
-                        const float a = AEXP(r, j);
-                        const float bu = myB[r * kCkX + j] * myDu[r * kCkX + j];
-                        const float up = hprev[j];
-                        const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
-                        const float h = fmaf(a, left + X, bu);
-                        acc_put(HA(r, j), h);
-                        hprev[j] = h;
-                        diag = up; left = h; al = a; aprev[j] = a;
-                    }
-                }
+                for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
+#ifdef SND_X_NOCKPT
+            if (false) {
+#else
+            if (J > 0) {
+#endif
+                const float4 *sh_ = (const float4 *)(xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
+                const float4 *ss_ = (const float4 *)(xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
+                const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
+                hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
+                hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
+                slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
+                slft[4] = s1.x; slft[5] = s1.y; slft[6] = s1.z; slft[7] = s1.w;
+            } else {
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
+            }
+#ifdef SND_X_NOCKPT
+            if (false) {
+#else
             if (I + 1 < geo.nCY && lvalid) {
+#endif
                 const float4 *src = (const float4 *)(gdown + (int64_t)J * DN8);
                 const float4 v0 = src[0], v1 = src[1];
                 Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
@@ -328,100 +325,175 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                 for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
             }
             const float gd_old0 = Gd[0];            // G[r0+8][j0]: the corner of the tile on the left
-            float Gd8 = GRc;
 
-            // ---- reverse sweep
-            float adn[kCkX];
-            float hcur[kCkX + 1], hupr[kCkX];       // h rows r (with left halo) and r-1, in VGPRs
+            // The tile is swept as two 8x4 halves, right then left, so that only 32 values of h
+            // are held at a time.  The right half starts from h, s at column 3, which a plain
+            // forward pass over the left half provides first (that half is recomputed when it is
+            // swept: 32 extra cell updates per tile buy about 60 registers).
+            float hmid[kRows], smid[kRows];
+            {
+                float aprev[4], hprev[4];
 #pragma unroll
-            for (int j = 0; j < kCkX; ++j) adn[j] = AEXP(kRows, j);
+                for (int j = 0; j < 4; ++j) { aprev[j] = AEXP(-1, j); hprev[j] = hu[j]; }
+                float diag0 = hc;
 #pragma unroll
-            for (int j = -1; j < kCkX; ++j) hcur[j + 1] = acc_get(HA(kRows - 1, j));
+                for (int r = 0; r < kRows; ++r) {
+                    float al = AEXP(r, -1), left = hlft[r], sl = slft[r], diag = diag0;
+                    diag0 = hlft[r];
 #pragma unroll
-            for (int r = kRows - 1; r >= 0; --r) {
-                __builtin_amdgcn_sched_barrier(0);
-                float arow[kCkX + 1], s[kCkX];
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) hupr[j] = acc_get(HA(r - 1, j));
-#pragma unroll
-                for (int j = 0; j <= kCkX; ++j) arow[j] = AEXP(r, j);
-                {
-                    float sp = slft[r];
-#pragma unroll
-                    for (int j = 0; j < kCkX; ++j) {
-                        sp = fmaf(arow[j], sp, myB[r * kCkX + j] * myDu[r * kCkX + j]);
-                        s[j] = sp;
+                    for (int j = 0; j < 4; ++j) {
+                        const float a = AEXP(r, j);
+                        const float bu = myB[r * kCkX + j] * myDu[r * kCkX + j];
+                        const float up = hprev[j];
+                        const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
+                        const float h = fmaf(a, left + X, bu);
+                        sl = fmaf(a, sl, bu);
+                        hprev[j] = h;
+                        diag = up; left = h; al = a; aprev[j] = a;
                     }
+                    hmid[r] = left; smid[r] = sl;
                 }
-                float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
-                float q[4], pp_[4], vB[4], vC[4], tB[4], tC[4];
-#pragma unroll
-                for (int j = kCkX - 1; j >= 0; --j) {
-                    const float dov = myDo[r * kCkX + j];
-                    const float Bv = myB[r * kCkX + j], Cv = myC[r * kCkX + j];
-                    const float duv = myDu[r * kCkX + j];
-                    const float bu = Bv * duv;
-                    const float dyC = dov * Cv;
-                    const float a = arow[j];
-                    const float g_ = fmaf(-0.5f * (arow[j + 1] + adn[j]), Gdiag, dyC + Gr + Gd[j]);
-                    const float gs = Gsr - dyC;
-                    const float dbu = fmaf(0.25f, dyC, g_ + gs);
-                    const float hb = hcur[j + 1] - bu, sb = s[j] - bu;
-                    const float cross = fmaf(Gd[j], hcur[j], Gr * hupr[j]);
-                    const float da = fmaf(-0.5f * a, cross, fmaf(g_, hb, gs * sb));
-                    dA_acc = fmaf(DL(r, j), da, dA_acc);
-                    dec_acc += da;
-                    const float Gn = a * g_;
-                    Gdiag = Gd[j];
-                    Gd[j] = Gn;
-                    Gr = Gn;
-                    Gsr = a * gs;
-                    // per-pixel sums over states, flushed per half row
-                    q[j & 3] = group_sum<NP>(dbu * Bv);
-                    pp_[j & 3] = group_sum<NP>(Av * da);
-                    if ((j & 3) == 0 && n == 0) {
-                        *(float4 *)(sQ + cl * kTile + r * kCkX + j) = make_float4(q[0], q[1], q[2], q[3]);
-                        *(float4 *)(sP + cl * kTile + r * kCkX + j) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
-                    }
-                    // dB, dC contributions: summed over the wave's channels pair by pair (j, j+4)
-                    const float vb = dbu * duv, vc = dov * fmaf(0.25f, bu, hb - sb);
-                    if (NP == 16) {
-                        if (j >= 4) { vB[j - 4] = vb; vC[j - 4] = vc; }
-                        else {
-                            float a0 = vb, a1 = vB[j]; swap32(a0, a1); tB[j] = a0 + a1;
-                            float c0 = vc, c1 = vC[j]; swap32(c0, c1); tC[j] = c0 + c1;
-                        }
-                    } else {
-                        lds_add(mydB + r * kCkX + j, vb);
-                        lds_add(mydC + r * kCkX + j, vc);
-                    }
-                }
-                if (NP == 16) {
-                    float b0, b1, c0, c1;
-                    { float x0 = tB[0], x1 = tB[2]; swap16(x0, x1); b0 = x0 + x1; }
-                    { float x0 = tB[1], x1 = tB[3]; swap16(x0, x1); b1 = x0 + x1; }
-                    { float x0 = tC[0], x1 = tC[2]; swap16(x0, x1); c0 = x0 + x1; }
-                    { float x0 = tC[1], x1 = tC[3]; swap16(x0, x1); c1 = x0 + x1; }
-                    *(float2 *)(mydB + r * kCkX + 2 * qrow) = make_float2(b0, b1);
-                    *(float2 *)(mydC + r * kCkX + 2 * qrow) = make_float2(c0, c1);
-                }
-                Gd8 = GR[r];                        // G[r][j0+8]: diagonal neighbour for the row above
-                GR[r] = Gr;                         // G[r][j0]: right neighbour for the tile on the left
-                GsR[r] = Gsr;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) { adn[j] = arow[j]; hcur[j + 1] = hupr[j]; }
-                hcur[0] = acc_get(HA(r - 1, -1));
             }
-#undef HA
+
+            // One half: recompute h on rows 0..7, columns C0..C0+3, then sweep it bottom-right to
+            // top-left.  top/corner: h of the row above; hL/sL: h, s of the column to the left;
+            // GR/GsR (in/out): G, Gs of the column to the right, replaced by those of column C0;
+            // GdH (in/out): G of the row below, replaced by G of row 0; gdiag0: G[8][C0+4].
+            auto sweep_half = [&](auto C0_, const float *top, float corner, const float (&hL)[kRows],
+                                  const float (&sL)[kRows], float *GdH, float gdiag0) {
+                constexpr int C0 = decltype(C0_)::value;
+                float hT[kRows][4];
+                {
+                    float aprev[4], hprev[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { aprev[j] = AEXP(-1, C0 + j); hprev[j] = top[j]; }
+                    float diag0 = corner;
+#pragma unroll
+                    for (int r = 0; r < kRows; ++r) {
+                        float al = AEXP(r, C0 - 1), left = hL[r], diag = diag0;
+                        diag0 = hL[r];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float a = AEXP(r, C0 + j);
+                            const float bu = myB[r * kCkX + C0 + j] * myDu[r * kCkX + C0 + j];
+                            const float up = hprev[j];
+                            const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
+                            const float h = fmaf(a, left + X, bu);
+                            hT[r][j] = h;
+                            hprev[j] = h;
+                            diag = up; left = h; al = a; aprev[j] = a;
+                        }
+                    }
+                }
+#ifndef SND_X_NOREV
+                float adn[4];
+                float Gd8 = gdiag0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) adn[j] = AEXP(kRows, C0 + j);
+#pragma unroll
+                for (int r = kRows - 1; r >= 0; --r) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    float arow[5], s[4];
+#pragma unroll
+                    for (int j = 0; j <= 4; ++j) arow[j] = AEXP(r, C0 + j);
+                    {
+                        float sp = sL[r];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            sp = fmaf(arow[j], sp, myB[r * kCkX + C0 + j] * myDu[r * kCkX + C0 + j]);
+                            s[j] = sp;
+                        }
+                    }
+                    float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
+                    float q[4], pp_[4], vB[4], vC[4];
+#pragma unroll
+                    for (int j = 3; j >= 0; --j) {
+                        const int o = r * kCkX + C0 + j;
+                        const float dov = myDo[o];
+                        const float Bv = myB[o], Cv = myC[o];
+                        const float duv = myDu[o];
+                        const float bu = Bv * duv;
+                        const float dyC = dov * Cv;
+                        const float a = arow[j];
+                        const float g_ = fmaf(-0.5f * (arow[j + 1] + adn[j]), Gdiag, dyC + Gr + GdH[j]);
+                        const float gs = Gsr - dyC;
+                        const float dbu = fmaf(0.25f, dyC, g_ + gs);
+                        const float h_l = (j == 0) ? hL[r] : hT[r][j - 1 < 0 ? 0 : j - 1];
+                        const float h_u = (r == 0) ? top[j] : hT[r - 1 < 0 ? 0 : r - 1][j];
+                        const float hb = hT[r][j] - bu, sb = s[j] - bu;
+                        const float cross = fmaf(GdH[j], h_l, Gr * h_u);
+                        const float da = fmaf(-0.5f * a, cross, fmaf(g_, hb, gs * sb));
+                        dA_acc = fmaf(DL(r, C0 + j), da, dA_acc);
+                        dec_acc += da;
+                        const float Gn = a * g_;
+                        Gdiag = GdH[j];
+                        GdH[j] = Gn;
+                        Gr = Gn;
+                        Gsr = a * gs;
+                        q[j] = group_sum<NP>(dbu * Bv);            // per-pixel sums over states
+                        pp_[j] = group_sum<NP>(Av * da);
+                        vB[j] = dbu * duv;                         // dB, dC contributions
+                        vC[j] = dov * fmaf(0.25f, bu, hb - sb);
+                    }
+                    if (n == 0) {
+                        *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
+                        *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
+                    }
+                    if (NP == 16) {
+                        // sum over the wave's 4 channels (its 16-lane rows): row q ends with column C0+q
+                        float b0 = vB[0], b2 = vB[2], b1 = vB[1], b3 = vB[3];
+                        swap32(b0, b2); swap32(b1, b3);
+                        float tb0 = b0 + b2, tb1 = b1 + b3;
+                        swap16(tb0, tb1);
+                        float c0 = vC[0], c2 = vC[2], c1 = vC[1], c3 = vC[3];
+                        swap32(c0, c2); swap32(c1, c3);
+                        float tc0 = c0 + c2, tc1 = c1 + c3;
+                        swap16(tc0, tc1);
+                        mydB[r * kCkX + C0 + qrow] = tb0 + tb1;
+                        mydC[r * kCkX + C0 + qrow] = tc0 + tc1;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            lds_add(mydB + r * kCkX + C0 + j, vB[j]);
+                            lds_add(mydC + r * kCkX + C0 + j, vC[j]);
+                        }
+                    }
+                    Gd8 = GR[r];                    // G[r][C0+4]: diagonal neighbour for the row above
+                    GR[r] = Gr;                     // G[r][C0]: right neighbour for the half on the left
+                    GsR[r] = Gsr;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) adn[j] = arow[j];
+                }
+#endif
+            };
+            const float gd_old4 = Gd[4];            // G[r0+8][j0+4]: corner of the left half
+            sweep_half(std::integral_constant<int, 4>{}, hu + 4, hu[3], hmid, smid, Gd + 4, GRc);
+            sweep_half(std::integral_constant<int, 0>{}, hu, hc, hlft, slft, Gd, gd_old4);
             GRc = gd_old0;
+#ifdef SND_X_NOCKPT
+            if (false) {
+#else
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
+#endif
                 float4 *dst = (float4 *)(gdown + (int64_t)J * DN8);
                 dst[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
                 dst[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
             }
-            __syncthreads();
+            SND_SYNC();
+#ifdef SND_BWD_PREFETCH
+            {   // the next tile's loads are issued here, after the register-hungry sweep, and complete
+                // under the per-pixel epilogue below and under the other resident block's compute
+                int In = I, Jn = J - 1;
+                if (Jn < 0) { Jn = geo.nCX - 1; In = I - 1; }
+                if (In >= 0) prefetch(In, Jn);
+            }
+#endif
 
+#ifndef SND_X_NOEPI
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
+            {
+            SND_THREAD_MAPS(NP);
+            const int cG = cc * H * W;
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
@@ -438,8 +510,10 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                     stg(ddb, cG + row * W + col, ddl);
                 }
             }
+            }
             // ---- dB, dC of this tile leave the block (summed over its channels)
             {
+                SND_THREAD_MAPS(NP);
                 const int row = r0 + pr, col = j0 + pj;
                 const bool in = row < H && col < W;
 #pragma unroll
@@ -459,6 +533,7 @@ __global__ __launch_bounds__(16 * NP) void bwd_kernel(const snd_bwd_params p, co
                     if (NP != 16) { sdB[sn * NSTR + px] = 0.f; sdC[sn * NSTR + px] = 0.f; }
                 }
             }
+#endif
         }
     }
 #undef DL

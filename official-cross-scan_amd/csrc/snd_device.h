@@ -101,5 +101,18 @@ __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &p
 }
 __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8) * 8 * nChunks; }
 
+// Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging
+// section so that the compiler recomputes a few integer ops per tile instead of hoisting dozens of
+// loop-invariant addresses out of the tile loop and keeping (or spilling) them across it.
+// Expects `tid`, `cbase`, `cend` in scope; defines wave, px, pr, pj, n, cl, cvalid, cc.
+#define SND_THREAD_MAPS(NP)                                                        \
+    int t_ = tid;                                                                  \
+    asm volatile("" : "+v"(t_));                                                   \
+    const int wave = t_ >> 6, px = t_ & 63, pr = px >> 3, pj = px & 7;             \
+    const int n = t_ % (NP), cl = t_ / (NP);                                       \
+    const int c_ = cbase + cl;                                                     \
+    const bool cvalid = c_ < cend;                                                 \
+    const int cc = cvalid ? c_ : cend - 1;                                         \
+    (void)wave; (void)pr; (void)pj; (void)n; (void)cc
 
 }  // namespace snd

@@ -71,7 +71,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride;
     const int esz_out = p.out_dtype == SND_F32 ? 4 : 2;
     void *outb = (char *)p.out + (int64_t)b * p.out_batch_stride * esz_out;
-    const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride, cO = cc * (int)p.out_d_stride;
+    const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
     const int Bh = (int)p.B_h_stride, Ch = (int)p.C_h_stride, Uh = (int)p.u_h_stride, Dh = (int)p.delta_h_stride;
     const int Bs = (int)p.B_dstate_stride, Cs = (int)p.C_dstate_stride, Oh = (int)p.out_h_stride;
 
@@ -94,6 +94,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto prefetch = [&](int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
+        // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
+        // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
+        SND_THREAD_MAPS(NP);
+        const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
         if (I > 0 && geo.nCX > 1) {                 // with one column tile the row comes from registers
             const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
             const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
@@ -133,6 +137,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&]() {
+        SND_THREAD_MAPS(NP);
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
             const int sn = wave + WPB * k;
@@ -242,6 +247,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             __syncthreads();
 
             // ---- out = D*u + y, written by the thread that staged the pixel
+            SND_THREAD_MAPS(NP);
+            const int cO = cc * (int)p.out_d_stride;
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
