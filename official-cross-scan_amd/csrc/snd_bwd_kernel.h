@@ -430,11 +430,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         GdH[j] = Gn;
                         Gr = Gn;
                         Gsr = a * gs;
-                        q[j] = group_sum<NP>(dbu * Bv);            // per-pixel sums over states
-                        pp_[j] = group_sum<NP>(Av * da);
+                        q[j] = dbu * Bv;                           // per-pixel terms, summed over states below
+                        pp_[j] = Av * da;
                         vB[j] = dbu * duv;                         // dB, dC contributions
                         vC[j] = dov * fmaf(0.25f, bu, hb - sb);
                     }
+                    group_sum4<NP>(q[0], q[1], q[2], q[3]);
+                    group_sum4<NP>(pp_[0], pp_[1], pp_[2], pp_[3]);
                     if (n == 0) {
                         *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
                         *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);

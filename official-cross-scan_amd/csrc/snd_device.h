@@ -91,6 +91,25 @@ template <int NP> __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// The same sum for four independent values at once, written out as fused v_add_f32_dpp steps.
+// Interleaving the four values puts three instructions between a step and the next step of the
+// same value, which covers the VALU-write -> DPP-read hazard; the leading s_nop covers the first.
+#define SND_DPP4(ctrl)                                                   \
+    "v_add_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+    "v_add_f32_dpp %1, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+    "v_add_f32_dpp %2, %2, %2 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t" \
+    "v_add_f32_dpp %3, %3, %3 " ctrl " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+template <int NP> __device__ __forceinline__ void group_sum4(float &a, float &b, float &c, float &d) {
+    if (NP == 16)
+        asm("s_nop 1\n\t" SND_DPP4("quad_perm:[1,0,3,2]") SND_DPP4("quad_perm:[2,3,0,1]") SND_DPP4("row_half_mirror")
+                SND_DPP4("row_mirror")
+            : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    else if (NP == 8)
+        asm("s_nop 1\n\t" SND_DPP4("quad_perm:[1,0,3,2]") SND_DPP4("quad_perm:[2,3,0,1]") SND_DPP4("row_half_mirror")
+            : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    else { a = group_sum<NP>(a); b = group_sum<NP>(b); c = group_sum<NP>(c); d = group_sum<NP>(d); }
+}
+
 // Blocks are dealt round-robin to the 8 XCDs (each with its own L2).  Keep every chunk of one
 // (batch, group) pair - they all stream the same B/C planes - on one XCD.
 __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &pair, int &chunk) {

@@ -217,8 +217,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     }
                 }
                 hl[r] = left; sl[r] = sleft; al[r] = aleft;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) y[j] = group_sum<NP>(y[j]);
+                group_sum4<NP>(y[0], y[1], y[2], y[3]);
+                group_sum4<NP>(y[4], y[5], y[6], y[7]);
                 if (n == 0) {
                     float4 *dst = (float4 *)(sY + cl * kTile + r * kCkX);
                     dst[0] = make_float4(y[0], y[1], y[2], y[3]);
