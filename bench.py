@@ -113,6 +113,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this operator is measured on ONE GPU (every (batch, channel, state) plane is an "
@@ -120,10 +123,18 @@ def main():
                  "Run with --gpus 1.")
 
     import torch
+    dev = torch.device("cuda:0")
+    if args.copy_probe:
+        x = torch.randn(64 * 1024 * 1024, device=dev)          # 256 MiB read + 256 MiB written per copy
+        y = torch.empty_like(x)
+        for _ in range(5):
+            y.copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes_each_way": x.numel() * 4}))
+        return
     import selective_nd_scan as snd
     from selective_nd_scan import capi
 
-    dev = torch.device("cuda:0")
     Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
     dtype = getattr(torch, dtn)
     u, delta, A, B, C, D, bias, dout = make_inputs(torch, Bt, Dm, H, W, N, K, dtype, dev)

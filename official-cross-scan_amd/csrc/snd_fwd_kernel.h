@@ -93,12 +93,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo = 0.f;
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto prefetch = [&](int I, int J) {
+#ifdef SND_XF_NOLOAD
+        for (int k = 0; k < NBC; ++k) { qb[k] = 0.1f; qc[k] = 0.2f; }
+        for (int k = 0; k < NPX; ++k) { qdl[k] = 0.01f; qu[k] = 0.3f; }
+        qhalo = 0.01f; (void)I; (void)J;
+        return;
+#endif
         const int r0 = I * kRows, j0 = J * kCkX;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
+#ifdef SND_XF_NOXVLD
+        if (false) {
+#else
         if (I > 0 && geo.nCX > 1) {                 // with one column tile the row comes from registers
+#endif
             const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
             const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
@@ -230,12 +240,20 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];
                 qcorner = 0.f;
             }
+#ifdef SND_XF_NOXVST
+            if (false) {
+#else
             if (lvalid) {
+#endif
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float4 *dst = (float4 *)(xv + ((int64_t)I * geo.nCX + J) * DN8);
                 dst[0] = make_float4(hup[0], hup[1], hup[2], hup[3]);
                 dst[1] = make_float4(hup[4], hup[5], hup[6], hup[7]);
+#ifdef SND_XF_NOCOL
+                if (false) {
+#else
                 if (SAVE && J + 1 < geo.nCX) {      // column checkpoints: only if a tile follows
+#endif
                     float4 *dh = (float4 *)(xh + ((int64_t)J * geo.nCY + I) * DN8);
                     float4 *ds = (float4 *)(xs + ((int64_t)J * geo.nCY + I) * DN8);
                     dh[0] = make_float4(hl[0], hl[1], hl[2], hl[3]);
@@ -253,7 +271,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
+#ifdef SND_XF_NOOUT
+                if (false)
+#else
                 if (cvalid && row < H && col < W)
+#endif
                     st_f32(outb, cO + row * Oh + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
