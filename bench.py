@@ -113,6 +113,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips"],
+                    help="block mapping: chosen by shape (default), one block per plane chunk, or pipelined row strips")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -135,6 +137,8 @@ def main():
     import selective_nd_scan as snd
     from selective_nd_scan import capi
 
+    sched = {"auto": 0, "plane": 1, "strips": 2}[args.schedule]
+    snd.set_schedule(sched)
     Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
     dtype = getattr(torch, dtn)
     u, delta, A, B, C, D, bias, dout = make_inputs(torch, Bt, Dm, H, W, N, K, dtype, dev)
@@ -154,9 +158,9 @@ def main():
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # kernel-only durations: HIP events on the launch stream around each launch through the C ABI
-    fcall = capi.FwdCall(u, delta, A, B, C, D, bias, True, True, None)
+    fcall = capi.FwdCall(u, delta, A, B, C, D, bias, True, True, None, True, sched)
     fcall.launch()
-    bcall = capi.BwdCall(u, delta, A, B, C, D, bias, dout, fcall.x, fcall.x_v, True, None, fcall.x_sd)
+    bcall = capi.BwdCall(u, delta, A, B, C, D, bias, dout, fcall.x, fcall.x_v, True, None, fcall.x_sd, sched)
     stream = torch.cuda.current_stream()
     kf, kb = [], []
     for i in range(args.warmup + args.steps):
@@ -178,7 +182,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: selective_nd_scan fwd+bwd, B=%d D=%d H=%d W=%d N=%d K=%d, %s inputs, fp32 state"
                                % (args.workload, Bt, Dm, H, W, N, K, dtn),
-                   "algorithmic_bytes": fb + bb, "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+                   "schedule": args.schedule, "algorithmic_bytes": fb + bb, "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
                    "pixels_per_s": round(Bt * Dm * H * W / (ms * 1e-3), 1),
                    "state_cells_per_s": round(Bt * Dm * H * W * N / (ms * 1e-3), 1),
                    "kernel_ms": {"fwd": round(kf_ms, 4), "bwd": round(kb_ms, 4)},

@@ -69,7 +69,16 @@ typedef struct snd_plan {
     int32_t x_inner, xv_inner;
     int64_t x_elems, x_sd_elems, x_v_elems;    /* fp32 element counts of the three tensors */
     int64_t bwd_workspace_bytes;               /* scratch bwd needs (16-byte aligned, uninitialised) */
+    int64_t fwd_workspace_bytes;               /* scratch fwd uses when it splits planes into strips
+                                                  (16-byte aligned, uninitialised; a few KB) */
 } snd_plan;
+
+/* How a launch maps work to blocks.  The reference has one fixed mapping (one block per
+ * (batch, channel), fwd.cuh:359-392); here the library picks by shape unless told otherwise:
+ *   PLANE   one block per (batch, group, 16-channel chunk) walks the whole plane;
+ *   STRIPS  one block per 8-row strip of such a chunk, the strips of a plane pipelined one tile
+ *           apart (for few, large planes: c3/c4-like shapes).  Needs the workspace. */
+typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2 } snd_schedule;
 
 /* Replaces SSMParamsBase (selective_scan_oflex.h:4-51); 64-bit strides instead of uint32. */
 typedef struct snd_fwd_params {
@@ -91,6 +100,11 @@ typedef struct snd_fwd_params {
     int64_t B_batch_stride, B_group_stride, B_dstate_stride, B_h_stride;
     int64_t C_batch_stride, C_group_stride, C_dstate_stride, C_h_stride;
     int64_t out_batch_stride, out_d_stride, out_h_stride;
+    void *workspace;               /* plan.fwd_workspace_bytes bytes, 16-byte aligned, or null (then the
+                                      PLANE schedule is used).  In snd_bwd_params.f it is ignored. */
+    int64_t workspace_bytes;
+    int32_t schedule;              /* snd_schedule, for fwd and (through snd_bwd_params.f) for bwd */
+    int32_t reserved_;             /* set to 0 */
 } snd_fwd_params;
 
 /* Replaces SSMParamsBwd (selective_scan_oflex.h:53-86). Gradient buffers are dense (contiguous):

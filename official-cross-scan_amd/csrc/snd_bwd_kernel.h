@@ -72,12 +72,7 @@ __device__ __forceinline__ float acc_get(const float &slot) { return slot; }
 #ifndef SND_BWD_WAVES
 #define SND_BWD_WAVES 2
 #endif
-#ifdef SND_X_NOBAR
-#define SND_SYNC() __builtin_amdgcn_wave_barrier()
-#else
-#define SND_SYNC() __syncthreads()
-#endif
-template <typename T, int NP>
+template <typename T, int NP, bool PIPE>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD_WAVES, SND_BWD_WAVES))) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
@@ -110,7 +105,32 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
-    if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
+    int I_hi = geo.nCY - 1, I_lo = 0;               // strips this block walks, bottom to top
+    int *sync = (int *)p.workspace, *progress = nullptr;
+    const int64_t nSync = sync_words((int64_t)sh.batch * G * nChunks, geo.nCY);
+    bool dead = false;
+#ifdef SND_PIPE_TRACE
+    int *trace_ = nullptr, trace_wait_ = 0;
+#endif
+    if (PIPE) {
+        __shared__ int sTicket;
+        if (threadIdx.x == 0) sTicket = __hip_atomic_fetch_add(sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        // tickets run strip-major from the bottom strip up (all plane chunks' last strip, then every
+        // strip above it, ...): a job's predecessor holds an earlier ticket, and a strip only takes a
+        // slot about when it can start
+        const int nPC = sh.batch * G * nChunks;
+        const int pc = sTicket % nPC;
+        if (sTicket / nPC >= geo.nCY) return;
+        I_hi = I_lo = geo.nCY - 1 - sTicket / nPC;
+        pair = pc / nChunks;
+        chunk = pc - pair * nChunks;
+        progress = sync + kSyncHeader + pc * geo.nCY;
+#ifdef SND_PIPE_TRACE
+        trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_hi);
+        if (threadIdx.x == 0) trace_[0] = (int)wall_clock64();
+#endif
+    } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
 
@@ -151,7 +171,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
     const float *xh = f.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
     const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
-    float *gdown = (float *)p.workspace + (int64_t)b * geo.nCX * DN8 + lane_off;
+    float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + lane_off;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
@@ -168,13 +188,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // ---- register staging of one tile's raw inputs (global loads issued one tile ahead)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
-#ifdef SND_X_NOLOAD
-        for (int k = 0; k < NBC; ++k) { qb[k] = 0.1f; qc[k] = 0.2f; }
-        for (int k = 0; k < NPX; ++k) { qdl[k] = 0.01f; qu[k] = 0.3f; qdo[k] = 0.4f; }
-        for (int k = 0; k < NHK; ++k) qh[k] = 0.01f;
-        (void)I; (void)J;
-        return;
-#endif
         const int r0 = I * kRows, j0 = J * kCkX;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
@@ -261,9 +274,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
 
 #ifdef SND_BWD_PREFETCH
-    prefetch(geo.nCY - 1, geo.nCX - 1);
+    prefetch(I_hi, geo.nCX - 1);
 #endif
-    for (int I = geo.nCY - 1; I >= 0; --I) {
+    for (int I = I_hi; I >= I_lo; --I) {
         const int r0 = I * kRows;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
         float GRc = 0.f;                            // G[r0+8][j0+8]
@@ -276,16 +289,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
 #endif
             commit();
-            SND_SYNC();
+            // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
+            // others wait at the barrier.
+            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, sync, dead SND_TRACE_PASS);
+            __syncthreads();
 
             // ---- checkpoints and carried adjoints of this tile
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
             float Gd[kCkX];                                        // G of the row below
-#ifdef SND_X_NOCKPT
-            if (false) {
-#else
             if (I > 0) {
-#endif
                 const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
                 const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
                 hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
@@ -295,11 +307,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
-#ifdef SND_X_NOCKPT
-            if (false) {
-#else
             if (J > 0) {
-#endif
                 const float4 *sh_ = (const float4 *)(xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
                 const float4 *ss_ = (const float4 *)(xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
                 const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
@@ -311,15 +319,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
             }
-#ifdef SND_X_NOCKPT
-            if (false) {
-#else
             if (I + 1 < geo.nCY && lvalid) {
-#endif
-                const float4 *src = (const float4 *)(gdown + (int64_t)J * DN8);
-                const float4 v0 = src[0], v1 = src[1];
-                Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
-                Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
+                const float *src = gdown + (int64_t)J * DN8;
+                if (PIPE) {
+#pragma unroll
+                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + k, Gd[k], Gd[k + 1]);
+                } else {
+                    const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                    Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
+                    Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
@@ -385,7 +394,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         }
                     }
                 }
-#ifndef SND_X_NOREV
                 float adn[4];
                 float Gd8 = gdiag0;
 #pragma unroll
@@ -466,32 +474,33 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                     for (int j = 0; j < 4; ++j) adn[j] = arow[j];
                 }
-#endif
             };
             const float gd_old4 = Gd[4];            // G[r0+8][j0+4]: corner of the left half
             sweep_half(std::integral_constant<int, 4>{}, hu + 4, hu[3], hmid, smid, Gd + 4, GRc);
             sweep_half(std::integral_constant<int, 0>{}, hu, hc, hlft, slft, Gd, gd_old4);
             GRc = gd_old0;
-#ifdef SND_X_NOCKPT
-            if (false) {
-#else
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
-#endif
-                float4 *dst = (float4 *)(gdown + (int64_t)J * DN8);
-                dst[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
-                dst[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
+                float *dst = gdown + (int64_t)J * DN8;
+                if (PIPE) {
+#pragma unroll
+                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + k, Gd[k], Gd[k + 1]);
+                } else {
+                    ((float4 *)dst)[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
+                    ((float4 *)dst)[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
+                }
             }
-            SND_SYNC();
+            if (PIPE && I > 0) strip_stores_done();
+            __syncthreads();
+            if (PIPE && I > 0) strip_signal(progress + I);   // tile J is handed over to the strip above
 #ifdef SND_BWD_PREFETCH
             {   // the next tile's loads are issued here, after the register-hungry sweep, and complete
                 // under the per-pixel epilogue below and under the other resident block's compute
                 int In = I, Jn = J - 1;
                 if (Jn < 0) { Jn = geo.nCX - 1; In = I - 1; }
-                if (In >= 0) prefetch(In, Jn);
+                if (In >= I_lo) prefetch(In, Jn);
             }
 #endif
 
-#ifndef SND_X_NOEPI
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
             {
             SND_THREAD_MAPS(NP);
@@ -535,12 +544,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     if (NP != 16) { sdB[sn * NSTR + px] = 0.f; sdC[sn * NSTR + px] = 0.f; }
                 }
             }
-#endif
         }
     }
 #undef DL
 #undef AEXP
 
+#ifdef SND_PIPE_TRACE
+    if (PIPE && threadIdx.x == 0) { trace_[1] = (int)wall_clock64(); trace_[2] = trace_wait_; }
+#endif
     // ---- per-lane / per-channel sums leave the kernel
     if (lvalid) glb_add(p.dA + (int64_t)c * N + n, dA_acc);
     dD_acc = group_sum<NP>(dD_acc);
@@ -570,16 +581,27 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     const Geo geo = make_geo(sh.nrows, sh.ncols);
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
-    const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
+    const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
     constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = (NP == 16) ? WPB : 1;
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void *)bwd_kernel<T, NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            return SND_ERR_LAUNCH;
-        configured = true;
+    const bool pipe = use_strip_pipeline(p.f.schedule, nPC, geo.nCY, p.workspace);
+    // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
+    static bool configured[2][64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SND_ERR_LAUNCH;
+    if (!configured[pipe][dev]) {
+        const void *fn = pipe ? (const void *)bwd_kernel<T, NP, true> : (const void *)bwd_kernel<T, NP, false>;
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return SND_ERR_LAUNCH;
+        configured[pipe][dev] = true;
     }
-    hipLaunchKernelGGL((bwd_kernel<T, NP>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
+    if (pipe) {
+        if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
+        if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
+        hipLaunchKernelGGL((bwd_kernel<T, NP, true>), dim3((int)(nPC * geo.nCY)), dim3(16 * NP), lds, stream, p, geo);
+    } else {
+        const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, false>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
+    }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 

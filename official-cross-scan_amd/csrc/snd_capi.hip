@@ -12,7 +12,22 @@ int launch_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
 }  // namespace snd
 
+namespace snd {
+__global__ void zero_words_kernel(int *p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+int zero_words(int *p, int64_t n, hipStream_t stream) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
+    return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+}  // namespace snd
+
 namespace {
+
+int64_t plane_chunks(const snd_shape &s) {
+    return (int64_t)s.batch * s.n_groups * ((s.dim / s.n_groups + 15) / 16);
+}
 
 int check_shape(const snd_shape &s) {
     if (s.batch <= 0 || s.dim <= 0 || s.nrows <= 0 || s.ncols <= 0 || s.dstate <= 0 || s.n_groups <= 0 ||
@@ -58,7 +73,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 100; }
+int snd_version(void) { return 101; }
 
 const char *snd_status_string(int status) {
     switch (status) {
@@ -87,8 +102,11 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->x_elems = planes * g.nCX * g.Hp;
     plan->x_sd_elems = plan->x_elems;
     plan->x_v_elems = planes * g.nCY * g.Wp;
-    // backward scratch: one row of G = a*g per plane (the adjoint carried from the strip below)
-    plan->bwd_workspace_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);
+    // strip-pipeline sync words, then (backward only) one row of G = a*g per plane: the adjoint
+    // carried from the strip below
+    const int64_t sync_bytes = snd::sync_words(plane_chunks(*shape), g.nCY) * (int64_t)sizeof(int);
+    plan->fwd_workspace_bytes = sync_bytes;
+    plan->bwd_workspace_bytes = sync_bytes + planes * (int64_t)g.Wp * (int64_t)sizeof(float);
     return SND_OK;
 }
 
@@ -100,6 +118,15 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (params->out_dtype != SND_F32 && params->out_dtype != params->shape.in_dtype) return SND_ERR_DTYPE;
     if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols))
         return SND_ERR_STRIDE;
+    if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
+    if (params->workspace) {
+        snd_plan plan;
+        snd_make_plan(&params->shape, &plan);
+        if (params->workspace_bytes < plan.fwd_workspace_bytes) return SND_ERR_WORKSPACE;
+        if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+    } else if (params->schedule == SND_SCHED_STRIPS) {
+        return SND_ERR_WORKSPACE;
+    }
     switch (params->shape.in_dtype) {
         case SND_F32: return snd::launch_fwd_f32(*params, (hipStream_t)stream);
         case SND_BF16: return snd::launch_fwd_bf16(*params, (hipStream_t)stream);
@@ -122,6 +149,7 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
     if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+    if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
     if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
                 params->f.shape.ncols))
         return SND_ERR_STRIDE;

@@ -60,6 +60,18 @@ __device__ __forceinline__ void st_f32(void *base, int i, int dt, float v) {
     else ((f16_t *)base)[i] = (f16_t)v;
 }
 
+// Streaming 16-byte accesses for data that is written once and read once much later (saved state):
+// marked non-temporal so that they do not displace the input lines that neighbouring tiles reuse.
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st4_stream(float *dst, float a, float b, float c, float d) {
+    v4f_t v = {a, b, c, d};
+    __builtin_nontemporal_store(v, (v4f_t *)dst);
+}
+__device__ __forceinline__ float4 ld4_stream(const float *src) {
+    const v4f_t v = __builtin_nontemporal_load((const v4f_t *)src);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 // ---------------------------------------------------------------- math
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -119,6 +131,89 @@ __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &p
     return pair < nPairs;
 }
 __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8) * 8 * nChunks; }
+
+// ---------------------------------------------------------------- strip pipeline
+// With few (batch, channel) planes a plane is split into its row strips, one block per strip; the
+// strips of a plane then run as a pipeline, each one tile behind the strip it depends on.
+// Blocks take (plane chunk, strip) jobs from a ticket counter in dependency order, so the block a
+// job waits for always holds an earlier ticket and is already running or finished.
+// Sync words (int32, zeroed before the launch): [0] ticket, [1] error flag, [4 + job] per-strip count
+// of tiles whose hand-over row the strip's block has written.
+#ifndef SND_POLL_SLEEP
+#define SND_POLL_SLEEP 16                           // s_sleep units (64 cycles) between polls
+#endif
+constexpr int kSyncHeader = 4;
+constexpr int kSpinLimit = 1 << 21;                 // polls (a memory round trip each) before giving up
+__host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips) {
+#ifdef SND_PIPE_TRACE   // timing study only: 4 extra words per job (start, end, time spent waiting, -)
+    return (kSyncHeader + 5 * nPlaneChunks * nStrips + 3) / 4 * 4;
+#else
+    return (kSyncHeader + nPlaneChunks * nStrips + 3) / 4 * 4;
+#endif
+}
+
+// Data handed from one block to another inside a launch is written and read with agent-scope
+// relaxed atomics (they go through to the coherence point and are never served from a stale line).
+__device__ __forceinline__ void st2_coherent(float *dst, float a, float b) {
+    const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+    __hip_atomic_store((uint64_t *)dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void ld2_coherent(const float *src, float &a, float &b) {
+    const uint64_t v = __hip_atomic_load((const uint64_t *)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    a = __builtin_bit_cast(float, (uint32_t)v);
+    b = __builtin_bit_cast(float, (uint32_t)(v >> 32));
+}
+__device__ __forceinline__ float ld1_coherent(const float *src) {
+    return __builtin_bit_cast(float, __hip_atomic_load((const uint32_t *)src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+// Publish in two steps: every wave waits for its own hand-over stores to complete (vmcnt 0) before
+// it reaches the block barrier; after the barrier one thread moves the count.
+__device__ __forceinline__ void strip_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void strip_signal(int *count) {
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+#ifdef SND_PIPE_TRACE
+#define SND_TRACE_ARG , int &trace_wait_
+#define SND_TRACE_PASS , trace_wait_
+#define g_wait_ticks trace_wait_
+#else
+#define SND_TRACE_ARG
+#define SND_TRACE_PASS
+#endif
+// Wait until *count >= need.  Bounded: after kSpinLimit polls the error word is set and the wave
+// goes on (with wrong data) so that the grid always drains; `dead` then disables further waits.
+__device__ __forceinline__ void strip_wait(const int *count, int need, int *sync, bool &dead SND_TRACE_ARG) {
+    if (dead) return;
+#ifdef SND_PIPE_TRACE
+    const long long t0_ = wall_clock64();
+#endif
+    int polls = 0;
+    while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+        __builtin_amdgcn_s_sleep(SND_POLL_SLEEP);
+        if (++polls > kSpinLimit) {
+            dead = true;
+            __hip_atomic_store(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+    }
+    asm volatile("" ::: "memory");
+#ifdef SND_PIPE_TRACE
+    g_wait_ticks += (int)(wall_clock64() - t0_);
+#endif
+}
+// Enqueue a fill kernel that zeroes n int32 words (defined with the C entry points).
+int zero_words(int *p, int64_t n, hipStream_t stream);
+// How a launch is scheduled (snd_fwd_params::schedule): one block per plane chunk walking all its
+// strips, or one block per strip with the strips of a plane pipelined.
+enum { kSchedAuto = 0, kSchedPlane = 1, kSchedStrips = 2 };
+// Strip pipelining pays when there are fewer whole-plane blocks than CUs (256): a strip waits for
+// the strip above at every tile, which costs more than it gains once the planes alone fill the chip
+// (measured at 768 plane blocks of 7x7 tiles: 2.2x slower forward, 1.3x slower backward).
+__host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int nStrips, const void *sync) {
+    if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return false;
+    if (schedule == kSchedStrips) return true;
+    return planeBlocks < 128 || (planeBlocks < 256 && nStrips >= 16);
+}
 
 // Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging
 // section so that the compiler recomputes a few integer ops per tile instead of hoisting dozens of

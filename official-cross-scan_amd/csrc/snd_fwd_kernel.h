@@ -26,7 +26,7 @@
 
 namespace snd {
 
-template <typename T, int NP, bool SAVE>
+template <typename T, int NP, bool SAVE, bool PIPE>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
     constexpr int CB = 16;                          // channels per block
@@ -46,7 +46,31 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
-    if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
+    int I_begin = 0, I_end = geo.nCY;               // strips this block walks
+    int *sync = (int *)p.workspace, *progress = nullptr;
+    bool dead = false;
+#ifdef SND_PIPE_TRACE
+    int *trace_ = nullptr, trace_wait_ = 0;
+#endif
+    if (PIPE) {
+        __shared__ int sTicket;
+        if (threadIdx.x == 0) sTicket = __hip_atomic_fetch_add(sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        // tickets run strip-major (all plane chunks' strip 0, then every strip 1, ...): a job's
+        // predecessor holds an earlier ticket, and a strip only takes a slot about when it can start
+        const int nPC = sh.batch * G * nChunks;
+        const int pc = sTicket % nPC;
+        I_begin = sTicket / nPC;
+        if (I_begin >= geo.nCY) return;
+        I_end = I_begin + 1;
+        pair = pc / nChunks;
+        chunk = pc - pair * nChunks;
+        progress = sync + kSyncHeader + pc * geo.nCY;
+#ifdef SND_PIPE_TRACE
+        trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_begin);
+        if (threadIdx.x == 0) trace_[0] = (int)wall_clock64();
+#endif
+    } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
 
@@ -93,24 +117,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo = 0.f;
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto prefetch = [&](int I, int J) {
-#ifdef SND_XF_NOLOAD
-        for (int k = 0; k < NBC; ++k) { qb[k] = 0.1f; qc[k] = 0.2f; }
-        for (int k = 0; k < NPX; ++k) { qdl[k] = 0.01f; qu[k] = 0.3f; }
-        qhalo = 0.01f; (void)I; (void)J;
-        return;
-#endif
         const int r0 = I * kRows, j0 = J * kCkX;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
-#ifdef SND_XF_NOXVLD
-        if (false) {
-#else
-        if (I > 0 && geo.nCX > 1) {                 // with one column tile the row comes from registers
-#endif
+        if (PIPE) {
+            // the row above comes from another block: fetched as late as possible (fetch_row_above)
+        } else if (I > 0 && geo.nCX > 1) {          // with one column tile the row comes from registers
             const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
-            const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+            const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
             qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
             qcorner = J > 0 ? src[7 - DN8] : 0.f;
@@ -145,6 +161,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
         }
     };
+    // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
+    // right before the tile needs it, so that a strip runs one tile behind the strip above.  One wave
+    // polls for the hand-over (more pollers only slow the counters down); the rest wait at the barrier.
+    auto fetch_row_above = [&](int I, int J) {
+        if (I == 0) return;
+        const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+#pragma unroll
+        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + k, qxv[k], qxv[k + 1]);
+        qcorner = J > 0 ? ld1_coherent(src + 7 - DN8) : 0.f;
+    };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&]() {
         SND_THREAD_MAPS(NP);
@@ -170,8 +196,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         }
     };
 
-    prefetch(0, 0);
-    for (int I = 0; I < geo.nCY; ++I) {
+    prefetch(I_begin, 0);
+    for (int I = I_begin; I < I_end; ++I) {
         const int r0 = I * kRows;
         float hl[kRows], sl[kRows], al[kRows];      // h, s, a at the column left of the tile
 #pragma unroll
@@ -180,16 +206,27 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         for (int J = 0; J < geo.nCX; ++J) {
             const int j0 = J * kCkX;
             commit();
-            // row above this tile: fetched one tile ahead (or handed over in registers)
-            float hup[kCkX], aup[kCkX];
-            float corner = (I > 0) ? qcorner : 0.f; // h[r0-1][j0-1]
-#pragma unroll
-            for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
+            if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, sync, dead SND_TRACE_PASS);
             __syncthreads();
+            // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
+            // registers), handed over in registers, or - strip pipeline - fetched here
+            float hup[kCkX], aup[kCkX];
+            float corner = 0.f;                     // h[r0-1][j0-1]
+            if (PIPE) fetch_row_above(I, J);
+            if (!PIPE) {
+                corner = (I > 0) ? qcorner : 0.f;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
+            }
             {   // issue the next tile's loads now; they complete while this tile is computed
                 int In = I, Jn = J + 1;
                 if (Jn == geo.nCX) { Jn = 0; In = I + 1; }
-                if (In < geo.nCY) prefetch(In, Jn);
+                if (In < I_end) prefetch(In, Jn);
+            }
+            if (PIPE) {
+                corner = (I > 0) ? qcorner : 0.f;
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
             }
 
             // ---- per-lane tile walk
@@ -235,34 +272,33 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     dst[1] = make_float4(y[4], y[5], y[6], y[7]);
                 }
             }
-            if (geo.nCX == 1) {                     // the next strip's row above is this tile's last row
+            if (!PIPE && geo.nCX == 1) {            // the next strip's row above is this tile's last row
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];
                 qcorner = 0.f;
             }
-#ifdef SND_XF_NOXVST
-            if (false) {
-#else
             if (lvalid) {
-#endif
                 // row checkpoint / carry to the next strip: h at the strip's last row
-                float4 *dst = (float4 *)(xv + ((int64_t)I * geo.nCX + J) * DN8);
-                dst[0] = make_float4(hup[0], hup[1], hup[2], hup[3]);
-                dst[1] = make_float4(hup[4], hup[5], hup[6], hup[7]);
-#ifdef SND_XF_NOCOL
-                if (false) {
-#else
-                if (SAVE && J + 1 < geo.nCX) {      // column checkpoints: only if a tile follows
-#endif
-                    float4 *dh = (float4 *)(xh + ((int64_t)J * geo.nCY + I) * DN8);
-                    float4 *ds = (float4 *)(xs + ((int64_t)J * geo.nCY + I) * DN8);
-                    dh[0] = make_float4(hl[0], hl[1], hl[2], hl[3]);
-                    dh[1] = make_float4(hl[4], hl[5], hl[6], hl[7]);
-                    ds[0] = make_float4(sl[0], sl[1], sl[2], sl[3]);
-                    ds[1] = make_float4(sl[4], sl[5], sl[6], sl[7]);
+                float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
+                if (PIPE) {
+#pragma unroll
+                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + k, hup[k], hup[k + 1]);
+                } else {
+                    st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
+                    st4_stream(dst + 4, hup[4], hup[5], hup[6], hup[7]);
                 }
             }
+            if (PIPE) strip_stores_done();
+            if (lvalid && SAVE && J + 1 < geo.nCX) {   // column checkpoints: only if a tile follows
+                float *dh = xh + ((int64_t)J * geo.nCY + I) * DN8;
+                float *ds = xs + ((int64_t)J * geo.nCY + I) * DN8;
+                st4_stream(dh, hl[0], hl[1], hl[2], hl[3]);
+                st4_stream(dh + 4, hl[4], hl[5], hl[6], hl[7]);
+                st4_stream(ds, sl[0], sl[1], sl[2], sl[3]);
+                st4_stream(ds + 4, sl[4], sl[5], sl[6], sl[7]);
+            }
             __syncthreads();
+            if (PIPE) strip_signal(progress + I);   // tile J is handed over to the strip below
 
             // ---- out = D*u + y, written by the thread that staged the pixel
             SND_THREAD_MAPS(NP);
@@ -271,17 +307,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-#ifdef SND_XF_NOOUT
-                if (false)
-#else
                 if (cvalid && row < H && col < W)
-#endif
                     st_f32(outb, cO + row * Oh + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
         }
     }
+#ifdef SND_PIPE_TRACE
+    if (PIPE && threadIdx.x == 0) { trace_[1] = (int)wall_clock64(); trace_[2] = trace_wait_; }
+#endif
 }
 
 template <typename T, int NP>
@@ -290,11 +325,22 @@ static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
     const Geo geo = make_geo(sh.nrows, sh.ncols);
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
-    const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
-    if (p.x != nullptr)
-        hipLaunchKernelGGL((fwd_kernel<T, NP, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
-    else
-        hipLaunchKernelGGL((fwd_kernel<T, NP, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+    const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
+    if (use_strip_pipeline(p.schedule, nPC, geo.nCY, p.workspace)) {
+        if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
+        if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
+        const int grid = (int)(nPC * geo.nCY);
+        if (p.x != nullptr)
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+        else
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+    } else {
+        const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
+        if (p.x != nullptr)
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+        else
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+    }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 

@@ -95,6 +95,9 @@ Checked check_inputs(const at::Tensor &u, const at::Tensor &delta, const at::Ten
     return c;
 }
 
+// snd_schedule used by fwd and bwd (0 = chosen by shape); set_schedule() is for tests and tuning.
+int g_schedule = SND_SCHED_AUTO;
+
 void fill_fwd(snd_fwd_params &p, const Checked &c, const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
               const at::Tensor &B, const at::Tensor &C, const c10::optional<at::Tensor> &D_,
               const c10::optional<at::Tensor> &delta_bias_, const c10::optional<at::Tensor> &A_decay_,
@@ -134,6 +137,11 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     p.out_dtype = dtype_code(out.scalar_type());
     p.out_batch_stride = out.stride(0); p.out_d_stride = out.stride(1); p.out_h_stride = out.stride(2);
     p.x = x.data_ptr<float>(); p.x_v = x_v.data_ptr<float>(); p.x_sd = x_sd.data_ptr<float>();
+    // scratch for the strip-pipelined schedule; released to the caching allocator in stream order
+    at::Tensor ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
+    p.workspace = ws.data_ptr();
+    p.workspace_bytes = c.plan.fwd_workspace_bytes;
+    p.schedule = g_schedule;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");
     return {out, x, x_v, x_sd};
@@ -194,6 +202,7 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     p.dA_decay = dA_decay.defined() ? dA_decay.data_ptr<float>() : nullptr;
     p.workspace = ws.data_ptr();
     p.workspace_bytes = c.plan.bwd_workspace_bytes;
+    p.f.schedule = g_schedule;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
 
@@ -212,4 +221,8 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)");
     m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)");
+    m.def("set_schedule", [](int mode) {
+        TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_STRIPS, "schedule must be 0 (auto), 1 (plane) or 2 (strips)");
+        g_schedule = mode;
+    }, "Force how fwd/bwd map work to blocks: 0 auto, 1 one block per plane chunk, 2 pipelined row strips");
 }

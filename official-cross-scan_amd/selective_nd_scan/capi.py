@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(PKG, "libsnd_scan.so")
 HEADER = os.path.join(ROOT, "include", "snd_scan.h")
 
 SND_F32, SND_F16, SND_BF16 = 0, 1, 2
+SCHED_AUTO, SCHED_PLANE, SCHED_STRIPS = 0, 1, 2
 i32, i64, vp = C.c_int32, C.c_int64, C.c_void_p
 
 
@@ -23,7 +24,8 @@ class Shape(C.Structure):
 
 class Plan(C.Structure):
     _fields_ = [("n_chunks_x", i32), ("n_chunks_y", i32), ("x_inner", i32), ("xv_inner", i32),
-                ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64)]
+                ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64),
+                ("fwd_workspace_bytes", i64)]
 
 
 class FwdParams(C.Structure):
@@ -34,7 +36,8 @@ class FwdParams(C.Structure):
                                     "A_d_stride", "A_dstate_stride",
                                     "B_batch_stride", "B_group_stride", "B_dstate_stride", "B_h_stride",
                                     "C_batch_stride", "C_group_stride", "C_dstate_stride", "C_h_stride",
-                                    "out_batch_stride", "out_d_stride", "out_h_stride")])
+                                    "out_batch_stride", "out_d_stride", "out_h_stride")] +
+                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("reserved_", i32)])
 
 
 class BwdParams(C.Structure):
@@ -88,8 +91,10 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, out, x, x_v, x_sd):
+def _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, out, x, x_v, x_sd,
+              schedule=SCHED_AUTO):
     fp.shape = shape
+    fp.schedule = schedule
     fp.out_dtype = _dt(out) if out is not None else SND_F32
     fp.delta_softplus = int(bool(delta_softplus))
     fp.u, fp.delta, fp.B, fp.C, fp.A = _ptr(u), _ptr(delta), _ptr(B), _ptr(Cc), _ptr(A)
@@ -118,7 +123,7 @@ class FwdCall:
     """Outputs, saved state and the filled snd_fwd_params of one forward; launch() only enqueues."""
 
     def __init__(self, u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True,
-                 A_decay=None, save=True):
+                 A_decay=None, save=True, schedule=SCHED_AUTO):
         import torch
         self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay)
         shape = make_shape(u, delta, A, B)
@@ -133,7 +138,9 @@ class FwdCall:
         self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.params = FwdParams()
         _fill_fwd(self.params, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, self.out,
-                  self.x, self.x_v, self.x_sd)
+                  self.x, self.x_v, self.x_sd, schedule)
+        self.ws = torch.empty(plan.fwd_workspace_bytes // 4 + 4, **f32)
+        self.params.workspace, self.params.workspace_bytes = self.ws.data_ptr(), plan.fwd_workspace_bytes
 
     def launch(self, stream=None):
         check(lib().snd_fwd(C.byref(self.params), _stream(stream)))
@@ -144,7 +151,8 @@ class BwdCall:
     the accumulated gradients (as the reference host does, selective_scan_oflex.cpp:395-403) and
     enqueues the kernel; launch_kernel_only() skips the zero-fill (timing)."""
 
-    def __init__(self, u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd):
+    def __init__(self, u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd,
+                 schedule=SCHED_AUTO):
         import torch
         self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, dout, x, x_v, x_sd)
         shape = make_shape(u, delta, A, B)
@@ -160,7 +168,8 @@ class BwdCall:
         self.ddec = torch.zeros_like(A_decay) if A_decay is not None else None
         self.ws = torch.empty(plan.bwd_workspace_bytes // 4 + 4, **f32)
         bp = self.params = BwdParams()
-        _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd)
+        _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd,
+                  schedule)
         bp.dout, bp.dout_dtype = dout.data_ptr(), _dt(dout)
         bp.dout_batch_stride, bp.dout_d_stride, bp.dout_h_stride = dout.stride(0), dout.stride(1), dout.stride(2)
         bp.du, bp.ddelta = self.du.data_ptr(), self.ddelta.data_ptr()
@@ -182,16 +191,17 @@ class BwdCall:
 
 
 def fwd(u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
-        save=True, stream=None):
+        save=True, stream=None, schedule=SCHED_AUTO):
     """Reference operator `fwd` (selective_scan_oflex.cpp:179-187) through the C ABI."""
-    call = FwdCall(u, delta, A, B, Cc, D, delta_bias, delta_softplus, out_float, A_decay, save)
+    call = FwdCall(u, delta, A, B, Cc, D, delta_bias, delta_softplus, out_float, A_decay, save, schedule)
     call.launch(stream)
     return call.out, call.x, call.x_v, call.x_sd
 
 
-def bwd(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, stream=None):
+def bwd(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, stream=None,
+        schedule=SCHED_AUTO):
     """Reference operator `bwd` (selective_scan_oflex.cpp:286-297, return list :432-438)."""
-    call = BwdCall(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd)
+    call = BwdCall(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, schedule)
     call.launch_kernel_only(stream)
     Bt, Dm, H, W = u.shape
     Dd = delta.shape[1]

@@ -35,6 +35,13 @@ def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay,
     return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd)
 
 
+def set_schedule(mode):
+    """How fwd/bwd map work to blocks: 0 = chosen by shape, 1 = one block per (batch, group,
+    16-channel chunk) plane, 2 = one block per 8-row strip, strips pipelined.  Results do not
+    depend on it (only the order of the atomic sums in dA, dB, dC, dD, ddelta_bias does)."""
+    ext().set_schedule(int(mode))
+
+
 def _last_dim_contiguous(t):
     return t if (t is None or t.stride(-1) == 1 or t.size(-1) == 1) else t.contiguous()
 

@@ -1,0 +1,87 @@
+"""Strip-pipelined schedule (one block per 8-row strip, strips of a plane pipelined through a
+ticket counter and per-strip progress counts) against the whole-plane schedule and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import capi
+from oracle import snd_oracle as O
+from oracle import snd_oracle_c as OC
+from test_gpu_fwd import relerr
+
+pytestmark = pytest.mark.gpu
+NAMES = ["du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias"]
+
+SHAPES = [
+    # Bt, Dm, H, W, N, K, dtype
+    (2, 16, 56, 56, 16, 4, torch.float32),     # 7 strips x 7 tiles
+    (1, 8, 17, 9, 16, 2, torch.float32),       # ragged edges, 3 strips x 2 tiles
+    (1, 32, 64, 8, 16, 1, torch.float32),      # one column tile: the row hand-over is the only carry
+    (1, 4, 24, 40, 4, 2, torch.float32),       # 8-state kernels
+    (1, 8, 100, 70, 16, 4, torch.bfloat16),
+    (3, 20, 33, 21, 5, 1, torch.float16),      # partial channel chunk (20 = 16 + 4), odd N
+]
+
+
+def sync_error(ws):
+    return int(ws.view(torch.int32)[1].item())
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,dtype", SHAPES)
+def test_strips_match_plane_and_oracle(gpu_device, Bt, Dm, H, W, N, K, dtype):
+    print("strips", Bt, Dm, H, W, N, K, dtype, flush=True)
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=5)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    for k in ("u", "delta", "B", "C"):
+        t[k] = t[k].to(dtype)
+    args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+    res = {}
+    for sched in (capi.SCHED_PLANE, capi.SCHED_STRIPS):
+        f = capi.FwdCall(*args, True, True, None, True, sched)
+        f.launch()
+        b = capi.BwdCall(*args, t["dout"], f.x, f.x_v, True, None, f.x_sd, sched)
+        b.launch()
+        torch.cuda.synchronize()
+        if sched == capi.SCHED_STRIPS:
+            assert sync_error(f.ws) == 0 and sync_error(b.ws) == 0, "a strip wait ran into its poll limit"
+        res[sched] = (f.out, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias], (f.x, f.x_v, f.x_sd))
+    out_p, g_p, st_p = res[capi.SCHED_PLANE]
+    out_s, g_s, st_s = res[capi.SCHED_STRIPS]
+    # same arithmetic in the same order per plane: everything that is not an atomic sum is bit-identical
+    assert torch.equal(out_p, out_s)
+    ncx = (W + 7) // 8
+    assert torch.equal(st_p[1], st_s[1])                      # x_v: every entry is written
+    for a, b_ in ((st_p[0], st_s[0]), (st_p[2], st_s[2])):    # x, x_sd: stored tile-major, last column tile unused
+        assert torch.equal(a.reshape(Bt, ncx, -1)[:, :ncx - 1], b_.reshape(Bt, ncx, -1)[:, :ncx - 1])
+    assert torch.equal(g_p[0], g_s[0]) and torch.equal(g_p[1], g_s[1])
+    r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    ref = OC.fwd(r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"], True, None, real="f64")
+    gref = OC.bwd(r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"], d["dout"], True, None, real="f64")
+    assert relerr(out_s.cpu().numpy(), ref) <= 1e-4
+    half = dtype != torch.float32
+    for nm, a, b_ in zip(NAMES, g_s, gref):
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 2e-4
+        assert relerr(a.float().cpu().numpy(), b_) <= tol, (nm, relerr(a.float().cpu().numpy(), b_))
+
+
+def test_strips_inference_only(gpu_device):
+    """x = x_sd = null (no column checkpoints) with the strip schedule."""
+    d = O.make_inputs(1, 16, 40, 24, N=16, K=2, seed=9)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+    f = capi.FwdCall(*args, True, True, None, False, capi.SCHED_STRIPS)
+    f.launch()
+    torch.cuda.synchronize()
+    assert sync_error(f.ws) == 0
+    ref = OC.fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True, None, real="f64")
+    assert relerr(f.out.cpu().numpy(), ref) <= 1e-4
+
+
+def test_strips_need_workspace(gpu_device):
+    d = O.make_inputs(1, 4, 16, 16, N=4, K=1, seed=1)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], None, None, False, True, None, True, capi.SCHED_STRIPS)
+    f.params.workspace = None
+    assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -6
+    f.params.workspace, f.params.workspace_bytes = f.ws.data_ptr(), 8
+    assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -6

@@ -21,9 +21,32 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
-    assert C.sizeof(capi.Plan) == 48
-    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8
+    assert C.sizeof(capi.Plan) == 56
+    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 8
     assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8
+
+
+def test_struct_layouts_match_the_c_compiler(tmp_path):
+    """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
+    import subprocess
+    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes"]),
+              ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule"]),
+              ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes"])]
+    src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
+    for cname, _, fields in probes:
+        src.append('printf("%%zu\\n", sizeof(%s));' % cname)
+        for f in fields:
+            src.append('printf("%%zu\\n", offsetof(%s, %s));' % (cname, f))
+    src += ["return 0; }"]
+    (tmp_path / "probe.c").write_text("\n".join(src))
+    exe = str(tmp_path / "probe")
+    subprocess.check_call(["gcc", "-I", os.path.join(capi.ROOT, "include"), str(tmp_path / "probe.c"), "-o", exe])
+    got = [int(v) for v in subprocess.check_output([exe]).split()]
+    want = []
+    for _, cls, fields in probes:
+        want.append(C.sizeof(cls))
+        want += [getattr(cls, f).offset for f in fields]
+    assert got == want
 
 
 @pytest.mark.parametrize("H,W,ncx,ncy", [(56, 56, 7, 7), (14, 14, 2, 2), (200, 336, 42, 25), (1, 37, 5, 1), (512, 512, 64, 64)])
@@ -35,7 +58,9 @@ def test_plan_geometry(H, W, ncx, ncy):
     planes = 2 * 8 * 16
     assert plan.x_elems == planes * ncx * plan.x_inner == plan.x_sd_elems
     assert plan.x_v_elems == planes * ncy * plan.xv_inner
-    assert plan.bwd_workspace_bytes == planes * plan.xv_inner * 4
+    sync_words = (4 + 2 * 4 * 1 * ncy + 3) // 4 * 4         # header + (batch * groups * chunks) * strips
+    assert plan.fwd_workspace_bytes == sync_words * 4
+    assert plan.bwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
 
 
 @pytest.mark.parametrize("shape,code", [
