@@ -20,7 +20,8 @@
 // from x_v, column to the left from x, s from x_sd) into 64 registers, then sweeps the tile
 // bottom-right to top-left.  The adjoint row handed to the strip above goes through a private
 // global scratch row; the column handed to the tile on the left stays in registers.  dB/dC are
-// reduced over the block's 16 channels with LDS atomics and leave the block once per tile;
+// reduced over a wave's channels with lane swaps, over the block's waves through LDS, and leave
+// the block once per tile;
 // du/ddelta are reduced over states by DPP and finished once per pixel by the thread that staged it.
 // As in the forward, tiles are computed in full on zero-padded staging (dout = B = C = 0 outside
 // the plane makes every adjoint there exactly zero), so the inner loops have no bounds checks.
@@ -30,9 +31,6 @@
 
 namespace snd {
 
-__device__ __forceinline__ void lds_add(float *p, float v) {
-    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-}
 __device__ __forceinline__ void glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -45,30 +43,6 @@ __device__ __forceinline__ void swap32(float &a, float &b) {
 __device__ __forceinline__ void swap16(float &a, float &b) {
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
-// Sum v[0..7] over the four 16-lane rows of a wave (= its four channels when a row holds the 16
-// states of one channel).  Row q of the wave ends up with the totals of v[2q] and v[2q+1]:
-// a reduce-scatter, 12 swaps + 12 adds for 8 values instead of 16 for a broadcast sum.
-__device__ __forceinline__ void rows_reduce8(const float (&v)[8], float &w0, float &w1) {
-    float t[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) { float a = v[k], b = v[k + 4]; swap32(a, b); t[k] = a + b; }
-    { float a = t[0], b = t[2]; swap16(a, b); w0 = a + b; }
-    { float a = t[1], b = t[3]; swap16(a, b); w1 = a + b; }
-}
-
-// Explicit use of the accumulation half of the unified register file as storage.
-#ifdef SND_TILE_IN_AGPR
-__device__ __forceinline__ void acc_put(float &slot, float v) { asm("v_accvgpr_write_b32 %0, %1" : "=a"(slot) : "v"(v)); }
-__device__ __forceinline__ float acc_get(const float &slot) {
-    float v;
-    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(slot));
-    return v;
-}
-#else
-__device__ __forceinline__ void acc_put(float &slot, float v) { slot = v; }
-__device__ __forceinline__ float acc_get(const float &slot) { return slot; }
-#endif
-
 #ifndef SND_BWD_WAVES
 #define SND_BWD_WAVES 2
 #endif
@@ -82,9 +56,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     constexpr int HG = 10, DLP = HG * HG;           // delta' on the tile plus a one-cell halo
     constexpr int NHALO = 36, NHK = (NHALO + NP - 1) / NP;
 
-    // NP == 16: a wave's four channels are reduced in registers (rows_reduce8) and every wave owns
-    // a partial dB/dC tile, written with plain stores.  NP == 8: one shared tile, LDS atomics.
-    constexpr int NPART = (NP == 16) ? WPB : 1;
+    // A wave's channels (four with 16 states per channel, eight with 8) are reduced in registers and
+    // every wave owns a partial dB/dC tile, written with plain stores.
+    constexpr int NPART = WPB;
     extern __shared__ __align__(16) float smem[];
     float *sB = smem;                               // [NP][NSTR]
     float *sC = sB + NP * NSTR;
@@ -178,12 +152,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const float *myDo = sDo + cl * kTile;
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
-    float *mydB = sdB + (NP == 16 ? wave * NP * NSTR : 0) + n * NSTR;
-    float *mydC = sdC + (NP == 16 ? wave * NP * NSTR : 0) + n * NSTR;
+    float *mydB = sdB + wave * NP * NSTR + n * NSTR;
+    float *mydC = sdC + wave * NP * NSTR + n * NSTR;
     const int qrow = (tid & 63) >> 4;               // 16-lane row of this lane inside its wave
-
-    if (NP != 16)
-        for (int i = tid; i < NP * NSTR; i += 16 * NP) { sdB[i] = 0.f; sdC[i] = 0.f; }
 
     // ---- register staging of one tile's raw inputs (global loads issued one tile ahead)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
@@ -449,8 +420,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
                         *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
                     }
-                    if (NP == 16) {
-                        // sum over the wave's 4 channels (its 16-lane rows): row q ends with column C0+q
+                    {
+                        // sum over the wave's channels: lane bits 4-5 by a swap reduce-scatter (the
+                        // 16-lane row q ends with column C0+q), bit 3 (8-state layout) by a row rotate
                         float b0 = vB[0], b2 = vB[2], b1 = vB[1], b3 = vB[3];
                         swap32(b0, b2); swap32(b1, b3);
                         float tb0 = b0 + b2, tb1 = b1 + b3;
@@ -459,13 +431,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         swap32(c0, c2); swap32(c1, c3);
                         float tc0 = c0 + c2, tc1 = c1 + c3;
                         swap16(tc0, tc1);
-                        mydB[r * kCkX + C0 + qrow] = tb0 + tb1;
-                        mydC[r * kCkX + C0 + qrow] = tc0 + tc1;
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            lds_add(mydB + r * kCkX + C0 + j, vB[j]);
-                            lds_add(mydC + r * kCkX + C0 + j, vC[j]);
+                        float tb = tb0 + tb1, tc = tc0 + tc1;
+                        if (NP == 8) { tb += dpp_mov<0x128>(tb); tc += dpp_mov<0x128>(tc); }   // row_ror:8
+                        if (NP == 16 || (tid & 8) == 0) {
+                            mydB[r * kCkX + C0 + qrow] = tb;
+                            mydC[r * kCkX + C0 + qrow] = tc;
                         }
                     }
                     Gd8 = GR[r];                    // G[r][C0+4]: diagonal neighbour for the row above
@@ -541,7 +511,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         glb_add(dBg + o, tb);
                         glb_add(dCg + o, tc);
                     }
-                    if (NP != 16) { sdB[sn * NSTR + px] = 0.f; sdC[sn * NSTR + px] = 0.f; }
                 }
             }
         }
@@ -582,7 +551,7 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
-    constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = (NP == 16) ? WPB : 1;
+    constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = WPB;
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
     const bool pipe = use_strip_pipeline(p.f.schedule, nPC, geo.nCY, p.workspace);
     // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
