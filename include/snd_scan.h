@@ -80,6 +80,16 @@ typedef struct snd_plan {
  *           apart (for few, large planes: c3/c4-like shapes).  Needs the workspace. */
 typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2 } snd_schedule;
 
+/* Scan origin per group.  The reference scans every group from the top-left corner and leaves the
+ * per-group order as a TODO (fwd.cuh:140); its callers build the four corner directions of the
+ * 2D-CrossScan block by flipping copies of the inputs and un-flipping the outputs.
+ *   TOPLEFT  every group runs top-left -> bottom-right (the reference's behaviour);
+ *   CORNERS  group g starts at corner g % 4: 0 top-left, 1 top-right (columns reversed),
+ *            2 bottom-left (rows reversed), 3 bottom-right (both).  All tensors stay in their natural
+ *            orientation in memory: the result equals flipping u, delta, B, C of that group, scanning
+ *            top-left, and flipping out (and every per-pixel gradient) back. */
+typedef enum snd_directions { SND_DIR_TOPLEFT = 0, SND_DIR_CORNERS = 1 } snd_directions;
+
 /* Replaces SSMParamsBase (selective_scan_oflex.h:4-51); 64-bit strides instead of uint32. */
 typedef struct snd_fwd_params {
     snd_shape shape;
@@ -104,7 +114,7 @@ typedef struct snd_fwd_params {
                                       PLANE schedule is used).  In snd_bwd_params.f it is ignored. */
     int64_t workspace_bytes;
     int32_t schedule;              /* snd_schedule, for fwd and (through snd_bwd_params.f) for bwd */
-    int32_t reserved_;             /* set to 0 */
+    int32_t directions;            /* snd_directions, for fwd and (through snd_bwd_params.f) for bwd */
 } snd_fwd_params;
 
 /* Replaces SSMParamsBwd (selective_scan_oflex.h:53-86). Gradient buffers are dense (contiguous):

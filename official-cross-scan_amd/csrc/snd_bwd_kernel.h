@@ -107,6 +107,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
+    // scan origin of this group (as in the forward): memory row = mrow(i), column = mcol(j)
+    const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
+    auto mrow = [&](int r) { return fv ? H - 1 - r : r; };
+    auto mcol = [&](int c_) { return fh ? W - 1 - c_ : c_; };
 
     const int tid = threadIdx.x, wave = tid >> 6;
     const int n = tid % NP, cl = tid / NP;
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
-            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
             const int ob = rc * Bh + cx, oc = rc * Ch + cx;
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
             const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
             const float vo = ld_f32(dob, cDo + rc * Doh + cx, p.dout_dtype);
             qdl[k] = ok ? vd : 0.f;
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             else { rr = hidx - 27; jj = 9; }
             const int row = r0 - 1 + rr, col = j0 - 1 + jj;
             const bool ok = cvalid && row >= 0 && row < H && col >= 0 && col < W;
-            const float vd = ldg(db, cD + min(max(row, 0), H - 1) * Dh + min(max(col, 0), W - 1));
+            const float vd = ldg(db, cD + mrow(min(max(row, 0), H - 1)) * Dh + mcol(min(max(col, 0), W - 1)));
             qh[k] = ok ? vd : 0.f;
         }
     };
@@ -487,8 +491,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 dD_acc = fmaf(dov, uv, dD_acc);
                 dbias_acc += ddl;
                 if (cvalid && row < H && col < W) {
-                    stg(dub, cG + row * W + col, duv);
-                    stg(ddb, cG + row * W + col, ddl);
+                    stg(dub, cG + mrow(row) * W + mcol(col), duv);
+                    stg(ddb, cG + mrow(row) * W + mcol(col), ddl);
                 }
             }
             }
@@ -507,7 +511,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         tc += sdC[w * NP * NSTR + sn * NSTR + px];
                     }
                     if (in && sn < N) {
-                        const int o = (sn * H + row) * W + col;
+                        const int o = (sn * H + mrow(row)) * W + mcol(col);
                         glb_add(dBg + o, tb);
                         glb_add(dCg + o, tc);
                     }

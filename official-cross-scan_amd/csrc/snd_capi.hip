@@ -73,7 +73,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 101; }
+int snd_version(void) { return 102; }
 
 const char *snd_status_string(int status) {
     switch (status) {
@@ -119,6 +119,7 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols))
         return SND_ERR_STRIDE;
     if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
+    if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (params->workspace) {
         snd_plan plan;
         snd_make_plan(&params->shape, &plan);
@@ -150,6 +151,7 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
     if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
     if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
     if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
+    if (params->f.directions != SND_DIR_TOPLEFT && params->f.directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
                 params->f.shape.ncols))
         return SND_ERR_STRIDE;

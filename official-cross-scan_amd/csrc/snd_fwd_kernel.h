@@ -73,6 +73,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
+    // scan origin of this group: the scan runs in (i, j) from (0, 0); memory row = mrow(i), column =
+    // mcol(j).  Only the staging loads and the output stores know about it.
+    const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
+    auto mrow = [&](int r) { return fv ? H - 1 - r : r; };
+    auto mcol = [&](int c_) { return fh ? W - 1 - c_ : c_; };
 
     const int tid = threadIdx.x, wave = tid >> 6;
     const int n = tid % NP, cl = tid / NP;          // state and block-local channel of this lane
@@ -135,7 +140,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
-            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
             const int ob = rc * Bh + cx, oc = rc * Ch + cx;
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
@@ -150,14 +155,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            const int rc = min(row, H - 1), cx = min(col, W - 1);
+            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
             const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
             qdl[k] = ok ? vd : 0.f;
             qu[k] = ok ? vu : 0.f;
         }
         if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
             const int row = r0 - 1, col = j0 + n;
-            const float vd = ldg(db, cD + max(row, 0) * Dh + min(col, W - 1));
+            const float vd = ldg(db, cD + mrow(max(row, 0)) * Dh + mcol(min(col, W - 1)));
             qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
         }
     };
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                 if (cvalid && row < H && col < W)
-                    st_f32(outb, cO + row * Oh + col, p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                    st_f32(outb, cO + mrow(row) * Oh + mcol(col), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it

@@ -121,7 +121,9 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
                                            const at::Tensor &B, const at::Tensor &C,
                                            const c10::optional<at::Tensor> &D_,
                                            const c10::optional<at::Tensor> &delta_bias_, bool delta_softplus,
-                                           bool out_float, const c10::optional<at::Tensor> &A_decay_) {
+                                           bool out_float, const c10::optional<at::Tensor> &A_decay_,
+                                           int64_t directions) {
+    TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
     at::hip::HIPGuardMasqueradingAsCUDA device_guard{u.device()};
     const auto f32 = u.options().dtype(at::ScalarType::Float);
@@ -142,6 +144,7 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     p.workspace = ws.data_ptr();
     p.workspace_bytes = c.plan.fwd_workspace_bytes;
     p.schedule = g_schedule;
+    p.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");
     return {out, x, x_v, x_sd};
@@ -153,7 +156,8 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
                                            const c10::optional<at::Tensor> &delta_bias_, const at::Tensor &dout,
                                            const c10::optional<at::Tensor> &x_, const c10::optional<at::Tensor> &x_v_,
                                            bool delta_softplus, const c10::optional<at::Tensor> &A_decay_,
-                                           const c10::optional<at::Tensor> &x_sd_) {
+                                           const c10::optional<at::Tensor> &x_sd_, int64_t directions) {
+    TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
     const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate;
     TORCH_CHECK(dout.scalar_type() == u.scalar_type() || dout.scalar_type() == at::ScalarType::Float,
@@ -203,6 +207,7 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     p.workspace = ws.data_ptr();
     p.workspace_bytes = c.plan.bwd_workspace_bytes;
     p.f.schedule = g_schedule;
+    p.f.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
 
@@ -219,8 +224,15 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
-    m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)");
-    m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)");
+    // the reference's positional lists (selective_scan_oflex.cpp:179-187,286-297) plus one trailing
+    // optional argument: the per-group scan origin the reference leaves as a TODO (fwd.cuh:140)
+    namespace py = pybind11;
+    m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
+          py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("delta_softplus"), py::arg("out_float"),
+          py::arg("A_decay"), py::arg("directions") = 0);
+    m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
+          py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("dout"), py::arg("x"), py::arg("x_v"),
+          py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0);
     m.def("set_schedule", [](int mode) {
         TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_STRIPS, "schedule must be 0 (auto), 1 (plane) or 2 (strips)");
         g_schedule = mode;

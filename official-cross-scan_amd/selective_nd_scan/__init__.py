@@ -2,3 +2,7 @@
 from .interface import SelectiveNdScanFn, bwd, fwd, selective_nd_scan, set_schedule  # noqa: F401
 
 __all__ = ["selective_nd_scan", "SelectiveNdScanFn", "fwd", "bwd", "set_schedule"]
+from .cross_scan import (cross_merge, cross_scan, cross_scan_2d, four_corner_scan,  # noqa: F401,E402
+                         four_corner_scan_by_flips)
+
+__all__ += ["cross_scan", "cross_merge", "cross_scan_2d", "four_corner_scan", "four_corner_scan_by_flips"]

@@ -15,6 +15,7 @@ HEADER = os.path.join(ROOT, "include", "snd_scan.h")
 
 SND_F32, SND_F16, SND_BF16 = 0, 1, 2
 SCHED_AUTO, SCHED_PLANE, SCHED_STRIPS = 0, 1, 2
+DIR_TOPLEFT, DIR_CORNERS = 0, 1
 i32, i64, vp = C.c_int32, C.c_int64, C.c_void_p
 
 
@@ -37,7 +38,7 @@ class FwdParams(C.Structure):
                                     "B_batch_stride", "B_group_stride", "B_dstate_stride", "B_h_stride",
                                     "C_batch_stride", "C_group_stride", "C_dstate_stride", "C_h_stride",
                                     "out_batch_stride", "out_d_stride", "out_h_stride")] +
-                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("reserved_", i32)])
+                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("directions", i32)])
 
 
 class BwdParams(C.Structure):
@@ -92,9 +93,10 @@ def _ptr(t):
 
 
 def _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, out, x, x_v, x_sd,
-              schedule=SCHED_AUTO):
+              schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
     fp.shape = shape
     fp.schedule = schedule
+    fp.directions = directions
     fp.out_dtype = _dt(out) if out is not None else SND_F32
     fp.delta_softplus = int(bool(delta_softplus))
     fp.u, fp.delta, fp.B, fp.C, fp.A = _ptr(u), _ptr(delta), _ptr(B), _ptr(Cc), _ptr(A)
@@ -123,7 +125,7 @@ class FwdCall:
     """Outputs, saved state and the filled snd_fwd_params of one forward; launch() only enqueues."""
 
     def __init__(self, u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True,
-                 A_decay=None, save=True, schedule=SCHED_AUTO):
+                 A_decay=None, save=True, schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
         import torch
         self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay)
         shape = make_shape(u, delta, A, B)
@@ -138,7 +140,7 @@ class FwdCall:
         self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.params = FwdParams()
         _fill_fwd(self.params, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, self.out,
-                  self.x, self.x_v, self.x_sd, schedule)
+                  self.x, self.x_v, self.x_sd, schedule, directions)
         self.ws = torch.empty(plan.fwd_workspace_bytes // 4 + 4, **f32)
         self.params.workspace, self.params.workspace_bytes = self.ws.data_ptr(), plan.fwd_workspace_bytes
 
@@ -152,7 +154,7 @@ class BwdCall:
     enqueues the kernel; launch_kernel_only() skips the zero-fill (timing)."""
 
     def __init__(self, u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd,
-                 schedule=SCHED_AUTO):
+                 schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
         import torch
         self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, dout, x, x_v, x_sd)
         shape = make_shape(u, delta, A, B)
@@ -169,7 +171,7 @@ class BwdCall:
         self.ws = torch.empty(plan.bwd_workspace_bytes // 4 + 4, **f32)
         bp = self.params = BwdParams()
         _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd,
-                  schedule)
+                  schedule, directions)
         bp.dout, bp.dout_dtype = dout.data_ptr(), _dt(dout)
         bp.dout_batch_stride, bp.dout_d_stride, bp.dout_h_stride = dout.stride(0), dout.stride(1), dout.stride(2)
         bp.du, bp.ddelta = self.du.data_ptr(), self.ddelta.data_ptr()
@@ -191,17 +193,18 @@ class BwdCall:
 
 
 def fwd(u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
-        save=True, stream=None, schedule=SCHED_AUTO):
+        save=True, stream=None, schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
     """Reference operator `fwd` (selective_scan_oflex.cpp:179-187) through the C ABI."""
-    call = FwdCall(u, delta, A, B, Cc, D, delta_bias, delta_softplus, out_float, A_decay, save, schedule)
+    call = FwdCall(u, delta, A, B, Cc, D, delta_bias, delta_softplus, out_float, A_decay, save, schedule, directions)
     call.launch(stream)
     return call.out, call.x, call.x_v, call.x_sd
 
 
 def bwd(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, stream=None,
-        schedule=SCHED_AUTO):
+        schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
     """Reference operator `bwd` (selective_scan_oflex.cpp:286-297, return list :432-438)."""
-    call = BwdCall(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, schedule)
+    call = BwdCall(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, schedule,
+                   directions)
     call.launch_kernel_only(stream)
     Bt, Dm, H, W = u.shape
     Dd = delta.shape[1]

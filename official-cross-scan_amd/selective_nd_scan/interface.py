@@ -15,24 +15,25 @@ order of those bindings (selective_scan_oflex.cpp:179-187).
     D      [D] fp32, delta_bias [Dd] fp32, A_decay [1] fp32 (all optional)
     out    [B, D, H, W]        fp32 if out_float else u.dtype
 
-Every group is scanned from the top-left corner, as the reference kernel does
-(selective_scan_fwd_kernel_oflex.cuh:140); the four corner directions are made by the caller
-(see cross_scan.py).
+With directions=0 every group is scanned from the top-left corner, as the reference kernel does
+(selective_scan_fwd_kernel_oflex.cuh:140).  directions=1 starts group g at corner g % 4 inside the
+kernels (no flipped copies); cross_scan.py builds the four-corner block on top of it.
 """
 import torch
 
 from ._ext import ext
 
 
-def fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None):
+def fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
+        directions=0):
     """Reference binding `fwd` -> [out, x, x_v, x_sd] (selective_scan_oflex.cpp:179-187,282)."""
-    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)
+    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)
 
 
-def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd):
+def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions=0):
     """Reference binding `bwd` -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
     (selective_scan_oflex.cpp:286-297,432-438)."""
-    return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd)
+    return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions)
 
 
 def set_schedule(mode):
@@ -50,10 +51,11 @@ class SelectiveNdScanFn(torch.autograd.Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
-                A_decay=None):
+                A_decay=None, directions=0):
         u, delta, B, C = map(_last_dim_contiguous, (u, delta, B, C))
-        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)
+        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)
         ctx.delta_softplus = delta_softplus
+        ctx.directions = directions
         ctx.has = (D is not None, delta_bias is not None, A_decay is not None)
         ctx.save_for_backward(u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd)
         return out
@@ -64,13 +66,14 @@ class SelectiveNdScanFn(torch.autograd.Function):
         u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd = ctx.saved_tensors
         dout = _last_dim_contiguous(dout)
         du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay = bwd(
-            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd)
+            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions)
         has_D, has_bias, has_decay = ctx.has
         return (du, ddelta, dA, dB, dC, dD if has_D else None, ddelta_bias if has_bias else None,
-                None, None, dA_decay if has_decay else None)
+                None, None, dA_decay if has_decay else None, None)
 
 
 def selective_nd_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
-                      A_decay=None):
-    """Differentiable 2D-CrossScan selective scan (forward and backward run on the HIP kernels)."""
-    return SelectiveNdScanFn.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay)
+                      A_decay=None, directions=0):
+    """Differentiable 2D-CrossScan selective scan (forward and backward run on the HIP kernels).
+    directions=1: group g of B/C (and its dim/G channels) is scanned from corner g % 4."""
+    return SelectiveNdScanFn.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)

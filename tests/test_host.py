@@ -106,3 +106,24 @@ def test_extension_checks_mirror_reference_messages():
         s.fwd(z(1, 4, 3, 4), z(1, 4, 3, 4), z(4, 2, dtype=torch.float16), z(1, 1, 2, 3, 4), z(1, 1, 2, 3, 4))
     with pytest.raises(RuntimeError):                       # dtype mismatch (:193)
         s.fwd(z(1, 4, 3, 4), z(1, 4, 3, 4, dtype=torch.float16), z(4, 2), z(1, 1, 2, 3, 4), z(1, 1, 2, 3, 4))
+
+
+def test_cross_scan_host_helpers():
+    """Direction-major layout helpers of the four-corner block (pure tensor bookkeeping, CPU)."""
+    import torch
+    from selective_nd_scan import cross_scan as cs
+    x = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).reshape(2, 3, 4, 5)
+    xs = cs.cross_scan(x)
+    assert xs.shape == (2, 12, 4, 5) and torch.equal(xs[:, 3:6], x) and torch.equal(xs[:, 9:], x)
+    f = cs.flip_groups(xs, 4)
+    assert torch.equal(f[:, 0:3], x) and torch.equal(f[:, 3:6], x.flip(-1))
+    assert torch.equal(f[:, 6:9], x.flip(-2)) and torch.equal(f[:, 9:12], x.flip(-2, -1))
+    assert torch.equal(cs.flip_groups(f, 4), xs)                       # an involution
+    b5 = torch.randn(2, 8, 3, 4, 5)
+    f5 = cs.flip_groups(b5, 8)
+    assert torch.equal(f5[:, 5], b5[:, 5].flip(-1)) and torch.equal(cs.flip_groups(f5, 8), b5)
+    assert torch.equal(cs.cross_merge(xs), 4 * x)
+    w = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    assert torch.allclose(cs.cross_merge(xs, w), 10 * x)
+    wc = torch.arange(12, dtype=torch.float32).reshape(4, 3)
+    assert torch.allclose(cs.cross_merge(xs, wc), x * wc.sum(0).reshape(1, 3, 1, 1))
