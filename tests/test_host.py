@@ -111,7 +111,8 @@ def test_extension_checks_mirror_reference_messages():
 def test_cross_scan_host_helpers():
     """Direction-major layout helpers of the four-corner block (pure tensor bookkeeping, CPU)."""
     import torch
-    from selective_nd_scan import cross_scan as cs
+    import importlib
+    cs = importlib.import_module("selective_nd_scan.cross_scan")   # the module, not the function of that name
     x = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).reshape(2, 3, 4, 5)
     xs = cs.cross_scan(x)
     assert xs.shape == (2, 12, 4, 5) and torch.equal(xs[:, 3:6], x) and torch.equal(xs[:, 9:], x)
