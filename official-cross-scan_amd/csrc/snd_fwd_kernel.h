@@ -118,24 +118,21 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
 
-    // raw values of one tile, held in registers between their global load and their LDS commit
-    float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo = 0.f;
+    // Raw values of a tile, held in registers between their global load and their LDS commit.
+    // Tiles are loaded in aligned pairs (columns 16m..16m+15, both tiles' loads issued together),
+    // so that the two 32-byte halves of each 64-byte run are requested while the memory line is in
+    // flight: a line is fetched from HBM twice per strip instead of four times.
+    // (Only where it pays and fits: the 16-state whole-plane kernels, which are bandwidth-bound.)
+    constexpr bool PAIR = NP == 16 && !PIPE;
+    struct Stage { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo; };
+    Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
-    auto prefetch = [&](int I, int J) {
+    auto load_tile = [&](Stage &q, int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
-        if (PIPE) {
-            // the row above comes from another block: fetched as late as possible (fetch_row_above)
-        } else if (I > 0 && geo.nCX > 1) {          // with one column tile the row comes from registers
-            const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
-            const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
-            qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
-            qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
-            qcorner = J > 0 ? src[7 - DN8] : 0.f;
-        }
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
@@ -146,8 +143,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             for (int k = 0; k < NBC; ++k) {
                 const int sn = wave + WPB * k, sc = min(sn, N - 1);
                 const float vb = ldg(Bb, sc * Bs + ob), vc = ldg(Cb, sc * Cs + oc);
-                qb[k] = (in && sn < N) ? vb : 0.f;
-                qc[k] = (in && sn < N) ? vc : 0.f;
+                q.qb[k] = (in && sn < N) ? vb : 0.f;
+                q.qc[k] = (in && sn < N) ? vc : 0.f;
             }
         }
 #pragma unroll
@@ -157,13 +154,29 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const bool ok = cvalid && row < H && col < W;
             const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
             const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
-            qdl[k] = ok ? vd : 0.f;
-            qu[k] = ok ? vu : 0.f;
+            q.qdl[k] = ok ? vd : 0.f;
+            q.qu[k] = ok ? vu : 0.f;
         }
+        q.qhalo = 0.f;
         if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
             const int row = r0 - 1, col = j0 + n;
             const float vd = ldg(db, cD + mrow(max(row, 0)) * Dh + mcol(min(col, W - 1)));
-            qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
+            q.qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
+        }
+    };
+    // the pair of tiles that starts at (I, J), J even (or the single tile when not pairing)
+    auto load_pair = [&](int I, int J) {
+        load_tile(st0, I, J);
+        if (PAIR && J + 1 < geo.nCX) load_tile(st1, I, J + 1);
+    };
+    // h of the row above tile (I, J), one tile ahead (whole-plane schedule)
+    auto prefetch_xv = [&](int I, int J) {
+        if (!PIPE && I > 0 && geo.nCX > 1) {        // with one column tile the row comes from registers
+            const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+            const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
+            qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
+            qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
+            qcorner = J > 0 ? src[7 - DN8] : 0.f;
         }
     };
     // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
@@ -177,40 +190,43 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         qcorner = J > 0 ? ld1_coherent(src + 7 - DN8) : 0.f;
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
-    auto commit = [&]() {
+    auto commit = [&](const Stage &q) {
         SND_THREAD_MAPS(NP);
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
             const int sn = wave + WPB * k;
-            sB[sn * NSTR + px] = qb[k];
-            sC[sn * NSTR + px] = qc[k];
+            sB[sn * NSTR + px] = q.qb[k];
+            sC[sn * NSTR + px] = q.qc[k];
         }
         float dsp;
 #pragma unroll
         for (int k = 0; k < NPX; ++k) {
             const int pp = n + NP * k;
-            const float raw = qdl[k] + bias;
+            const float raw = q.qdl[k] + bias;
             const float dl = softplus ? softplus20(raw, dsp) : raw;
             sDl[cl * DLP + kCkX + pp] = dl;
-            sDu[cl * kTile + pp] = dl * qu[k];
-            dukeep[k] = Dv * qu[k];
+            sDu[cl * kTile + pp] = dl * q.qu[k];
+            dukeep[k] = Dv * q.qu[k];
         }
         if (n < kCkX) {
-            const float raw = qhalo + bias;
+            const float raw = q.qhalo + bias;
             sDl[cl * DLP + n] = softplus ? softplus20(raw, dsp) : raw;
         }
     };
 
-    prefetch(I_begin, 0);
+    load_pair(I_begin, 0);
+    prefetch_xv(I_begin, 0);
     for (int I = I_begin; I < I_end; ++I) {
         const int r0 = I * kRows;
         float hl[kRows], sl[kRows], al[kRows];      // h, s, a at the column left of the tile
 #pragma unroll
         for (int r = 0; r < kRows; ++r) { hl[r] = 0.f; sl[r] = 0.f; al[r] = 0.f; }
 
-        for (int J = 0; J < geo.nCX; ++J) {
+        // one tile; `mine` holds its staged inputs, `last_of_pair` says that both register sets are
+        // free once it is committed, so the next pair's loads can be issued under its compute
+        auto do_tile = [&](const int J, const Stage &mine, const bool last_of_pair) {
             const int j0 = J * kCkX;
-            commit();
+            commit(mine);
             if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, sync, dead SND_TRACE_PASS);
             __syncthreads();
             // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
@@ -223,10 +239,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
             }
-            {   // issue the next tile's loads now; they complete while this tile is computed
+            {   // issue the next loads now; they complete while this tile is computed
                 int In = I, Jn = J + 1;
                 if (Jn == geo.nCX) { Jn = 0; In = I + 1; }
-                if (In < I_end) prefetch(In, Jn);
+                if (In < I_end) {
+                    prefetch_xv(In, Jn);
+                    if (last_of_pair) load_pair(In, Jn);
+                }
             }
             if (PIPE) {
                 corner = (I > 0) ? qcorner : 0.f;
@@ -317,6 +336,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
+        };
+        if (PAIR) {
+            for (int J = 0; J < geo.nCX; J += 2) {
+                const bool single = J + 1 >= geo.nCX;
+                do_tile(J, st0, single);
+                if (!single) do_tile(J + 1, st1, true);
+            }
+        } else {
+            for (int J = 0; J < geo.nCX; ++J) do_tile(J, st0, true);
         }
     }
 #ifdef SND_PIPE_TRACE
