@@ -418,11 +418,21 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         vB[j] = dbu * duv;                         // dB, dC contributions
                         vC[j] = dov * fmaf(0.25f, bu, hb - sb);
                     }
-                    group_sum4<NP>(q[0], q[1], q[2], q[3]);
-                    group_sum4<NP>(pp_[0], pp_[1], pp_[2], pp_[3]);
-                    if (n == 0) {
-                        *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
-                        *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
+                    if (NP == 16) {
+                        // sums over the channel's 16 states: quads 0,1 of the lane group end with
+                        // q[0..1], q[2..3], quads 2,3 with pp_[0..1], pp_[2..3]
+                        group_scatter8(q[0], q[1], q[2], q[3], pp_[0], pp_[1], pp_[2], pp_[3]);
+                        if ((n & 3) == 0) {
+                            float *dst = ((n & 8) ? sP : sQ) + cl * kTile + r * kCkX + C0 + ((n >> 1) & 2);
+                            *(float2 *)dst = make_float2(q[0], q[1]);
+                        }
+                    } else {
+                        group_sum4<NP>(q[0], q[1], q[2], q[3]);
+                        group_sum4<NP>(pp_[0], pp_[1], pp_[2], pp_[3]);
+                        if (n == 0) {
+                            *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
+                            *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
+                        }
                     }
                     {
                         // sum over the wave's channels: lane bits 4-5 by a swap reduce-scatter (the

@@ -122,6 +122,31 @@ template <int NP> __device__ __forceinline__ void group_sum4(float &a, float &b,
     else { a = group_sum<NP>(a); b = group_sum<NP>(b); c = group_sum<NP>(c); d = group_sum<NP>(d); }
 }
 
+// Reduce-scatter of eight values over an aligned group of 16 lanes (one DPP row): afterwards all
+// four lanes of quad b (lanes 4b..4b+3 of the row) hold in v0, v1 the group totals of the original
+// v[2b], v[2b+1]; v2..v7 are clobbered.  16 DPP adds instead of the 32 of eight broadcast sums:
+//   lane bit 3: banks 0-1 fold their partner's v0..v3 in place, banks 2-3 write v4..v7 folded into v0..v3;
+//   lane bit 2: banks 0,2 fold v0,v1 from the quad above, banks 1,3 write v2,v3 folded into v0,v1;
+//   lane bits 1,0: plain butterfly on v0, v1.
+// A DPP operand must not have been written by either of the two preceding VALU instructions; the
+// instruction order below and the s_nops keep that distance.
+#define SND_DPPA(d, s, ctrl, bank) "v_add_f32_dpp " d ", " s ", " s " " ctrl " row_mask:0xf bank_mask:" bank "\n\t"
+__device__ __forceinline__ void group_scatter8(float &v0, float &v1, float &v2, float &v3, float &v4, float &v5,
+                                               float &v6, float &v7) {
+    asm("s_nop 1\n\t"
+        SND_DPPA("%0", "%0", "row_ror:8", "0x3") SND_DPPA("%1", "%1", "row_ror:8", "0x3")
+        SND_DPPA("%2", "%2", "row_ror:8", "0x3") SND_DPPA("%3", "%3", "row_ror:8", "0x3")
+        SND_DPPA("%0", "%4", "row_ror:8", "0xc") SND_DPPA("%1", "%5", "row_ror:8", "0xc")
+        SND_DPPA("%2", "%6", "row_ror:8", "0xc") SND_DPPA("%3", "%7", "row_ror:8", "0xc")
+        SND_DPPA("%0", "%0", "row_shl:4", "0x5") SND_DPPA("%1", "%1", "row_shl:4", "0x5")
+        SND_DPPA("%0", "%2", "row_shr:4", "0xa") SND_DPPA("%1", "%3", "row_shr:4", "0xa")
+        "s_nop 0\n\t"
+        SND_DPPA("%0", "%0", "quad_perm:[1,0,3,2]", "0xf") SND_DPPA("%1", "%1", "quad_perm:[1,0,3,2]", "0xf")
+        "s_nop 0\n\t"
+        SND_DPPA("%0", "%0", "quad_perm:[2,3,0,1]", "0xf") SND_DPPA("%1", "%1", "quad_perm:[2,3,0,1]", "0xf")
+        : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7));
+}
+
 // Blocks are dealt round-robin to the 8 XCDs (each with its own L2).  Keep every chunk of one
 // (batch, group) pair - they all stream the same B/C planes - on one XCD.
 __device__ __forceinline__ bool xcd_job(int bid, int nPairs, int nChunks, int &pair, int &chunk) {

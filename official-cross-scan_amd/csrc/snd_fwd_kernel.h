@@ -288,12 +288,18 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     }
                 }
                 hl[r] = left; sl[r] = sleft; al[r] = aleft;
-                group_sum4<NP>(y[0], y[1], y[2], y[3]);
-                group_sum4<NP>(y[4], y[5], y[6], y[7]);
-                if (n == 0) {
-                    float4 *dst = (float4 *)(sY + cl * kTile + r * kCkX);
-                    dst[0] = make_float4(y[0], y[1], y[2], y[3]);
-                    dst[1] = make_float4(y[4], y[5], y[6], y[7]);
+                if (NP == 16) {
+                    // sum over the channel's 16 states; quad q of the lane group ends with columns 2q, 2q+1
+                    group_scatter8(y[0], y[1], y[2], y[3], y[4], y[5], y[6], y[7]);
+                    if ((n & 3) == 0) *(float2 *)(sY + cl * kTile + r * kCkX + (n >> 1)) = make_float2(y[0], y[1]);
+                } else {
+                    group_sum4<NP>(y[0], y[1], y[2], y[3]);
+                    group_sum4<NP>(y[4], y[5], y[6], y[7]);
+                    if (n == 0) {
+                        float4 *dst = (float4 *)(sY + cl * kTile + r * kCkX);
+                        dst[0] = make_float4(y[0], y[1], y[2], y[3]);
+                        dst[1] = make_float4(y[4], y[5], y[6], y[7]);
+                    }
                 }
             }
             if (!PIPE && geo.nCX == 1) {            // the next strip's row above is this tile's last row
