@@ -376,14 +376,19 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                 for (int r = kRows - 1; r >= 0; --r) {
                     __builtin_amdgcn_sched_barrier(0);
-                    float arow[5], s[4];
+                    float arow[5], s[4], buv[4];
 #pragma unroll
                     for (int j = 0; j <= 4; ++j) arow[j] = AEXP(r, C0 + j);
+                    const float4 vB4 = *(const float4 *)(myB + r * kCkX + C0), vC4 = *(const float4 *)(myC + r * kCkX + C0);
+                    const float4 vU4 = *(const float4 *)(myDu + r * kCkX + C0), vO4 = *(const float4 *)(myDo + r * kCkX + C0);
+                    const float aB[4] = {vB4.x, vB4.y, vB4.z, vB4.w}, aC[4] = {vC4.x, vC4.y, vC4.z, vC4.w};
+                    const float aU[4] = {vU4.x, vU4.y, vU4.z, vU4.w}, aO[4] = {vO4.x, vO4.y, vO4.z, vO4.w};
                     {
                         float sp = sL[r];
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
-                            sp = fmaf(arow[j], sp, myB[r * kCkX + C0 + j] * myDu[r * kCkX + C0 + j]);
+                            buv[j] = aB[j] * aU[j];
+                            sp = fmaf(arow[j], sp, buv[j]);
                             s[j] = sp;
                         }
                     }
@@ -391,11 +396,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     float q[4], pp_[4], vB[4], vC[4];
 #pragma unroll
                     for (int j = 3; j >= 0; --j) {
-                        const int o = r * kCkX + C0 + j;
-                        const float dov = myDo[o];
-                        const float Bv = myB[o], Cv = myC[o];
-                        const float duv = myDu[o];
-                        const float bu = Bv * duv;
+                        const float dov = aO[j];
+                        const float Bv = aB[j], Cv = aC[j];
+                        const float duv = aU[j];
+                        const float bu = buv[j];
                         const float dyC = dov * Cv;
                         const float a = arow[j];
                         const float g_ = fmaf(-0.5f * (arow[j + 1] + adn[j]), Gdiag, dyC + Gr + GdH[j]);

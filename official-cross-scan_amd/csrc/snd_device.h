@@ -47,6 +47,31 @@ __device__ __forceinline__ float ldg(const f16_t *base, int i) { return (float)b
 __device__ __forceinline__ void stg(float *base, int i, float v) { base[i] = v; }
 __device__ __forceinline__ void stg(bf16_t *base, int i, float v) { base[i].v = f32_to_bf16(v); }
 __device__ __forceinline__ void stg(f16_t *base, int i, float v) { base[i] = (f16_t)v; }
+// The same by byte offset from a block-uniform base pointer: base in scalar registers plus an
+// unsigned 32-bit per-lane offset is one address mode of the vector memory instructions, so no
+// 64-bit per-lane arithmetic is spent on addresses.  (The host entry points check that one batch
+// image of every tensor spans fewer than 2^32 bytes and that row pitches fit 24-bit multiplies.)
+__device__ __forceinline__ float ldg_b(const float *base, uint32_t off) { return *(const float *)((const char *)base + off); }
+__device__ __forceinline__ float ldg_b(const bf16_t *base, uint32_t off) { return bf16_to_f32(((const bf16_t *)((const char *)base + off))->v); }
+__device__ __forceinline__ float ldg_b(const f16_t *base, uint32_t off) { return (float)*(const f16_t *)((const char *)base + off); }
+__device__ __forceinline__ void stg_b(float *base, uint32_t off, float v) { *(float *)((char *)base + off) = v; }
+__device__ __forceinline__ void stg_b(bf16_t *base, uint32_t off, float v) { ((bf16_t *)((char *)base + off))->v = f32_to_bf16(v); }
+__device__ __forceinline__ void stg_b(f16_t *base, uint32_t off, float v) { *(f16_t *)((char *)base + off) = (f16_t)v; }
+__device__ __forceinline__ float ld_f32_b(const void *base, uint32_t off, int dt) {
+    const char *q = (const char *)base + off;
+    if (dt == SND_F32) return *(const float *)q;
+    if (dt == SND_BF16) return bf16_to_f32(*(const uint16_t *)q);
+    return (float)*(const f16_t *)q;
+}
+__device__ __forceinline__ void st_f32_b(void *base, uint32_t off, int dt, float v) {
+    char *q = (char *)base + off;
+    if (dt == SND_F32) *(float *)q = v;
+    else if (dt == SND_BF16) *(uint16_t *)q = f32_to_bf16(v);
+    else *(f16_t *)q = (f16_t)v;
+}
+// a*b + c with 24-bit a, b (full-rate multiply-add; 32-bit integer multiplies are quarter rate)
+__device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }
+
 // Same with the dtype chosen at run time (wave-uniform branch): used for out / dout, whose dtype
 // may differ from the inputs' (fp32 or the input dtype).
 __device__ __forceinline__ float ld_f32(const void *base, int i, int dt) {

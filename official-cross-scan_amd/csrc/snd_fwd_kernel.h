@@ -73,11 +73,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
-    // scan origin of this group: the scan runs in (i, j) from (0, 0); memory row = mrow(i), column =
-    // mcol(j).  Only the staging loads and the output stores know about it.
+    // scan origin of this group: the scan runs in (i, j) from (0, 0); memory row = mrow(i) = r0m + rs*i,
+    // memory column = mcol(j) = c0m + cs*j.  Only the staging loads and the output stores know about it.
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
-    auto mrow = [&](int r) { return fv ? H - 1 - r : r; };
-    auto mcol = [&](int c_) { return fh ? W - 1 - c_ : c_; };
+    const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1, c0m = fh ? W - 1 : 0, cs = fh ? -1 : 1;
+    auto mrow = [&](int r) { return mad24(r, rs, r0m); };
+    auto mcol = [&](int c_) { return mad24(c_, cs, c0m); };
 
     const int tid = threadIdx.x, wave = tid >> 6;
     const int n = tid % NP, cl = tid / NP;          // state and block-local channel of this lane
@@ -98,11 +99,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
     const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride;
     const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride;
-    const int esz_out = p.out_dtype == SND_F32 ? 4 : 2;
+    const int sh_out = p.out_dtype == SND_F32 ? 2 : 1, esz_out = 1 << sh_out;
     void *outb = (char *)p.out + (int64_t)b * p.out_batch_stride * esz_out;
-    const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
-    const int Bh = (int)p.B_h_stride, Ch = (int)p.C_h_stride, Uh = (int)p.u_h_stride, Dh = (int)p.delta_h_stride;
-    const int Bs = (int)p.B_dstate_stride, Cs = (int)p.C_dstate_stride, Oh = (int)p.out_h_stride;
+    // byte offsets inside the batch image: per-lane channel offsets (kept across the tile loop) and
+    // row pitches / state strides in bytes
+    constexpr int ESZ = (int)sizeof(T);
+    const uint32_t cUb = (uint32_t)cc * (uint32_t)p.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)p.delta_d_stride * ESZ;
+    const uint32_t cOb = (uint32_t)cc * (uint32_t)p.out_d_stride * esz_out;
+    const int BhB = (int)p.B_h_stride * ESZ, ChB = (int)p.C_h_stride * ESZ, UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ;
+    const int OhB = (int)p.out_h_stride * esz_out;
+    const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the wave index as a scalar
 
     // saved state, tile-major with the lane's 8 values innermost, so that each lane moves 32
     // contiguous bytes and a wave's 64 planes one contiguous 2 KB run:
@@ -132,17 +139,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
-        const int cU = cc * (int)p.u_d_stride, cD = (cc / rd) * (int)p.delta_d_stride;
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
-            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
-            const int ob = rc * Bh + cx, oc = rc * Ch + cx;
+            const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
+            const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
-                const int sn = wave + WPB * k, sc = min(sn, N - 1);
-                const float vb = ldg(Bb, sc * Bs + ob), vc = ldg(Cb, sc * Cs + oc);
+                const int sn = wave_u + WPB * k, sc = min(sn, N - 1);       // scalar: folded into the base
+                const float vb = ldg_b((const T *)((const char *)Bb + sc * BsB), ob);
+                const float vc = ldg_b((const T *)((const char *)Cb + sc * CsB), oc);
                 q.qb[k] = (in && sn < N) ? vb : 0.f;
                 q.qc[k] = (in && sn < N) ? vc : 0.f;
             }
@@ -152,15 +159,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
-            const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
+            const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
+            const float vd = ldg_b(db, cDb + mad24(mr, DhB, mcB)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mcB));
             q.qdl[k] = ok ? vd : 0.f;
             q.qu[k] = ok ? vu : 0.f;
         }
         q.qhalo = 0.f;
         if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
             const int row = r0 - 1, col = j0 + n;
-            const float vd = ldg(db, cD + mrow(max(row, 0)) * Dh + mcol(min(col, W - 1)));
+            const float vd = ldg_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
             q.qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
         }
     };
@@ -332,13 +339,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
 
             // ---- out = D*u + y, written by the thread that staged the pixel
             SND_THREAD_MAPS(NP);
-            const int cO = cc * (int)p.out_d_stride;
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                 if (cvalid && row < H && col < W)
-                    st_f32(outb, cO + mrow(row) * Oh + mcol(col), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                    st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
