@@ -107,10 +107,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G;
     const int cbase = g * rg + chunk * CB, cend = (g + 1) * rg;
-    // scan origin of this group (as in the forward): memory row = mrow(i), column = mcol(j)
+    // scan origin of this group (as in the forward): memory row = mrow(i) = r0m + rs*i, column = mcol(j)
     const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
-    auto mrow = [&](int r) { return fv ? H - 1 - r : r; };
-    auto mcol = [&](int c_) { return fh ? W - 1 - c_ : c_; };
+    const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1, c0m = fh ? W - 1 : 0, cs = fh ? -1 : 1;
+    auto mrow = [&](int r) { return mad24(r, rs, r0m); };
+    auto mcol = [&](int c_) { return mad24(c_, cs, c0m); };
 
     const int tid = threadIdx.x, wave = tid >> 6;
     const int n = tid % NP, cl = tid / NP;
@@ -132,15 +133,23 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
     const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride;
     const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride;
-    const int esz_do = p.dout_dtype == SND_F32 ? 4 : 2;
+    const int sh_do = p.dout_dtype == SND_F32 ? 2 : 1, esz_do = 1 << sh_do;
     const void *dob = (const char *)p.dout + (int64_t)b * p.dout_batch_stride * esz_do;
     T *dub = (T *)p.du + (int64_t)b * Dm * H * W;                    // du, ddelta: dense [b, c, H, W]
     T *ddb = (T *)p.ddelta + (int64_t)b * Dm * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;            // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
-    const int cU = cc * (int)f.u_d_stride, cD = (cc / rd) * (int)f.delta_d_stride, cDo = cc * (int)p.dout_d_stride;
-    const int Bh = (int)f.B_h_stride, Ch = (int)f.C_h_stride, Uh = (int)f.u_h_stride, Dh = (int)f.delta_h_stride;
-    const int Bs = (int)f.B_dstate_stride, Cs = (int)f.C_dstate_stride, Doh = (int)p.dout_h_stride;
+    // byte offsets inside the batch image: per-lane channel offsets (kept across the tile loop) and
+    // row pitches / state strides in bytes
+    constexpr int ESZ = (int)sizeof(T);
+    const uint32_t cUb = (uint32_t)cc * (uint32_t)f.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)f.delta_d_stride * ESZ;
+    const uint32_t cDob = ((uint32_t)cc * (uint32_t)p.dout_d_stride) << sh_do;
+    const uint32_t cGb = (uint32_t)cc * (uint32_t)(H * W) * ESZ;      // du, ddelta
+    const int BhB = (int)f.B_h_stride * ESZ, ChB = (int)f.C_h_stride * ESZ, UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ;
+    const int DohB = (int)p.dout_h_stride << sh_do, WB = W * ESZ, W4 = W * 4;
+    const int64_t BsB = f.B_dstate_stride * ESZ, CsB = f.C_dstate_stride * ESZ;
+    const int64_t HW4 = (int64_t)H * W * 4;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the wave index as a scalar
 
     // saved state and scratch, tile-major with the lane's 8 values innermost (as the forward writes):
     //   x_v [b][I][J][c][n][8 cols]   x, x_sd [b][J][I][c][n][8 rows]   scratch G row [b][J][c][n][8 cols]
@@ -167,18 +176,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
-        const int cU = cc * (int)f.u_d_stride, cD = (cc / rd) * (int)f.delta_d_stride;
-        const int cDo = cc * (int)p.dout_d_stride;
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
             const bool in = row < H && col < W;
-            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
-            const int ob = rc * Bh + cx, oc = rc * Ch + cx;
+            const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
+            const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
-                const int sn = wave + WPB * k, sc = min(sn, N - 1);
-                const float vb = ldg(Bb, sc * Bs + ob), vc = ldg(Cb, sc * Cs + oc);
+                const int sn = wave_u + WPB * k, sc = min(sn, N - 1);       // scalar: folded into the base
+                const float vb = ldg_b((const T *)((const char *)Bb + sc * BsB), ob);
+                const float vc = ldg_b((const T *)((const char *)Cb + sc * CsB), oc);
                 qb[k] = (in && sn < N) ? vb : 0.f;
                 qc[k] = (in && sn < N) ? vc : 0.f;
             }
@@ -188,9 +196,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && row < H && col < W;
-            const int rc = mrow(min(row, H - 1)), cx = mcol(min(col, W - 1));
-            const float vd = ldg(db, cD + rc * Dh + cx), vu = ldg(ub, cU + rc * Uh + cx);
-            const float vo = ld_f32(dob, cDo + rc * Doh + cx, p.dout_dtype);
+            const int mr = mrow(min(row, H - 1)), mc = mcol(min(col, W - 1));
+            const float vd = ldg_b(db, cDb + mad24(mr, DhB, mc * ESZ)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mc * ESZ));
+            const float vo = ld_f32_b(dob, cDob + mad24(mr, DohB, mc << sh_do), p.dout_dtype);
             qdl[k] = ok ? vd : 0.f;
             qu[k] = ok ? vu : 0.f;
             qdo[k] = ok ? vo : 0.f;
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             else { rr = hidx - 27; jj = 9; }
             const int row = r0 - 1 + rr, col = j0 - 1 + jj;
             const bool ok = cvalid && row >= 0 && row < H && col >= 0 && col < W;
-            const float vd = ldg(db, cD + mrow(min(max(row, 0), H - 1)) * Dh + mcol(min(max(col, 0), W - 1)));
+            const float vd = ldg_b(db, cDb + mad24(mrow(min(max(row, 0), H - 1)), DhB, mcol(min(max(col, 0), W - 1)) * ESZ));
             qh[k] = ok ? vd : 0.f;
         }
     };
@@ -492,7 +500,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
             {
             SND_THREAD_MAPS(NP);
-            const int cG = cc * H * W;
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
@@ -505,8 +512,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 dD_acc = fmaf(dov, uv, dD_acc);
                 dbias_acc += ddl;
                 if (cvalid && row < H && col < W) {
-                    stg(dub, cG + mrow(row) * W + mcol(col), duv);
-                    stg(ddb, cG + mrow(row) * W + mcol(col), ddl);
+                    const uint32_t o = cGb + mad24(mrow(row), WB, mcol(col) * ESZ);
+                    stg_b(dub, o, duv);
+                    stg_b(ddb, o, ddl);
                 }
             }
             }
@@ -515,9 +523,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 SND_THREAD_MAPS(NP);
                 const int row = r0 + pr, col = j0 + pj;
                 const bool in = row < H && col < W;
+                const uint32_t o = mad24(mrow(row), W4, mcol(col) * 4);
 #pragma unroll
                 for (int k = 0; k < NBC; ++k) {
-                    const int sn = wave + WPB * k;
+                    const int sn = wave_u + WPB * k;                        // scalar: folded into the base
                     float tb = 0.f, tc = 0.f;
 #pragma unroll
                     for (int w = 0; w < NPART; ++w) {
@@ -525,9 +534,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         tc += sdC[w * NP * NSTR + sn * NSTR + px];
                     }
                     if (in && sn < N) {
-                        const int o = (sn * H + mrow(row)) * W + mcol(col);
-                        glb_add(dBg + o, tb);
-                        glb_add(dCg + o, tc);
+                        glb_add((float *)((char *)dBg + sn * HW4 + o), tb);
+                        glb_add((float *)((char *)dCg + sn * HW4 + o), tc);
                     }
                 }
             }

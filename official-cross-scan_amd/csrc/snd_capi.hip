@@ -42,10 +42,14 @@ int check_shape(const snd_shape &s) {
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
-// The kernels address inside one batch image with 32-bit offsets.
-bool fits32(int64_t a_count, int64_t a_stride, int64_t b_count, int64_t b_stride, int64_t tail) {
-    if (a_stride < 0 || b_stride < 0) return false;
-    return (a_count - 1) * a_stride + (b_count - 1) * b_stride + tail < ((int64_t)1 << 31);
+// The kernels address inside one batch image with unsigned 32-bit BYTE offsets from a scalar base
+// and form row offsets with 24-bit multiplies: a (count x stride) walk plus rows must stay below
+// 2^32 bytes and a row pitch below 2^23 bytes.
+int esize(int dt) { return dt == SND_F32 ? 4 : 2; }
+bool fits32(int64_t a_count, int64_t a_stride, int64_t rows, int64_t h_stride, int64_t cols, int esz) {
+    if (a_stride < 0 || h_stride < 0) return false;
+    if (h_stride * esz >= ((int64_t)1 << 23) || rows >= ((int64_t)1 << 23) || cols >= ((int64_t)1 << 21)) return false;
+    return ((a_count - 1) * a_stride + (rows - 1) * h_stride + cols) * esz < ((int64_t)1 << 32);
 }
 
 int check_fwd(const snd_fwd_params &p, bool need_state) {
@@ -60,11 +64,12 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
         p.C_h_stride < p.shape.ncols)
         if (p.shape.nrows > 1) return SND_ERR_STRIDE;
     const snd_shape &s = p.shape;
-    if (!fits32(s.dim, p.u_d_stride, s.nrows, p.u_h_stride, s.ncols) ||
-        !fits32(s.delta_dim, p.delta_d_stride, s.nrows, p.delta_h_stride, s.ncols) ||
-        !fits32(s.dstate, p.B_dstate_stride, s.nrows, p.B_h_stride, s.ncols) ||
-        !fits32(s.dstate, p.C_dstate_stride, s.nrows, p.C_h_stride, s.ncols) ||
-        (int64_t)s.dim * s.nrows * s.ncols >= ((int64_t)1 << 31))
+    const int e = esize(s.in_dtype);
+    if (!fits32(s.dim, p.u_d_stride, s.nrows, p.u_h_stride, s.ncols, e) ||
+        !fits32(s.delta_dim, p.delta_d_stride, s.nrows, p.delta_h_stride, s.ncols, e) ||
+        !fits32(1, 0, s.nrows, p.B_h_stride, s.ncols, e) || p.B_dstate_stride < 0 ||
+        !fits32(1, 0, s.nrows, p.C_h_stride, s.ncols, e) || p.C_dstate_stride < 0 ||
+        !fits32(s.dim, (int64_t)s.nrows * s.ncols, s.nrows, s.ncols, s.ncols, 4))      // dense per-image gradients
         return SND_ERR_STRIDE;
     return SND_OK;
 }
@@ -81,7 +86,7 @@ const char *snd_status_string(int status) {
         case SND_ERR_NULL: return "a required pointer is null";
         case SND_ERR_SHAPE: return "bad shape: need dim % n_groups == 0, dim % delta_dim == 0, 1 <= dstate <= 16, all sizes > 0";
         case SND_ERR_DTYPE: return "unsupported dtype combination (inputs fp32/fp16/bf16; out and dout fp32 or the input dtype)";
-        case SND_ERR_STRIDE: return "bad stride: rows must not overlap, the last dimension must be contiguous and one batch image must span fewer than 2^31 elements";
+        case SND_ERR_STRIDE: return "bad stride: rows must not overlap, the last dimension must be contiguous, one batch image must span fewer than 2^32 bytes and a row pitch fewer than 2^23 bytes";
         case SND_ERR_LAUNCH: return "kernel launch failed";
         case SND_ERR_WORKSPACE: return "saved state (x, x_v, x_sd) or workspace missing or too small";
         case SND_ERR_ALIGN: return "saved state / workspace pointers must be 16-byte aligned";
@@ -116,7 +121,8 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->out) return SND_ERR_NULL;
     if (params->out_dtype != SND_F32 && params->out_dtype != params->shape.in_dtype) return SND_ERR_DTYPE;
-    if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols))
+    if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols,
+                esize(params->out_dtype)))
         return SND_ERR_STRIDE;
     if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
     if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
@@ -153,7 +159,7 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
     if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
     if (params->f.directions != SND_DIR_TOPLEFT && params->f.directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
-                params->f.shape.ncols))
+                params->f.shape.ncols, esize(params->dout_dtype)))
         return SND_ERR_STRIDE;
     switch (params->f.shape.in_dtype) {
         case SND_F32: return snd::launch_bwd_f32(*params, (hipStream_t)stream);

@@ -90,6 +90,32 @@ def test_entry_points_validate_before_touching_the_gpu():
     assert b"16-byte" in lib.snd_status_string(-7)
 
 
+def test_address_range_limits_are_status_codes():
+    """The kernels use unsigned 32-bit byte offsets inside a batch image and 24-bit row-pitch
+    multiplies; shapes or strides beyond that are refused before anything is launched."""
+    lib = capi.lib()
+
+    def params(H=4, W=4, dim=8, **strides):
+        fp = capi.FwdParams()
+        fp.shape = capi.Shape(1, dim, H, W, 16, 4, dim, capi.SND_F32)
+        fp.u = fp.delta = fp.A = fp.B = fp.C = fp.x_v = fp.out = 16
+        fp.u_h_stride = fp.delta_h_stride = fp.B_h_stride = fp.C_h_stride = fp.out_h_stride = W
+        fp.u_d_stride = fp.delta_d_stride = fp.out_d_stride = H * W
+        fp.B_dstate_stride = fp.C_dstate_stride = H * W
+        for k, v in strides.items():
+            setattr(fp, k, v)
+        return fp
+
+    assert lib.snd_fwd(C.byref(params(schedule=3)), None) == -2                  # unknown schedule
+    assert lib.snd_fwd(C.byref(params(directions=2)), None) == -2                # unknown directions
+    assert lib.snd_fwd(C.byref(params(u_h_stride=2)), None) == -4                # rows overlap
+    assert lib.snd_fwd(C.byref(params(u_h_stride=1 << 21)), None) == -4          # row pitch >= 2^23 bytes
+    assert lib.snd_fwd(C.byref(params(u_d_stride=1 << 28)), None) == -4          # image >= 2^32 bytes
+    assert lib.snd_fwd(C.byref(params(out_d_stride=-1)), None) == -4             # negative stride
+    assert lib.snd_fwd(C.byref(params(H=1 << 15, W=1 << 15, dim=8)), None) == -4  # dense gradients >= 2^32 bytes
+    assert b"2^32" in lib.snd_status_string(-4)
+
+
 def test_python_operator_has_no_cpu_fallback():
     torch = pytest.importorskip("torch")
     import selective_nd_scan as s
