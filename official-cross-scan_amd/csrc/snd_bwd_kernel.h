@@ -83,6 +83,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     int *sync = (int *)p.workspace, *progress = nullptr;
     const int64_t nSync = sync_words((int64_t)sh.batch * G * nChunks, geo.nCY);
     bool dead = false;
+    int seen = 0;                                   // last progress count read (strip pipeline)
 #ifdef SND_PIPE_TRACE
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             commit();
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
-            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, sync, dead SND_TRACE_PASS);
+            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
             __syncthreads();
 
             // ---- checkpoints and carried adjoints of this tile

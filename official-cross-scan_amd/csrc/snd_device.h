@@ -230,15 +230,17 @@ __device__ __forceinline__ void strip_signal(int *count) {
 #define SND_TRACE_ARG
 #define SND_TRACE_PASS
 #endif
-// Wait until *count >= need.  Bounded: after kSpinLimit polls the error word is set and the wave
-// goes on (with wrong data) so that the grid always drains; `dead` then disables further waits.
-__device__ __forceinline__ void strip_wait(const int *count, int need, int *sync, bool &dead SND_TRACE_ARG) {
-    if (dead) return;
+// Wait until *count >= need.  `seen` caches the last value read (counts only grow), so a consumer
+// that runs well behind its producer polls once per strip, not once per tile.  Bounded: after
+// kSpinLimit polls the error word is set and the wave goes on (with wrong data) so that the grid
+// always drains; `dead` then disables further waits.
+__device__ __forceinline__ void strip_wait(const int *count, int need, int &seen, int *sync, bool &dead SND_TRACE_ARG) {
+    if (dead || seen >= need) return;
 #ifdef SND_PIPE_TRACE
     const long long t0_ = wall_clock64();
 #endif
     int polls = 0;
-    while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+    while ((seen = __hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) < need) {
         __builtin_amdgcn_s_sleep(SND_POLL_SLEEP);
         if (++polls > kSpinLimit) {
             dead = true;

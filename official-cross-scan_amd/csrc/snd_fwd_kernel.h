@@ -49,6 +49,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     int I_begin = 0, I_end = geo.nCY;               // strips this block walks
     int *sync = (int *)p.workspace, *progress = nullptr;
     bool dead = false;
+    int seen = 0;                                   // last progress count read (strip pipeline)
 #ifdef SND_PIPE_TRACE
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         auto do_tile = [&](const int J, const Stage &mine, const bool last_of_pair) {
             const int j0 = J * kCkX;
             commit(mine);
-            if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, sync, dead SND_TRACE_PASS);
+            if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
             __syncthreads();
             // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
             // registers), handed over in registers, or - strip pipeline - fetched here
