@@ -6,3 +6,6 @@ from .cross_scan import (cross_merge, cross_scan, cross_scan_2d, four_corner_sca
                          four_corner_scan_by_flips)
 
 __all__ += ["cross_scan", "cross_merge", "cross_scan_2d", "four_corner_scan", "four_corner_scan_by_flips"]
+from .vss_block import SS2DCrossScan, VSSBlock  # noqa: F401,E402
+
+__all__ += ["SS2DCrossScan", "VSSBlock"]
