@@ -35,13 +35,31 @@ __device__ __forceinline__ void glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// v_permlane32_swap: upper 32 lanes of a <-> lower 32 lanes of b.  v_permlane16_swap: odd 16-lane
-// rows of a <-> even rows of b.  After either swap, a + b is the pair-sum of the value the lane keeps.
-__device__ __forceinline__ void swap32(float &a, float &b) {
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-__device__ __forceinline__ void swap16(float &a, float &b) {
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+// Sum two sets of four values over the four 16-lane rows of a wave (its four channels when a row
+// holds the 16 states of one channel): a reduce-scatter, row q of the wave ends with the totals of
+// b[q] (in b0) and c[q] (in c0).  v_permlane32_swap exchanges the upper 32 lanes of its first
+// operand with the lower 32 lanes of its second, v_permlane16_swap the odd 16-lane rows of the first
+// with the even rows of the second; after either, first + second is the pair-sum of the value the
+// lane keeps.  A swap must not read a register written by the two preceding VALU instructions and
+// its results must not be read by the two following ones: the order and the s_nops keep that distance.
+__device__ __forceinline__ void rows_scatter4x2(float &b0, float &b1, float &b2, float &b3, float &c0, float &c1,
+                                                float &c2, float &c3) {
+    asm volatile("s_nop 1\n\t"
+                 "v_permlane32_swap_b32 %0, %2\n\t"
+                 "v_permlane32_swap_b32 %1, %3\n\t"
+                 "v_permlane32_swap_b32 %4, %6\n\t"
+                 "v_permlane32_swap_b32 %5, %7\n\t"
+                 "v_add_f32 %0, %0, %2\n\t"
+                 "v_add_f32 %1, %1, %3\n\t"
+                 "v_add_f32 %4, %4, %6\n\t"
+                 "v_add_f32 %5, %5, %7\n\t"
+                 "s_nop 0\n\t"
+                 "v_permlane16_swap_b32 %0, %1\n\t"
+                 "v_permlane16_swap_b32 %4, %5\n\t"
+                 "s_nop 1\n\t"
+                 "v_add_f32 %0, %0, %1\n\t"
+                 "v_add_f32 %4, %4, %5\n\t"
+                 : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(c0), "+v"(c1), "+v"(c2), "+v"(c3));
 }
 #ifndef SND_BWD_WAVES
 #define SND_BWD_WAVES 2
@@ -450,15 +468,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     {
                         // sum over the wave's channels: lane bits 4-5 by a swap reduce-scatter (the
                         // 16-lane row q ends with column C0+q), bit 3 (8-state layout) by a row rotate
-                        float b0 = vB[0], b2 = vB[2], b1 = vB[1], b3 = vB[3];
-                        swap32(b0, b2); swap32(b1, b3);
-                        float tb0 = b0 + b2, tb1 = b1 + b3;
-                        swap16(tb0, tb1);
-                        float c0 = vC[0], c2 = vC[2], c1 = vC[1], c3 = vC[3];
-                        swap32(c0, c2); swap32(c1, c3);
-                        float tc0 = c0 + c2, tc1 = c1 + c3;
-                        swap16(tc0, tc1);
-                        float tb = tb0 + tb1, tc = tc0 + tc1;
+                        rows_scatter4x2(vB[0], vB[1], vB[2], vB[3], vC[0], vC[1], vC[2], vC[3]);
+                        float tb = vB[0], tc = vC[0];
                         if (NP == 8) { tb += dpp_mov<0x128>(tb); tc += dpp_mov<0x128>(tc); }   // row_ror:8
                         if (NP == 16 || (tid & 8) == 0) {
                             mydB[r * kCkX + C0 + qrow] = tb;
