@@ -281,9 +281,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     for (int I = I_hi; I >= I_lo; --I) {
         const int r0 = I * kRows;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
+        float aR[kRows];                            // a at that column (only ever multiplies G there)
         float GRc = 0.f;                            // G[r0+8][j0+8]
 #pragma unroll
-        for (int r = 0; r < kRows; ++r) { GR[r] = 0.f; GsR[r] = 0.f; }
+        for (int r = 0; r < kRows; ++r) { GR[r] = 0.f; GsR[r] = 0.f; aR[r] = 0.f; }
 
         for (int J = geo.nCX - 1; J >= 0; --J) {
             const int j0 = J * kCkX;
@@ -405,7 +406,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     __builtin_amdgcn_sched_barrier(0);
                     float arow[5], s[4], buv[4];
 #pragma unroll
-                    for (int j = 0; j <= 4; ++j) arow[j] = AEXP(r, C0 + j);
+                    for (int j = 0; j < 4; ++j) arow[j] = AEXP(r, C0 + j);
+                    arow[4] = aR[r];
                     const float4 vB4 = *(const float4 *)(myB + r * kCkX + C0), vC4 = *(const float4 *)(myC + r * kCkX + C0);
                     const float4 vU4 = *(const float4 *)(myDu + r * kCkX + C0), vO4 = *(const float4 *)(myDo + r * kCkX + C0);
                     const float aB[4] = {vB4.x, vB4.y, vB4.z, vB4.w}, aC[4] = {vC4.x, vC4.y, vC4.z, vC4.w};
@@ -479,6 +481,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     Gd8 = GR[r];                    // G[r][C0+4]: diagonal neighbour for the row above
                     GR[r] = Gr;                     // G[r][C0]: right neighbour for the half on the left
                     GsR[r] = Gsr;
+                    aR[r] = arow[0];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) adn[j] = arow[j];
                 }
