@@ -115,6 +115,12 @@ typedef struct snd_fwd_params {
     int64_t workspace_bytes;
     int32_t schedule;              /* snd_schedule, for fwd and (through snd_bwd_params.f) for bwd */
     int32_t directions;            /* snd_directions, for fwd and (through snd_bwd_params.f) for bwd */
+    int32_t u_shared;              /* 0: u is [batch, dim, nrows, ncols] (the reference's layout).
+                                      1: u is [batch, dim / n_groups, nrows, ncols] and every group scans
+                                      the same channels (channel g*(dim/n_groups) + i reads u channel i):
+                                      the CrossScan of one feature map without its n_groups copies.
+                                      out, du and every other tensor keep their dim-wide layouts. */
+    int32_t reserved_;             /* set to 0 */
 } snd_fwd_params;
 
 /* Replaces SSMParamsBwd (selective_scan_oflex.h:53-86). Gradient buffers are dense (contiguous):

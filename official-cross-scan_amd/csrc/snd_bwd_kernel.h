@@ -161,7 +161,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // byte offsets inside the batch image: per-lane channel offsets (kept across the tile loop) and
     // row pitches / state strides in bytes
     constexpr int ESZ = (int)sizeof(T);
-    const uint32_t cUb = (uint32_t)cc * (uint32_t)f.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)f.delta_d_stride * ESZ;
+    const uint32_t cUb = (uint32_t)(f.u_shared ? cc - g * rg : cc) * (uint32_t)f.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)f.delta_d_stride * ESZ;
     const uint32_t cDob = ((uint32_t)cc * (uint32_t)p.dout_d_stride) << sh_do;
     const uint32_t cGb = (uint32_t)cc * (uint32_t)(H * W) * ESZ;      // du, ddelta
     const int BhB = (int)f.B_h_stride * ESZ, ChB = (int)f.C_h_stride * ESZ, UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ;

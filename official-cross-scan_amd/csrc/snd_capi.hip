@@ -65,7 +65,8 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
         if (p.shape.nrows > 1) return SND_ERR_STRIDE;
     const snd_shape &s = p.shape;
     const int e = esize(s.in_dtype);
-    if (!fits32(s.dim, p.u_d_stride, s.nrows, p.u_h_stride, s.ncols, e) ||
+    if ((p.u_shared != 0 && p.u_shared != 1) ||
+        !fits32(p.u_shared ? s.dim / s.n_groups : s.dim, p.u_d_stride, s.nrows, p.u_h_stride, s.ncols, e) ||
         !fits32(s.delta_dim, p.delta_d_stride, s.nrows, p.delta_h_stride, s.ncols, e) ||
         !fits32(1, 0, s.nrows, p.B_h_stride, s.ncols, e) || p.B_dstate_stride < 0 ||
         !fits32(1, 0, s.nrows, p.C_h_stride, s.ncols, e) || p.C_dstate_stride < 0 ||
@@ -78,7 +79,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 102; }
+int snd_version(void) { return 103; }
 
 const char *snd_status_string(int status) {
     switch (status) {

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     // byte offsets inside the batch image: per-lane channel offsets (kept across the tile loop) and
     // row pitches / state strides in bytes
     constexpr int ESZ = (int)sizeof(T);
-    const uint32_t cUb = (uint32_t)cc * (uint32_t)p.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)p.delta_d_stride * ESZ;
+    const uint32_t cUb = (uint32_t)(p.u_shared ? cc - g * rg : cc) * (uint32_t)p.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)p.delta_d_stride * ESZ;
     const uint32_t cOb = (uint32_t)cc * (uint32_t)p.out_d_stride * esz_out;
     const int BhB = (int)p.B_h_stride * ESZ, ChB = (int)p.C_h_stride * ESZ, UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ;
     const int OhB = (int)p.out_h_stride * esz_out;

@@ -37,6 +37,7 @@ void check_status(int st, const char *what) {
 
 struct Checked {
     int batch, dim, nrows, ncols, dstate, n_groups, delta_dim;
+    bool u_shared;                 // u is [batch, dim / n_groups, H, W]: one feature map scanned by every group
     snd_shape shape;
     snd_plan plan;
 };
@@ -59,14 +60,19 @@ Checked check_inputs(const at::Tensor &u, const at::Tensor &delta, const at::Ten
     TORCH_CHECK(delta.stride(-1) == 1 || delta.size(-1) == 1, "delta must be contiguous in its last dimension");
 
     Checked c;
-    c.batch = u.size(0); c.dim = u.size(1); c.nrows = u.size(2); c.ncols = u.size(3);
+    // dim is A's (the reference takes it from u, selective_scan_oflex.cpp:206): u may carry only
+    // dim / n_groups channels, shared by all groups (the CrossScan of one feature map without copies)
+    c.batch = u.size(0); c.dim = A.size(0); c.nrows = u.size(2); c.ncols = u.size(3);
     c.dstate = A.size(1); c.n_groups = B.size(1); c.delta_dim = delta.size(1);
+    c.u_shared = u.size(1) != c.dim;
+    TORCH_CHECK(!c.u_shared || u.size(1) * c.n_groups == c.dim,
+                "u must have dim = A.size(0) channels, or dim / n_groups channels shared by the groups");
     TORCH_CHECK(c.dim % c.n_groups == 0, "dims should be dividable by n_groups");
     TORCH_CHECK(c.dim % c.delta_dim == 0, "dims should be dividable by delta_dim");
     TORCH_CHECK(c.dstate <= SND_MAX_DSTATE, "selective_scan only supports state dimension <= 16");
     const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate,
               n_groups = c.n_groups, delta_dim = c.delta_dim;
-    CHECK_SHAPE(u, batch_size, dim, nrows, ncols);
+    CHECK_SHAPE(u, batch_size, c.u_shared ? dim / n_groups : dim, nrows, ncols);
     CHECK_SHAPE(delta, batch_size, delta_dim, nrows, ncols);
     CHECK_SHAPE(A, dim, dstate);
     CHECK_SHAPE(B, batch_size, n_groups, dstate, nrows, ncols);
@@ -104,6 +110,7 @@ void fill_fwd(snd_fwd_params &p, const Checked &c, const at::Tensor &u, const at
               bool delta_softplus) {
     memset(&p, 0, sizeof(p));
     p.shape = c.shape;
+    p.u_shared = c.u_shared ? 1 : 0;
     p.delta_softplus = delta_softplus ? 1 : 0;
     p.u = u.data_ptr(); p.delta = delta.data_ptr(); p.B = B.data_ptr(); p.C = C.data_ptr();
     p.A = A.data_ptr<float>();
@@ -218,6 +225,8 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
         result[1] = ddelta.view({batch_size, c.delta_dim, rep, nrows, ncols}).sum(2);
         if (delta_bias_.has_value()) result[6] = ddelta_bias.view({c.delta_dim, rep}).sum(1);
     }
+    if (c.u_shared)   // one feature map scanned by every group: its gradient is the sum over the groups
+        result[0] = du.view({batch_size, c.n_groups, dim / c.n_groups, nrows, ncols}).sum(1);
     return result;
 }
 

@@ -38,7 +38,7 @@ class FwdParams(C.Structure):
                                     "B_batch_stride", "B_group_stride", "B_dstate_stride", "B_h_stride",
                                     "C_batch_stride", "C_group_stride", "C_dstate_stride", "C_h_stride",
                                     "out_batch_stride", "out_d_stride", "out_h_stride")] +
-                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("directions", i32)])
+                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("directions", i32), ("u_shared", i32), ("reserved_", i32)])
 
 
 class BwdParams(C.Structure):
@@ -79,7 +79,8 @@ def _dt(t):
 
 
 def make_shape(u, delta, A, B):
-    return Shape(u.shape[0], u.shape[1], u.shape[2], u.shape[3], A.shape[1], B.shape[1], delta.shape[1], _dt(u))
+    """dim comes from A: u may be [batch, dim / n_groups, H, W] (shared by the groups, u_shared)."""
+    return Shape(u.shape[0], A.shape[0], u.shape[2], u.shape[3], A.shape[1], B.shape[1], delta.shape[1], _dt(u))
 
 
 def make_plan(shape):
@@ -97,6 +98,7 @@ def _fill_fwd(fp, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_de
     fp.shape = shape
     fp.schedule = schedule
     fp.directions = directions
+    fp.u_shared = int(u.shape[1] != A.shape[0])
     fp.out_dtype = _dt(out) if out is not None else SND_F32
     fp.delta_softplus = int(bool(delta_softplus))
     fp.u, fp.delta, fp.B, fp.C, fp.A = _ptr(u), _ptr(delta), _ptr(B), _ptr(Cc), _ptr(A)
@@ -132,9 +134,9 @@ class FwdCall:
         st, plan = make_plan(shape)
         check(st)
         self.plan = plan
-        Bt, Dm, N = u.shape[0], u.shape[1], A.shape[1]
+        Bt, Dm, N = u.shape[0], A.shape[0], A.shape[1]
         f32 = dict(device=u.device, dtype=torch.float32)
-        self.out = torch.empty(u.shape, device=u.device, dtype=torch.float32 if out_float else u.dtype)
+        self.out = torch.empty((Bt, Dm, u.shape[2], u.shape[3]), device=u.device, dtype=torch.float32 if out_float else u.dtype)
         self.x_v = torch.empty((Bt, Dm, N, plan.n_chunks_y, plan.xv_inner), **f32)
         self.x = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
@@ -160,9 +162,10 @@ class BwdCall:
         shape = make_shape(u, delta, A, B)
         st, plan = make_plan(shape)
         check(st)
-        Dm = u.shape[1]
+        Dm = A.shape[0]
         f32 = dict(device=u.device, dtype=torch.float32)
-        self.du, self.ddelta = torch.empty_like(u), torch.empty_like(u)
+        self.du = torch.empty((u.shape[0], Dm, u.shape[2], u.shape[3]), device=u.device, dtype=u.dtype)
+        self.ddelta = torch.empty_like(self.du)
         self.dA = torch.zeros_like(A)
         self.dB, self.dC = torch.zeros(B.shape, **f32), torch.zeros(Cc.shape, **f32)
         self.dD = torch.zeros_like(D) if D is not None else None
@@ -206,11 +209,14 @@ def bwd(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay
     call = BwdCall(u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, schedule,
                    directions)
     call.launch_kernel_only(stream)
-    Bt, Dm, H, W = u.shape
-    Dd = delta.shape[1]
+    Bt, _, H, W = u.shape
+    Dm, Dd = A.shape[0], delta.shape[1]
     ddelta, dbias = call.ddelta, call.dbias
+    du = call.du
+    if u.shape[1] != Dm:                         # u shared by the groups: its gradient is the sum over them
+        du = du.view(Bt, Dm // u.shape[1], u.shape[1], H, W).sum(1)
     if Dd != Dm:
         ddelta = ddelta.view(Bt, Dd, Dm // Dd, H, W).sum(2)
         if dbias is not None:
             dbias = dbias.view(Dd, Dm // Dd).sum(1)
-    return call.du, ddelta, call.dA, call.dB.to(B.dtype), call.dC.to(Cc.dtype), call.dD, dbias, call.ddec
+    return du, ddelta, call.dA, call.dB.to(B.dtype), call.dC.to(Cc.dtype), call.dD, dbias, call.ddec

@@ -56,7 +56,8 @@ def cross_merge(y, weights=None):
 def four_corner_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
                      A_decay=None):
     """u, delta [B, G*r, H, W], B, C [B, G, N, H, W] in natural orientation; group g is scanned from
-    corner g % 4 by the kernels.  Returns out [B, G*r, H, W] in natural orientation."""
+    corner g % 4 by the kernels.  u may also be [B, r, H, W]: one feature map shared by the G groups.
+    Returns out [B, G*r, H, W] in natural orientation."""
     return selective_nd_scan(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions=1)
 
 
@@ -64,6 +65,8 @@ def four_corner_scan_by_flips(u, delta, A, B, C, D=None, delta_bias=None, delta_
                               A_decay=None):
     """Same result through flipped copies and the top-left-only op (how the reference op is used)."""
     G = B.shape[1]
+    if u.shape[1] != A.shape[0]:
+        u = u.repeat(1, G, 1, 1)
     out = selective_nd_scan(flip_groups(u, G), flip_groups(delta, G) if delta.shape[1] % G == 0 else delta, A,
                             flip_groups(B, G), flip_groups(C, G), D, delta_bias, delta_softplus, out_float, A_decay)
     return flip_groups(out, G)
@@ -73,6 +76,7 @@ def cross_scan_2d(x, delta, A, B, C, D=None, delta_bias=None, delta_softplus=Tru
                   A_decay=None):
     """The block's scan stage: x [B, C, H, W] is scanned from the four corners (delta [B, 4*C, H, W],
     A [4*C, N], B, C [B, 4, N, H, W], D, delta_bias [4*C] are per direction) and the four results are
-    fused into [B, C, H, W] (fp32)."""
-    y = four_corner_scan(cross_scan(x), delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay)
+    fused into [B, C, H, W] (fp32).  x is passed as it is: the kernels let every direction group read
+    the same C channels (u with dim / n_groups channels), so not even cross_scan's copies are made."""
+    y = four_corner_scan(x, delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay)
     return cross_merge(y, merge_weights)

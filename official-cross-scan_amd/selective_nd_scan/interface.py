@@ -8,7 +8,7 @@ order of those bindings (selective_scan_oflex.cpp:179-187).
     out = selective_nd_scan(u, delta, A, B, C, D=None, delta_bias=None,
                             delta_softplus=False, out_float=True, A_decay=None)
 
-    u      [B, D, H, W]        fp32 / fp16 / bf16
+    u      [B, D, H, W]        fp32 / fp16 / bf16   (or [B, D/G, H, W]: one map shared by the G groups)
     delta  [B, Dd, H, W]       same dtype, D % Dd == 0
     A      [D, N]              fp32, N <= 16
     B, C   [B, G, N, H, W]     same dtype as u, D % G == 0

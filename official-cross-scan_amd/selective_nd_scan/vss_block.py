@@ -11,7 +11,8 @@ follows the upstream VMamba SS2D layout of that caller so the op can be dropped 
       -> fuse the four results with trainable weights (README.md:45) -> LayerNorm -> * SiLU(z) -> out_proj
 
 Because the scan origins are handled inside the kernels, every tensor stays in its natural
-orientation: the projections are pointwise, so no flipped copy of the feature map is ever built.
+orientation: the projections are pointwise, so no flipped (or even repeated) copy of the feature
+map is ever built - the four direction groups read the same u.
 Everything outside the scan is plain PyTorch (GEMMs / elementwise); `scan_fn` can be replaced for
 testing.
 """
@@ -21,7 +22,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .cross_scan import cross_merge, cross_scan, four_corner_scan
+from .cross_scan import cross_merge, four_corner_scan
 
 
 class SS2DCrossScan(nn.Module):
@@ -58,7 +59,7 @@ class SS2DCrossScan(nn.Module):
         dts, Bs, Cs = torch.split(x_dbl, [R, N, N], dim=2)
         delta = torch.einsum("bkrhw,kdr->bkdhw", dts, self.dt_projs_weight.to(x.dtype)).reshape(Bt, K * Di, H, W)
         A = -torch.exp(self.A_logs.float())
-        return (cross_scan(x), delta.contiguous(), A, Bs.contiguous(), Cs.contiguous(), self.Ds.float(),
+        return (x, delta.contiguous(), A, Bs.contiguous(), Cs.contiguous(), self.Ds.float(),
                 self.dt_projs_bias.float().reshape(-1))
 
     def forward(self, x):

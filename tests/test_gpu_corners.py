@@ -88,3 +88,28 @@ def test_four_corner_block_in_kernel_equals_flipped_copies(gpu_device):
     assert relerr(y1.detach().cpu().numpy(), y2.detach().cpu().numpy()) <= 1e-5
     for a, b_ in zip(g1, g2):
         assert relerr(a.float().cpu().numpy(), b_.float().cpu().numpy()) <= 2e-2, relerr(a.float().cpu().numpy(), b_.float().cpu().numpy())
+
+
+@pytest.mark.parametrize("dirs", [capi.DIR_TOPLEFT, capi.DIR_CORNERS])
+def test_u_shared_by_the_groups_equals_repeated_u(gpu_device, dirs):
+    """u with dim / n_groups channels (one feature map scanned by every group) against the same
+    call on u repeated per group: identical out and gradients, du summed over the groups."""
+    Bt, r, H, W, N, K = 2, 12, 23, 18, 16, 4
+    d = O.make_inputs(Bt, K * r, H, W, N=N, K=K, seed=31)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    x = t["u"][:, :r].contiguous()
+    rest = (t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+    res = []
+    for u in (x, x.repeat(1, K, 1, 1)):
+        f = capi.FwdCall(u, *rest, True, True, None, True, capi.SCHED_AUTO, dirs)
+        f.launch()
+        g = capi.bwd(u, *rest, t["dout"], f.x, f.x_v, True, None, f.x_sd, None, capi.SCHED_AUTO, dirs)
+        torch.cuda.synchronize()
+        res.append((f.out, g))
+    (out_s, g_s), (out_r, g_r) = res
+    assert out_s.shape == (Bt, K * r, H, W) and torch.equal(out_s, out_r)
+    assert g_s[0].shape == x.shape
+    assert relerr(g_s[0].cpu().numpy(), g_r[0].view(Bt, K, r, H, W).sum(1).cpu().numpy()) <= 1e-6
+    assert torch.equal(g_s[1], g_r[1])
+    for a, b_ in zip(g_s[2:7], g_r[2:7]):
+        assert relerr(a.cpu().numpy(), b_.cpu().numpy()) <= 1e-5      # atomic sums: order may differ

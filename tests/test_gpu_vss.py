@@ -15,6 +15,8 @@ def torch_four_corner_scan(u, delta, A, B, C, D, delta_bias, delta_softplus, out
     import importlib
     cs = importlib.import_module("selective_nd_scan.cross_scan")
     G = B.shape[1]
+    if u.shape[1] != A.shape[0]:
+        u = u.repeat(1, G, 1, 1)
     f64 = lambda t: t.double().cpu()
     out = selective_nd_scan_torch(f64(cs.flip_groups(u, G)), f64(cs.flip_groups(delta, G)), f64(A), f64(cs.flip_groups(B, G)),
                                   f64(cs.flip_groups(C, G)), f64(D), f64(delta_bias), delta_softplus)

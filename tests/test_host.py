@@ -22,7 +22,7 @@ def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
     assert C.sizeof(capi.Plan) == 56
-    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 8
+    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4
     assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8
 
 
@@ -30,7 +30,7 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
     probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes"]),
-              ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule"]),
+              ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared"]),
               ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
     for cname, _, fields in probes:
