@@ -17,12 +17,12 @@
 //
 // Organisation (not a translation): the same lane = one (channel, state) plane, 8x8 tile walk as the
 // forward, in reverse.  For each tile a lane recomputes h from the forward's checkpoints (row above
-// from x_v, column to the left from x, s from x_sd) into 64 registers, then sweeps the tile
-// bottom-right to top-left.  The adjoint row handed to the strip above goes through a private
-// global scratch row; the column handed to the tile on the left stays in registers.  dB/dC are
-// reduced over a wave's channels with lane swaps, over the block's waves through LDS, and leave
-// the block once per tile;
-// du/ddelta are reduced over states by DPP and finished once per pixel by the thread that staged it.
+// from x_v, column to the left from x, s from x_sd), one 8x4 half of the tile at a time into 32
+// registers, and sweeps that half bottom-right to top-left.  The adjoint row handed to the strip
+// above goes through a private global scratch row; the column handed to the tile on the left stays
+// in registers.  dB/dC are reduced over a wave's channels with lane swaps, over the block's waves
+// through LDS, and leave the block once per tile; du/ddelta are reduced over states by DPP and
+// finished once per pixel by the thread that staged it.
 // As in the forward, tiles are computed in full on zero-padded staging (dout = B = C = 0 outside
 // the plane makes every adjoint there exactly zero), so the inner loops have no bounds checks.
 #pragma once
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float *mydC = sdC + wave * NP * NSTR + n * NSTR;
     const int qrow = (tid & 63) >> 4;               // 16-lane row of this lane inside its wave
 
-    // ---- register staging of one tile's raw inputs (global loads issued one tile ahead)
+    // ---- register staging of one tile's raw inputs (loaded at the start of the tile, then committed to LDS)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
         const int r0 = I * kRows, j0 = J * kCkX;
@@ -275,9 +275,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float dA_acc = 0.f, dec_acc = 0.f;              // per lane: sum delta'*da*a, sum da*a
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
 
-#ifdef SND_BWD_PREFETCH
-    prefetch(I_hi, geo.nCX - 1);
-#endif
     for (int I = I_hi; I >= I_lo; --I) {
         const int r0 = I * kRows;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
@@ -288,9 +285,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 
         for (int J = geo.nCX - 1; J >= 0; --J) {
             const int j0 = J * kCkX;
-#ifndef SND_BWD_PREFETCH
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
-#endif
             commit();
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
@@ -503,14 +498,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             if (PIPE && I > 0) strip_stores_done();
             __syncthreads();
             if (PIPE && I > 0) strip_signal(progress + I);   // tile J is handed over to the strip above
-#ifdef SND_BWD_PREFETCH
-            {   // the next tile's loads are issued here, after the register-hungry sweep, and complete
-                // under the per-pixel epilogue below and under the other resident block's compute
-                int In = I, Jn = J - 1;
-                if (Jn < 0) { Jn = geo.nCX - 1; In = I - 1; }
-                if (In >= I_lo) prefetch(In, Jn);
-            }
-#endif
 
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
             {
