@@ -70,7 +70,10 @@ typedef struct snd_plan {
     int64_t x_elems, x_sd_elems, x_v_elems;    /* fp32 element counts of the three tensors */
     int64_t bwd_workspace_bytes;               /* scratch bwd needs (16-byte aligned, uninitialised) */
     int64_t fwd_workspace_bytes;               /* scratch fwd uses when it splits planes into strips
-                                                  (16-byte aligned, uninitialised; a few KB) */
+                                                  (16-byte aligned, uninitialised; one row per plane) */
+    int32_t auto_schedule;                     /* what SND_SCHED_AUTO resolves to for this shape (PLANE or
+                                                  STRIPS): a caller may skip the fwd workspace for PLANE */
+    int32_t reserved_;
 } snd_plan;
 
 /* How a launch maps work to blocks.  The reference has one fixed mapping (one block per

@@ -177,7 +177,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
     const float *xh = f.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
     const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
-    float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + lane_off;
+    // whole-plane schedule: [J][c][n][8 cols]; strip schedule: [J][pair k][c][n][2], so that a wave's
+    // 8-byte coherent accesses cover whole lines
+    const int64_t DN2 = (int64_t)Dm * N * 2;
+    float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + (PIPE ? ((int64_t)cc * N + nn) * 2 : lane_off);
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * kTile;
@@ -321,7 +324,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 const float *src = gdown + (int64_t)J * DN8;
                 if (PIPE) {
 #pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + k, Gd[k], Gd[k + 1]);
+                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
                 } else {
                     const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
                     Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
@@ -489,7 +492,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 float *dst = gdown + (int64_t)J * DN8;
                 if (PIPE) {
 #pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + k, Gd[k], Gd[k + 1]);
+                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
                 } else {
                     ((float4 *)dst)[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
                     ((float4 *)dst)[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);

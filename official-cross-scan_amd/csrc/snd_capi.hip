@@ -108,11 +108,15 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->x_elems = planes * g.nCX * g.Hp;
     plan->x_sd_elems = plan->x_elems;
     plan->x_v_elems = planes * g.nCY * g.Wp;
-    // strip-pipeline sync words, then (backward only) one row of G = a*g per plane: the adjoint
-    // carried from the strip below
+    // strip-pipeline sync words, then one row per plane: forward, h handed from a strip to the strip
+    // below (strip schedule only); backward, the adjoint G = a*g handed to the strip above
     const int64_t sync_bytes = snd::sync_words(plane_chunks(*shape), g.nCY) * (int64_t)sizeof(int);
-    plan->fwd_workspace_bytes = sync_bytes;
-    plan->bwd_workspace_bytes = sync_bytes + planes * (int64_t)g.Wp * (int64_t)sizeof(float);
+    const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);
+    plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
+    plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
+    plan->auto_schedule = snd::use_strip_pipeline(SND_SCHED_AUTO, plane_chunks(*shape), g.nCY, plan) ? SND_SCHED_STRIPS
+                                                                                                   : SND_SCHED_PLANE;
+    plan->reserved_ = 0;
     return SND_OK;
 }
 

@@ -190,12 +190,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
     // right before the tile needs it, so that a strip runs one tile behind the strip above.  One wave
     // polls for the hand-over (more pollers only slow the counters down); the rest wait at the barrier.
+    // The hand-over goes through a one-row buffer per plane in the workspace, laid out
+    // [col tile J][pair k][c][n][2] so that a wave's 8-byte coherent accesses cover whole lines (the
+    // x_v checkpoint keeps its own layout and plain streaming stores).  A strip overwrites slot J with
+    // its own row once it has consumed it, so the corner h[r0-1][j0-1] is kept from the previous fetch.
+    const int64_t DN2 = (int64_t)Dm * N * 2;
+    float *hrow = PIPE ? (float *)p.workspace + sync_words((int64_t)sh.batch * G * nChunks, geo.nCY) +
+                             (int64_t)b * geo.nCX * DN8 + ((int64_t)cc * N + nn) * 2
+                       : nullptr;
+    float xv_last = 0.f;
     auto fetch_row_above = [&](int I, int J) {
         if (I == 0) return;
-        const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+        const float *src = hrow + (int64_t)J * DN8;
+        qcorner = J > 0 ? xv_last : 0.f;
 #pragma unroll
-        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + k, qxv[k], qxv[k + 1]);
-        qcorner = J > 0 ? ld1_coherent(src + 7 - DN8) : 0.f;
+        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, qxv[k], qxv[k + 1]);
+        xv_last = qxv[kCkX - 1];
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&](const Stage &q) {
@@ -318,12 +328,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
-                if (PIPE) {
+                st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
+                st4_stream(dst + 4, hup[4], hup[5], hup[6], hup[7]);
+                if (PIPE && I + 1 < geo.nCY) {      // and the hand-over copy for the strip below
+                    float *ho = hrow + (int64_t)J * DN8;
 #pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + k, hup[k], hup[k + 1]);
-                } else {
-                    st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
-                    st4_stream(dst + 4, hup[4], hup[5], hup[6], hup[7]);
+                    for (int k = 0; k < kCkX; k += 2) st2_coherent(ho + (k >> 1) * DN2, hup[k], hup[k + 1]);
                 }
             }
             if (PIPE) strip_stores_done();

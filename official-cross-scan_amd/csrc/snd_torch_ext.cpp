@@ -146,11 +146,15 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     p.out_dtype = dtype_code(out.scalar_type());
     p.out_batch_stride = out.stride(0); p.out_d_stride = out.stride(1); p.out_h_stride = out.stride(2);
     p.x = x.data_ptr<float>(); p.x_v = x_v.data_ptr<float>(); p.x_sd = x_sd.data_ptr<float>();
-    // scratch for the strip-pipelined schedule; released to the caching allocator in stream order
-    at::Tensor ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
-    p.workspace = ws.data_ptr();
-    p.workspace_bytes = c.plan.fwd_workspace_bytes;
+    // scratch for the strip-pipelined schedule (only when it will be used); released to the caching
+    // allocator in stream order
     p.schedule = g_schedule;
+    at::Tensor ws;
+    if (g_schedule == SND_SCHED_STRIPS || (g_schedule == SND_SCHED_AUTO && c.plan.auto_schedule == SND_SCHED_STRIPS)) {
+        ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
+        p.workspace = ws.data_ptr();
+        p.workspace_bytes = c.plan.fwd_workspace_bytes;
+    }
     p.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");

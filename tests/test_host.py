@@ -21,7 +21,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
-    assert C.sizeof(capi.Plan) == 56
+    assert C.sizeof(capi.Plan) == 64
     assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4
     assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8
 
@@ -29,7 +29,7 @@ def test_struct_layouts_match_header_sizes():
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
-    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes"]),
+    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule"]),
               ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared"]),
               ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
@@ -59,7 +59,8 @@ def test_plan_geometry(H, W, ncx, ncy):
     assert plan.x_elems == planes * ncx * plan.x_inner == plan.x_sd_elems
     assert plan.x_v_elems == planes * ncy * plan.xv_inner
     sync_words = (4 + 2 * 4 * 1 * ncy + 3) // 4 * 4         # header + (batch * groups * chunks) * strips
-    assert plan.fwd_workspace_bytes == sync_words * 4
+    assert plan.fwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
+    assert plan.auto_schedule == (capi.SCHED_STRIPS if ncy > 1 else capi.SCHED_PLANE)   # 8 plane chunks only
     assert plan.bwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
 
 
