@@ -131,7 +131,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     // so that the two 32-byte halves of each 64-byte run are requested while the memory line is in
     // flight: a line is fetched from HBM twice per strip instead of four times.
     // (Only where it pays and fits: the 16-state whole-plane kernels, which are bandwidth-bound.)
-    constexpr bool PAIR = NP == 16 && !PIPE;
+    constexpr bool PAIR = NP == 16;
     struct Stage { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo; };
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
