@@ -288,14 +288,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 
         for (int J = geo.nCX - 1; J >= 0; --J) {
             const int j0 = J * kCkX;
-            prefetch(I, J);                         // no loads in flight across the register-hungry sweep
-            commit();
-            // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
-            // others wait at the barrier.
-            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
-            __syncthreads();
-
-            // ---- checkpoints and carried adjoints of this tile
+            // ---- checkpoints and carried adjoints of this tile: requested first, so that they arrive
+            // under the staging below instead of being waited for after the barrier
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
             float Gd[kCkX];                                        // G of the row below
             if (I > 0) {
@@ -320,19 +314,33 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
             }
-            if (I + 1 < geo.nCY && lvalid) {
-                const float *src = gdown + (int64_t)J * DN8;
-                if (PIPE) {
-#pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
-                } else {
+            if (!PIPE) {
+                if (I + 1 < geo.nCY && lvalid) {
+                    const float *src = gdown + (int64_t)J * DN8;
                     const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
                     Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
                     Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
-                }
-            } else {
+                } else {
 #pragma unroll
-                for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
+                    for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
+                }
+            }
+            prefetch(I, J);                         // no loads in flight across the register-hungry sweep
+            commit();
+            // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
+            // others wait at the barrier.
+            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
+            __syncthreads();
+
+            if (PIPE) {                             // written by another block: only after the wait above
+                if (I + 1 < geo.nCY && lvalid) {
+                    const float *src = gdown + (int64_t)J * DN8;
+#pragma unroll
+                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
+                }
             }
             const float gd_old0 = Gd[0];            // G[r0+8][j0]: the corner of the tile on the left
 
