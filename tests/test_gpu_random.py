@@ -1,0 +1,92 @@
+"""Seeded random sweep over shapes, dtypes and options through the C ABI, each case against the
+float64 C oracle: catches interactions (schedule x directions x optional inputs x ragged sizes x
+state counts x shared delta groups) that the targeted tests do not enumerate."""
+import numpy as np
+import pytest
+import torch
+
+import capi
+from oracle import snd_oracle as O
+from oracle import snd_oracle_c as OC
+from test_gpu_corners import flip_groups_np
+from test_gpu_fwd import relerr
+
+pytestmark = pytest.mark.gpu
+DT = {0: torch.float32, 1: torch.bfloat16, 2: torch.float16}
+
+
+def draw(seed):
+    r = np.random.RandomState(1000 + seed)
+    K = int(r.choice([1, 2, 4, 8]))
+    rg = int(r.choice([1, 3, 4, 16, 20]))
+    c = dict(Bt=int(r.randint(1, 4)), K=K, Dm=K * rg, H=int(r.randint(1, 45)), W=int(r.randint(1, 45)),
+             N=int(r.choice([1, 2, 3, 4, 7, 8, 9, 12, 16])), dt=int(r.choice([0, 0, 1, 2])),
+             sched=int(r.choice([0, 1, 2])), dirs=int(r.choice([0, 1])), softplus=bool(r.randint(2)),
+             has_D=bool(r.randint(2)), has_bias=bool(r.randint(2)), has_decay=bool(r.randint(4) == 0),
+             out_float=bool(r.randint(2)), share_delta=bool(r.randint(3) == 0))
+    if not c["softplus"]:
+        c["has_bias"] = False                              # delta + (negative) bias must stay positive without softplus
+    c["Dd"] = c["Dm"] // 2 if (c["share_delta"] and c["Dm"] % 2 == 0) else c["Dm"]
+    return c
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_case(gpu_device, seed):
+    c = draw(seed)
+    print("random case", seed, c, flush=True)
+    d = O.make_inputs(c["Bt"], c["Dm"], c["H"], c["W"], N=c["N"], K=c["K"], seed=seed, Dd=c["Dd"])
+    if not c["softplus"]:
+        d["delta"] = np.abs(d["delta"]) + 0.01            # a plain delta must be positive to keep a < 1
+    dtype = DT[c["dt"]]
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    for k in ("u", "delta", "B", "C"):
+        t[k] = t[k].to(dtype)
+    D = t["D"] if c["has_D"] else None
+    bias = t["delta_bias"] if c["has_bias"] else None
+    dec = torch.tensor([0.9], device=gpu_device) if c["has_decay"] else None
+    dout = t["dout"] if c["out_float"] else t["dout"].to(dtype)
+    f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, c["softplus"], c["out_float"], dec, True,
+                     c["sched"], c["dirs"])
+    f.launch()
+    g = capi.bwd(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, dout, f.x, f.x_v, c["softplus"], dec, f.x_sd,
+                 None, c["sched"], c["dirs"])
+    torch.cuda.synchronize()
+    strips = c["sched"] == capi.SCHED_STRIPS or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule == capi.SCHED_STRIPS)
+    if strips and f.plan.n_chunks_y > 1:                   # a single strip always runs as a whole plane
+        assert int(f.ws.view(torch.int32)[1]) == 0         # no strip wait gave up
+
+    # oracle on the values the kernels saw; corner directions by flipping group-wise
+    K = c["K"]
+    r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    r["dout"] = dout.float().cpu().numpy()
+    rep = c["Dm"] // c["Dd"]
+    fl = (lambda a: flip_groups_np(a, K)) if c["dirs"] else (lambda a: a)
+    if c["dirs"] and rep > 1:                              # flip delta per channel group: expand it first
+        r["delta"] = np.repeat(r["delta"], rep, axis=1)
+    oD = d["D"] if c["has_D"] else None
+    ob = d["delta_bias"] if c["has_bias"] else None
+    if c["dirs"] and rep > 1 and ob is not None:
+        ob = np.repeat(ob, rep)
+    od = np.array([0.9], dtype=np.float32) if c["has_decay"] else None
+    a = (fl(r["u"]), fl(r["delta"]), d["A"], fl(r["B"]), fl(r["C"]), oD, ob)
+    ref = fl(OC.fwd(*a, c["softplus"], od, real="f64"))
+    gref = OC.bwd(*a, fl(r["dout"]), c["softplus"], od, real="f64")
+    half = c["dt"] != 0
+    assert relerr(f.out.float().cpu().numpy(), ref) <= (1e-4 if c["out_float"] or not half else 1e-2)
+    names = ["du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias", "dA_decay"]
+    for i, nm in enumerate(names):
+        if g[i] is None:
+            assert gref[i] is None or nm in ("dD", "ddelta_bias", "dA_decay"), nm
+            continue
+        want = gref[i]
+        if nm in ("du", "dB", "dC"):
+            want = fl(want)
+        if nm == "ddelta":
+            want = fl(want)
+            if c["dirs"] and rep > 1:                      # fold the expanded delta back
+                want = want.reshape(c["Bt"], c["Dd"], rep, c["H"], c["W"]).sum(2)
+        if nm == "ddelta_bias" and c["dirs"] and rep > 1:
+            want = want.reshape(c["Dd"], rep).sum(1)
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 3e-4
+        e = relerr(g[i].float().cpu().numpy(), np.asarray(want))
+        assert e <= tol, (nm, e)
