@@ -102,12 +102,15 @@ def cpu_baseline(workload, budget_s=20.0):
 
 
 def measured_traffic(workload):
-    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary."""
+    """HBM bytes per launch of the dominant kernel, and the fraction of cycles its SIMDs spend
+    issuing vector ALU instructions, from the committed rocprofv3 --pmc summary."""
     path = os.path.join(ROOT, "profiles", "bwd_kernel_%s_pmc.txt" % workload)
     if not os.path.exists(path):
-        return None
-    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read())
-    return float(m.group(1)) if m else None
+        return None, None
+    text = open(path).read()
+    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", text)
+    v = re.search(r"backward [0-9.e]+ / \([0-9.e]+ / 2\) = ([0-9.]+)", text)
+    return (float(m.group(1)) if m else None), (float(v.group(1)) if v else None)
 
 
 def main():
@@ -180,6 +183,7 @@ def main():
 
     value = (fb + bb) / (ms * 1e-3) / 1e9
     achieved = bb / (kb_ms * 1e-3) / 1e9
+    traffic, valu_frac = measured_traffic(args.workload)
     rec = {
         "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
@@ -193,7 +197,9 @@ def main():
                    "kernel_only_GBs": round((fb + bb) / ((kf_ms + kb_ms) * 1e-3) / 1e9, 2)},
         "roofline": {"bound": "hbm", "kernel": "snd::bwd_kernel", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic(args.workload), "algorithmic_bytes_per_launch": bb},
+                     "traffic": traffic, "algorithmic_bytes_per_launch": bb,
+                     # the kernel is bound by vector-ALU issue, not by HBM: fraction of SIMD cycles issuing VALU
+                     "valu_issue_frac": valu_frac},
     }
     if not args.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(args.workload)
