@@ -64,7 +64,7 @@ __device__ __forceinline__ void rows_scatter4x2(float &b0, float &b1, float &b2,
 #ifndef SND_BWD_WAVES
 #define SND_BWD_WAVES 2
 #endif
-template <typename T, int NP, bool PIPE>
+template <typename T, int NP, bool PIPE, int TE>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD_WAVES, SND_BWD_WAVES))) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     constexpr int NBC = 4;
     constexpr int NPX = kTile / NP;
     constexpr int HG = 10, DLP = HG * HG;           // delta' on the tile plus a one-cell halo
-    constexpr int NHALO = 36, NHK = (NHALO + NP - 1) / NP;
+    constexpr int NHALO = 4 * TE + 4, NHK = (NHALO + NP - 1) / NP;   // ring around the TE x TE tile
 
     // A wave's channels (four with 16 states per channel, eight with 8) are reduced in registers and
     // every wave owns a partial dB/dC tile, written with plain stores.
@@ -194,14 +194,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // ---- register staging of one tile's raw inputs (loaded at the start of the tile, then committed to LDS)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
-        const int r0 = I * kRows, j0 = J * kCkX;
+        const int r0 = I * TE, j0 = J * TE;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
-            const bool in = row < H && col < W;
+            const bool in = pr < TE && pj < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
             const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
 #pragma unroll
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         for (int k = 0; k < NPX; ++k) {
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-            const bool ok = cvalid && row < H && col < W;
+            const bool ok = cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mc = mcol(min(col, W - 1));
             const float vd = ldg_b(db, cDb + mad24(mr, DhB, mc * ESZ)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mc * ESZ));
             const float vo = ld_f32_b(dob, cDob + mad24(mr, DohB, mc << sh_do), p.dout_dtype);
@@ -226,15 +226,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             qdo[k] = ok ? vo : 0.f;
         }
 #pragma unroll
-        for (int k = 0; k < NHK; ++k) {   // the 36 halo cells of the 10x10 delta' grid
+        for (int k = 0; k < NHK; ++k) {   // the ring of halo cells around the tile in the delta' grid
             const int hidx = n + NP * k;
             int rr, jj;
-            if (hidx < 10) { rr = 0; jj = hidx; }
-            else if (hidx < 20) { rr = 9; jj = hidx - 10; }
-            else if (hidx < 28) { rr = hidx - 19; jj = 0; }
-            else { rr = hidx - 27; jj = 9; }
+            if (hidx < TE + 2) { rr = 0; jj = hidx; }
+            else if (hidx < 2 * TE + 4) { rr = TE + 1; jj = hidx - (TE + 2); }
+            else if (hidx < 3 * TE + 4) { rr = hidx - (2 * TE + 3); jj = 0; }
+            else { rr = hidx - (3 * TE + 3); jj = TE + 1; }
             const int row = r0 - 1 + rr, col = j0 - 1 + jj;
-            const bool ok = cvalid && row >= 0 && row < H && col >= 0 && col < W;
+            const bool ok = cvalid && hidx < NHALO && row >= 0 && row < H && col >= 0 && col < W;
             const float vd = ldg_b(db, cDb + mad24(mrow(min(max(row, 0), H - 1)), DhB, mcol(min(max(col, 0), W - 1)) * ESZ));
             qh[k] = ok ? vd : 0.f;
         }
@@ -253,7 +253,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const float raw = qdl[k] + bias;
             float dsp = 1.f;
             const float dl = softplus ? softplus20(raw, dsp) : raw;
-            sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1] = dl;
+            if (TE == 8 || ((pp >> 3) < TE && (pp & 7) < TE))     // slots beyond the tile belong to the halo ring
+                sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1] = dl;
             sDu[cl * kTile + pp] = dl * qu[k];
             sU[cl * kTile + pp] = qu[k];
             sDo[cl * kTile + pp] = qdo[k];
@@ -263,10 +264,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         for (int k = 0; k < NHK; ++k) {
             const int hidx = n + NP * k;
             int rr, jj;
-            if (hidx < 10) { rr = 0; jj = hidx; }
-            else if (hidx < 20) { rr = 9; jj = hidx - 10; }
-            else if (hidx < 28) { rr = hidx - 19; jj = 0; }
-            else { rr = hidx - 27; jj = 9; }
+            if (hidx < TE + 2) { rr = 0; jj = hidx; }
+            else if (hidx < 2 * TE + 4) { rr = TE + 1; jj = hidx - (TE + 2); }
+            else if (hidx < 3 * TE + 4) { rr = hidx - (2 * TE + 3); jj = 0; }
+            else { rr = hidx - (3 * TE + 3); jj = TE + 1; }
             const float raw = qh[k] + bias;
             float dsp;
             if (hidx < NHALO) sDl[cl * DLP + rr * HG + jj] = softplus ? softplus20(raw, dsp) : raw;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
 
     for (int I = I_hi; I >= I_lo; --I) {
-        const int r0 = I * kRows;
+        const int r0 = I * TE;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
         float aR[kRows];                            // a at that column (only ever multiplies G there)
         float GRc = 0.f;                            // G[r0+8][j0+8]
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         for (int r = 0; r < kRows; ++r) { GR[r] = 0.f; GsR[r] = 0.f; aR[r] = 0.f; }
 
         for (int J = geo.nCX - 1; J >= 0; --J) {
-            const int j0 = J * kCkX;
+            const int j0 = J * TE;
             // ---- checkpoints and carried adjoints of this tile: requested first, so that they arrive
             // under the staging below instead of being waited for after the barrier
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
                 hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
                 hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
-                if (J > 0) hc = src[7 - DN8];
+                if (J > 0) hc = src[TE - 1 - DN8];          // last column of the tile on the left
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
@@ -348,14 +349,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // are held at a time.  The right half starts from h, s at column 3, which a plain
             // forward pass over the left half provides first (that half is recomputed when it is
             // swept: 32 extra cell updates per tile buy about 60 registers).
-            float hmid[kRows], smid[kRows];
+            float hmid[kRows] = {}, smid[kRows] = {};
             {
                 float aprev[4], hprev[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { aprev[j] = AEXP(-1, j); hprev[j] = hu[j]; }
                 float diag0 = hc;
 #pragma unroll
-                for (int r = 0; r < kRows; ++r) {
+                for (int r = 0; r < TE; ++r) {
                     float al = AEXP(r, -1), left = hlft[r], sl = slft[r], diag = diag0;
                     diag0 = hlft[r];
 #pragma unroll
@@ -380,18 +381,19 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             auto sweep_half = [&](auto C0_, const float *top, float corner, const float (&hL)[kRows],
                                   const float (&sL)[kRows], float *GdH, float gdiag0) {
                 constexpr int C0 = decltype(C0_)::value;
+                constexpr int HW = C0 == 0 ? 4 : TE - 4;        // columns of this half inside the tile
                 float hT[kRows][4];
                 {
                     float aprev[4], hprev[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) { aprev[j] = AEXP(-1, C0 + j); hprev[j] = top[j]; }
+                    for (int j = 0; j < HW; ++j) { aprev[j] = AEXP(-1, C0 + j); hprev[j] = top[j]; }
                     float diag0 = corner;
 #pragma unroll
-                    for (int r = 0; r < kRows; ++r) {
+                    for (int r = 0; r < TE; ++r) {
                         float al = AEXP(r, C0 - 1), left = hL[r], diag = diag0;
                         diag0 = hL[r];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
+                        for (int j = 0; j < HW; ++j) {
                             const float a = AEXP(r, C0 + j);
                             const float bu = myB[r * kCkX + C0 + j] * myDu[r * kCkX + C0 + j];
                             const float up = hprev[j];
@@ -406,14 +408,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 float adn[4];
                 float Gd8 = gdiag0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) adn[j] = AEXP(kRows, C0 + j);
+                for (int j = 0; j < HW; ++j) adn[j] = AEXP(TE, C0 + j);
 #pragma unroll
-                for (int r = kRows - 1; r >= 0; --r) {
+                for (int r = TE - 1; r >= 0; --r) {
                     __builtin_amdgcn_sched_barrier(0);
                     float arow[5], s[4], buv[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) arow[j] = AEXP(r, C0 + j);
-                    arow[4] = aR[r];
+                    for (int j = 0; j < HW; ++j) arow[j] = AEXP(r, C0 + j);
+                    arow[HW] = aR[r];
                     const float4 vB4 = *(const float4 *)(myB + r * kCkX + C0), vC4 = *(const float4 *)(myC + r * kCkX + C0);
                     const float4 vU4 = *(const float4 *)(myDu + r * kCkX + C0), vO4 = *(const float4 *)(myDo + r * kCkX + C0);
                     const float aB[4] = {vB4.x, vB4.y, vB4.z, vB4.w}, aC[4] = {vC4.x, vC4.y, vC4.z, vC4.w};
@@ -421,16 +423,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     {
                         float sp = sL[r];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
+                        for (int j = 0; j < HW; ++j) {
                             buv[j] = aB[j] * aU[j];
                             sp = fmaf(arow[j], sp, buv[j]);
                             s[j] = sp;
                         }
                     }
                     float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
-                    float q[4], pp_[4], vB[4], vC[4];
+                    float q[4] = {}, pp_[4] = {}, vB[4] = {}, vC[4] = {};
 #pragma unroll
-                    for (int j = 3; j >= 0; --j) {
+                    for (int j = HW - 1; j >= 0; --j) {
                         const float dov = aO[j];
                         const float Bv = aB[j], Cv = aC[j];
                         const float duv = aU[j];
@@ -489,7 +491,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     GsR[r] = Gsr;
                     aR[r] = arow[0];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) adn[j] = arow[j];
+                    for (int j = 0; j < HW; ++j) adn[j] = arow[j];
                 }
             };
             const float gd_old4 = Gd[4];            // G[r0+8][j0+4]: corner of the left half
@@ -522,9 +524,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 const float uv = sU[cl * kTile + pp], dov = sDo[cl * kTile + pp], sg = sSg[cl * kTile + pp];
                 const float duv = fmaf(Dv, dov, dl * qv);
                 const float ddl = fmaf(uv, qv, pv) * sg;
-                dD_acc = fmaf(dov, uv, dD_acc);
-                dbias_acc += ddl;
-                if (cvalid && row < H && col < W) {
+                if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W) {
+                    dD_acc = fmaf(dov, uv, dD_acc);
+                    dbias_acc += ddl;
                     const uint32_t o = cGb + mad24(mrow(row), WB, mcol(col) * ESZ);
                     stg_b(dub, o, duv);
                     stg_b(ddb, o, ddl);
@@ -535,7 +537,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             {
                 SND_THREAD_MAPS(NP);
                 const int row = r0 + pr, col = j0 + pj;
-                const bool in = row < H && col < W;
+                const bool in = pr < TE && pj < TE && row < H && col < W;
                 const uint32_t o = mad24(mrow(row), W4, mcol(col) * 4);
 #pragma unroll
                 for (int k = 0; k < NBC; ++k) {
@@ -583,10 +585,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     }
 }
 
-template <typename T, int NP>
-static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
+template <typename T, int NP, int TE>
+static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
-    const Geo geo = make_geo(sh.nrows, sh.ncols);
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
@@ -598,19 +599,25 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SND_ERR_LAUNCH;
     if (!configured[pipe][dev]) {
-        const void *fn = pipe ? (const void *)bwd_kernel<T, NP, true> : (const void *)bwd_kernel<T, NP, false>;
+        const void *fn = pipe ? (const void *)bwd_kernel<T, NP, true, TE> : (const void *)bwd_kernel<T, NP, false, TE>;
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return SND_ERR_LAUNCH;
         configured[pipe][dev] = true;
     }
     if (pipe) {
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
-        hipLaunchKernelGGL((bwd_kernel<T, NP, true>), dim3((int)(nPC * geo.nCY)), dim3(16 * NP), lds, stream, p, geo);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE>), dim3((int)(nPC * geo.nCY)), dim3(16 * NP), lds, stream, p, geo);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
-        hipLaunchKernelGGL((bwd_kernel<T, NP, false>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, false, TE>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T, int NP>
+static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
+    const Geo geo = make_geo(p.f.shape.nrows, p.f.shape.ncols);
+    return geo.te == 7 ? launch_bwd_te<T, NP, 7>(p, geo, stream) : launch_bwd_te<T, NP, 8>(p, geo, stream);
 }
 
 // One instantiation per input dtype, each in its own translation unit.

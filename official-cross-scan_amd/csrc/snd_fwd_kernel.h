@@ -26,7 +26,7 @@
 
 namespace snd {
 
-template <typename T, int NP, bool SAVE, bool PIPE>
+template <typename T, int NP, bool SAVE, bool PIPE, int TE>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
     constexpr int CB = 16;                          // channels per block
@@ -136,14 +136,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto load_tile = [&](Stage &q, int I, int J) {
-        const int r0 = I * kRows, j0 = J * kCkX;
+        const int r0 = I * TE, j0 = J * TE;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
-            const bool in = row < H && col < W;
+            const bool in = pr < TE && pj < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
             const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
 #pragma unroll
@@ -159,14 +159,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         for (int k = 0; k < NPX; ++k) {
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-            const bool ok = cvalid && row < H && col < W;
+            const bool ok = cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
             const float vd = ldg_b(db, cDb + mad24(mr, DhB, mcB)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mcB));
             q.qdl[k] = ok ? vd : 0.f;
             q.qu[k] = ok ? vu : 0.f;
         }
         q.qhalo = 0.f;
-        if (n < kCkX) {   // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
+        if (n < TE) {     // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
             const int row = r0 - 1, col = j0 + n;
             const float vd = ldg_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
             q.qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
             qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
-            qcorner = J > 0 ? src[7 - DN8] : 0.f;
+            qcorner = J > 0 ? src[TE - 1 - DN8] : 0.f;      // last column of the tile on the left
         }
     };
     // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         qcorner = J > 0 ? xv_last : 0.f;
 #pragma unroll
         for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, qxv[k], qxv[k + 1]);
-        xv_last = qxv[kCkX - 1];
+        xv_last = qxv[TE - 1];
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&](const Stage &q) {
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     load_pair(I_begin, 0);
     prefetch_xv(I_begin, 0);
     for (int I = I_begin; I < I_end; ++I) {
-        const int r0 = I * kRows;
+        const int r0 = I * TE;
         float hl[kRows], sl[kRows], al[kRows];      // h, s, a at the column left of the tile
 #pragma unroll
         for (int r = 0; r < kRows; ++r) { hl[r] = 0.f; sl[r] = 0.f; al[r] = 0.f; }
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         // one tile; `mine` holds its staged inputs, `last_of_pair` says that both register sets are
         // free once it is committed, so the next pair's loads can be issued under its compute
         auto do_tile = [&](const int J, const Stage &mine, const bool last_of_pair) {
-            const int j0 = J * kCkX;
+            const int j0 = J * TE;
             commit(mine);
             if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
             __syncthreads();
@@ -273,10 +273,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
 
             // ---- per-lane tile walk
 #pragma unroll
-            for (int j = 0; j < kCkX; ++j) aup[j] = (I > 0) ? fast_exp2(fmaf(myDl[j], A2, ld)) : 0.f;
+            for (int j = 0; j < kCkX; ++j) aup[j] = (I > 0 && j < TE) ? fast_exp2(fmaf(myDl[j], A2, ld)) : 0.f;
 
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) {
+            for (int r = 0; r < TE; ++r) {
                 float left = hl[r], sleft = sl[r], aleft = al[r];
                 float diag = corner;
                 corner = hl[r];                     // h[r0+r][j0-1] is the next row's corner
@@ -294,6 +294,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int j = j4 + q;
+                        if (j >= TE) { y[j] = 0.f; continue; }   // storage column beyond the tile
                         const float a = fast_exp2(fmaf(adl[q], A2, ld));
                         const float bu = ab[q] * adu[q];
                         const float X = fmaf(-0.5f * (aup[j] + aleft), diag, hup[j]);
@@ -354,7 +355,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-                if (cvalid && row < H && col < W)
+                if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
                     st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
@@ -375,10 +376,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
 #endif
 }
 
-template <typename T, int NP>
-static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
+template <typename T, int NP, int TE>
+static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t stream) {
     const snd_shape &sh = p.shape;
-    const Geo geo = make_geo(sh.nrows, sh.ncols);
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
@@ -387,17 +387,23 @@ static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
         const int grid = (int)(nPC * geo.nCY);
         if (p.x != nullptr)
-            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
         else
-            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
         if (p.x != nullptr)
-            hipLaunchKernelGGL((fwd_kernel<T, NP, true, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, false, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
         else
-            hipLaunchKernelGGL((fwd_kernel<T, NP, false, false>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, false, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T, int NP>
+static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
+    const Geo geo = make_geo(p.shape.nrows, p.shape.ncols);
+    return geo.te == 7 ? launch_fwd_te<T, NP, 7>(p, geo, stream) : launch_fwd_te<T, NP, 8>(p, geo, stream);
 }
 
 // One instantiation per input dtype, each in its own translation unit.

@@ -21,6 +21,11 @@ CONFIGS = [
     ("c4-plane", 1, 8, 512, 512, 16, 4, torch.bfloat16),
     ("c4-plane-n1", 1, 8, 512, 512, 1, 4, torch.bfloat16),
     ("odd", 1, 4, 61, 43, 16, 2, torch.float32),
+    # planes that are walked in 7x7 tiles (fewer padded cells than with 8x8)
+    ("stage-28", 2, 16, 28, 28, 16, 4, torch.float32),
+    ("stage-7", 2, 32, 7, 7, 16, 4, torch.bfloat16),
+    ("te7-ragged", 1, 8, 20, 33, 8, 2, torch.float32),
+    ("te7-row", 3, 4, 6, 40, 16, 1, torch.float16),
 ]
 
 

@@ -20,6 +20,8 @@ SHAPES = [
     (1, 4, 24, 40, 4, 2, torch.float32),       # 8-state kernels
     (1, 8, 100, 70, 16, 4, torch.bfloat16),
     (3, 20, 33, 21, 5, 1, torch.float16),      # partial channel chunk (20 = 16 + 4), odd N
+    (1, 8, 35, 21, 16, 2, torch.float32),      # 7x7 tiles: 5 strips x 3 tiles
+    (2, 16, 27, 14, 8, 4, torch.bfloat16),     # 7x7 tiles, ragged last strip, 8-state kernels
 ]
 
 
@@ -49,7 +51,7 @@ def test_strips_match_plane_and_oracle(gpu_device, Bt, Dm, H, W, N, K, dtype):
     out_s, g_s, st_s = res[capi.SCHED_STRIPS]
     # same arithmetic in the same order per plane: everything that is not an atomic sum is bit-identical
     assert torch.equal(out_p, out_s)
-    ncx = (W + 7) // 8
+    ncx = f.plan.n_chunks_x
     assert torch.equal(st_p[1], st_s[1])                      # x_v: every entry is written
     for a, b_ in ((st_p[0], st_s[0]), (st_p[2], st_s[2])):    # x, x_sd: stored tile-major, last column tile unused
         assert torch.equal(a.reshape(Bt, ncx, -1)[:, :ncx - 1], b_.reshape(Bt, ncx, -1)[:, :ncx - 1])

@@ -49,7 +49,8 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
     assert got == want
 
 
-@pytest.mark.parametrize("H,W,ncx,ncy", [(56, 56, 7, 7), (14, 14, 2, 2), (200, 336, 42, 25), (1, 37, 5, 1), (512, 512, 64, 64)])
+@pytest.mark.parametrize("H,W,ncx,ncy", [(56, 56, 7, 7), (14, 14, 2, 2), (200, 336, 42, 25), (1, 37, 5, 1), (512, 512, 64, 64),
+                                         (28, 28, 4, 4), (21, 35, 5, 3), (7, 7, 1, 1)])   # the last three use 7x7 tiles
 def test_plan_geometry(H, W, ncx, ncy):
     st, plan = capi.make_plan(capi.Shape(2, 8, H, W, 16, 4, 8, capi.SND_F32))
     assert st == 0
@@ -155,3 +156,14 @@ def test_cross_scan_host_helpers():
     assert torch.allclose(cs.cross_merge(xs, w), 10 * x)
     wc = torch.arange(12, dtype=torch.float32).reshape(4, 3)
     assert torch.allclose(cs.cross_merge(xs, wc), x * wc.sum(0).reshape(1, 3, 1, 1))
+
+
+def test_tile_extent_choice():
+    """7x7 tiles where they leave clearly fewer padded cells (the 14 / 28 / 7 stage sizes), else 8x8."""
+    def tiles(H, W):
+        st, plan = capi.make_plan(capi.Shape(1, 4, H, W, 16, 1, 4, capi.SND_F32))
+        assert st == 0
+        return plan.n_chunks_y, plan.n_chunks_x
+    assert tiles(14, 14) == (2, 2) and tiles(28, 28) == (4, 4) and tiles(7, 7) == (1, 1) and tiles(21, 35) == (3, 5)
+    assert tiles(56, 56) == (7, 7) and tiles(64, 64) == (8, 8) and tiles(512, 512) == (64, 64) and tiles(200, 336) == (25, 42)
+    assert tiles(1, 37) == (1, 5)                 # 294 vs 320 padded cells: not worth the smaller tile
