@@ -15,9 +15,9 @@
 // enters its right and lower neighbours, which the reference scatters to ddelta_vals[nrow-1][i],
 // ddelta_vals[nrow][i-1] and stitches across chunk seams; here they are gathered at the cell.)
 //
-// Organisation (not a translation): the same lane = one (channel, state) plane, 8x8 tile walk as the
-// forward, in reverse.  For each tile a lane recomputes h from the forward's checkpoints (row above
-// from x_v, column to the left from x, s from x_sd), one 8x4 half of the tile at a time into 32
+// Organisation (not a translation): the same lane = one (channel, state) plane, TE x TE tile walk
+// as the forward (TE = 8 or 7), in reverse.  For each tile a lane recomputes h from the forward's checkpoints (row above
+// from x_v, column to the left from x, s from x_sd), one half of the tile (4 columns, then the rest) at a time into 32
 // registers, and sweeps that half bottom-right to top-left.  The adjoint row handed to the strip
 // above goes through a private global scratch row; the column handed to the tile on the left stays
 // in registers.  dB/dC are reduced over a wave's channels with lane swaps, over the block's waves

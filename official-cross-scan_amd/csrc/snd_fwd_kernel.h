@@ -9,18 +9,22 @@
 //     s[i,j] = a*s[i,j-1] + bu                                          (:306-327)
 //     out    = D*u + sum_n C*(h - s + 0.25*bu)                          (:226-228,301,334)
 // but is organised for CDNA4 rather than translated:
-//   * one lane owns one (channel, state) plane and walks it in 8x8 tiles in plain row-major
-//     order, so the recurrence needs no block scans, shuffles or barriers in its dependency
-//     chain; a wave holds 64/NP channels x NP states of one (batch, group);
+//   * one lane owns one (channel, state) plane and walks it in TE x TE tiles (TE = 8, or 7 for
+//     planes that 7 divides better) in plain row-major order, so the recurrence needs no block
+//     scans, shuffles or barriers in its dependency chain; a wave holds 64/NP channels x NP
+//     states of one (batch, group);
 //   * the block stages each B/C tile once in LDS for its 16 channels; the per-pixel work
 //     (softplus, delta*u) is done once per pixel while staging, not once per state;
-//   * the next tile's global loads are issued before the current tile is computed;
+//   * the next tiles' global loads are issued before the current tile is computed (an aligned
+//     pair of tiles at a time, so that memory lines are not fetched once per tile);
 //   * tiles are always computed in full on zero-padded staging: cells outside the plane only
 //     feed cells further right/down, so they never reach a stored value and the inner loops
 //     carry no bounds checks;
 //   * the sum over states is a DPP reduction inside aligned lane groups;
 //   * h at strip bottoms (x_v) doubles as the carry to the next strip and as the backward's row
-//     checkpoint; h and s at tile right edges (x, x_sd) are the backward's column checkpoints.
+//     checkpoint; h and s at tile right edges (x, x_sd) are the backward's column checkpoints;
+//   * a block either walks a whole plane or (PIPE) one strip of it, the strips of a plane running
+//     as a pipeline of blocks one tile apart (few, large planes).
 #pragma once
 #include "snd_device.h"
 
