@@ -19,7 +19,7 @@ def draw(seed):
     r = np.random.RandomState(1000 + seed)
     K = int(r.choice([1, 2, 4, 8]))
     rg = int(r.choice([1, 3, 4, 16, 20]))
-    c = dict(Bt=int(r.randint(1, 4)), K=K, Dm=K * rg, H=int(r.randint(1, 45)), W=int(r.randint(1, 45)),
+    c = dict(Bt=int(r.randint(1, 4)), K=K, Dm=K * rg, H=int(r.randint(1, MAX_HW + 1)), W=int(r.randint(1, MAX_HW + 1)),
              N=int(r.choice([1, 2, 3, 4, 7, 8, 9, 12, 16])), dt=int(r.choice([0, 0, 1, 2])),
              sched=int(r.choice([0, 1, 2])), dirs=int(r.choice([0, 1])), softplus=bool(r.randint(2)),
              has_D=bool(r.randint(2)), has_bias=bool(r.randint(2)), has_decay=bool(r.randint(4) == 0),
@@ -30,7 +30,13 @@ def draw(seed):
     return c
 
 
-@pytest.mark.parametrize("seed", range(48))
+import os
+
+N_CASES = int(os.environ.get("SND_RANDOM_CASES", "48"))     # a longer sweep: SND_RANDOM_CASES=500 pytest ...
+MAX_HW = int(os.environ.get("SND_RANDOM_MAX_HW", "44"))     # larger planes: SND_RANDOM_MAX_HW=160
+
+
+@pytest.mark.parametrize("seed", range(N_CASES))
 def test_random_case(gpu_device, seed):
     c = draw(seed)
     print("random case", seed, c, flush=True)
