@@ -277,6 +277,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #define AEXP(r, j) fast_exp2(fmaf(DL(r, j), A2, ld))
 
     float dA_acc = 0.f, dec_acc = 0.f;              // per lane: sum delta'*da*a, sum da*a
+    const bool want_decay = p.dA_decay != nullptr;  // the second sum is skipped when nobody reads it
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
 
     for (int I = I_hi; I >= I_lo; --I) {
@@ -349,7 +350,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // are held at a time.  The right half starts from h, s at column 3, which a plain
             // forward pass over the left half provides first (that half is recomputed when it is
             // swept: 32 extra cell updates per tile buy about 60 registers).
-            float hmid[kRows] = {}, smid[kRows] = {};
+            float hmid[kRows] = {}, smid[kRows] = {}, amid[kRows] = {};   // h, s, a at column 3
             {
                 float aprev[4], hprev[4];
 #pragma unroll
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         hprev[j] = h;
                         diag = up; left = h; al = a; aprev[j] = a;
                     }
-                    hmid[r] = left; smid[r] = sl;
+                    hmid[r] = left; smid[r] = sl; amid[r] = al;
                 }
             }
 
@@ -383,6 +384,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 constexpr int C0 = decltype(C0_)::value;
                 constexpr int HW = C0 == 0 ? 4 : TE - 4;        // columns of this half inside the tile
                 float hT[kRows][4];
+                // the left half keeps a of its first KA columns from this pass for the sweep (as many as
+                // fit under 256 registers without spilling); everything else is recomputed there
+                constexpr int KA = C0 == 0 ? (TE == 7 ? 4 : 2) : 0;
+                float aT[KA ? kRows : 1][KA ? KA : 1];
                 {
                     float aprev[4], hprev[4];
 #pragma unroll
@@ -390,7 +395,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     float diag0 = corner;
 #pragma unroll
                     for (int r = 0; r < TE; ++r) {
-                        float al = AEXP(r, C0 - 1), left = hL[r], diag = diag0;
+                        float al = C0 == 0 ? AEXP(r, C0 - 1) : amid[r], left = hL[r], diag = diag0;
                         diag0 = hL[r];
 #pragma unroll
                         for (int j = 0; j < HW; ++j) {
@@ -400,6 +405,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                             const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
                             const float h = fmaf(a, left + X, bu);
                             hT[r][j] = h;
+                            if (j < KA) aT[r][j] = a;
                             hprev[j] = h;
                             diag = up; left = h; al = a; aprev[j] = a;
                         }
@@ -414,7 +420,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     __builtin_amdgcn_sched_barrier(0);
                     float arow[5], s[4], buv[4];
 #pragma unroll
-                    for (int j = 0; j < HW; ++j) arow[j] = AEXP(r, C0 + j);
+                    for (int j = 0; j < HW; ++j) arow[j] = j < KA ? aT[KA ? r : 0][j < KA ? j : 0] : AEXP(r, C0 + j);
                     arow[HW] = aR[r];
                     const float4 vB4 = *(const float4 *)(myB + r * kCkX + C0), vC4 = *(const float4 *)(myC + r * kCkX + C0);
                     const float4 vU4 = *(const float4 *)(myDu + r * kCkX + C0), vO4 = *(const float4 *)(myDo + r * kCkX + C0);
@@ -430,7 +436,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         }
                     }
                     float Gr = GR[r], Gsr = GsR[r], Gdiag = Gd8;
-                    float q[4] = {}, pp_[4] = {}, vB[4] = {}, vC[4] = {};
+                    float q[4] = {}, pp_[4] = {}, vB[4] = {}, vC[4] = {}, dsum[4] = {};
 #pragma unroll
                     for (int j = HW - 1; j >= 0; --j) {
                         const float dov = aO[j];
@@ -444,11 +450,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         const float dbu = fmaf(0.25f, dyC, g_ + gs);
                         const float h_l = (j == 0) ? hL[r] : hT[r][j - 1 < 0 ? 0 : j - 1];
                         const float h_u = (r == 0) ? top[j] : hT[r - 1 < 0 ? 0 : r - 1][j];
-                        const float hb = hT[r][j] - bu, sb = s[j] - bu;
+                        // g(h - bu) + gs(s - bu) = g(h - s) + (g + gs)(s - bu)
+                        const float hs = hT[r][j] - s[j], sb = s[j] - bu;
                         const float cross = fmaf(GdH[j], h_l, Gr * h_u);
-                        const float da = fmaf(-0.5f * a, cross, fmaf(g_, hb, gs * sb));
+                        const float da = fmaf(-0.5f * a, cross, fmaf(g_, hs, (g_ + gs) * sb));
                         dA_acc = fmaf(DL(r, C0 + j), da, dA_acc);
-                        dec_acc += da;
+                        dsum[j] = da;
                         const float Gn = a * g_;
                         Gdiag = GdH[j];
                         GdH[j] = Gn;
@@ -457,8 +464,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         q[j] = dbu * Bv;                           // per-pixel terms, summed over states below
                         pp_[j] = Av * da;
                         vB[j] = dbu * duv;                         // dB, dC contributions
-                        vC[j] = dov * fmaf(0.25f, bu, hb - sb);
+                        vC[j] = dov * fmaf(0.25f, bu, hs);
                     }
+                    if (want_decay) dec_acc += (dsum[0] + dsum[1]) + (dsum[2] + dsum[3]);
                     if (NP == 16) {
                         // sums over the channel's 16 states: quads 0,1 of the lane group end with
                         // q[0..1], q[2..3], quads 2,3 with pp_[0..1], pp_[2..3]
