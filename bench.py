@@ -120,7 +120,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
-    ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips"],
+    ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands"],
                     help="block mapping: chosen by shape (default), one block per plane chunk, or pipelined row strips")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
@@ -144,7 +144,7 @@ def main():
     import selective_nd_scan as snd
     from selective_nd_scan import capi
 
-    sched = {"auto": 0, "plane": 1, "strips": 2}[args.schedule]
+    sched = {"auto": 0, "plane": 1, "strips": 2, "bands": 3}[args.schedule]
     snd.set_schedule(sched)
     Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
     dtype = getattr(torch, dtn)

@@ -105,19 +105,19 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #ifdef SND_PIPE_TRACE
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
+    __shared__ int sSeen;                           // (pipelined) progress count of the strip below, as last polled
     if (PIPE) {
-        __shared__ int sTicket;
-        if (threadIdx.x == 0) sTicket = __hip_atomic_fetch_add(sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        // tickets run strip-major from the bottom strip up (all plane chunks' last strip, then every
-        // strip above it, ...): a job's predecessor holds an earlier ticket, and a strip only takes a
-        // slot about when it can start
+        if (threadIdx.x == 0) sSeen = 0;            // ordered before its readers by the barrier in draw_job
+        // A job is a band of consecutive strips (one strip each in the fully pipelined case), drawn
+        // bottom band first; band k from the bottom covers strips ceil(k*nCY/nBands) ..
+        // ceil((k+1)*nCY/nBands)-1, counted from the bottom.
+        int band;
+        if (!draw_job(sync, sh.batch * G, nChunks, geo.nBands, geo.nQueues, pair, chunk, band)) return;
         const int nPC = sh.batch * G * nChunks;
-        const int pc = sTicket % nPC;
-        if (sTicket / nPC >= geo.nCY) return;
-        I_hi = I_lo = geo.nCY - 1 - sTicket / nPC;
-        pair = pc / nChunks;
-        chunk = pc - pair * nChunks;
+        const int pc = pair * nChunks + chunk;
+        I_hi = geo.nCY - 1 - (band * geo.nCY + geo.nBands - 1) / geo.nBands;
+        I_lo = geo.nCY - ((band + 1) * geo.nCY + geo.nBands - 1) / geo.nBands;
+        (void)nPC;
         progress = sync + kSyncHeader + pc * geo.nCY;
 #ifdef SND_PIPE_TRACE
         trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_hi);
@@ -316,12 +316,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                 for (int r = 0; r < kRows; ++r) { hlft[r] = 0.f; slft[r] = 0.f; }
             }
-            if (!PIPE) {
+            // the adjoint row of the strip below: written by this block, or - first strip of a
+            // pipelined band - by another block.  It is requested here if it is known to be there (own
+            // rows; rows whose hand-over an earlier poll has already seen), else after the wait below.
+            const bool handed = PIPE && I == I_hi && I + 1 < geo.nCY;
+            const bool late = handed && __builtin_amdgcn_readfirstlane(*(volatile int *)&sSeen) < geo.nCX - J;
+            if (!late) {
                 if (I + 1 < geo.nCY && lvalid) {
                     const float *src = gdown + (int64_t)J * DN8;
-                    const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
-                    Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
-                    Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
+                    if (PIPE) {
+#pragma unroll
+                        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
+                    } else {
+                        const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                        Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
+                        Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
+                    }
                 } else {
 #pragma unroll
                     for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
@@ -331,10 +341,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             commit();
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
-            if (PIPE && I + 1 < geo.nCY && wave == 0) strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
+            if (handed && wave == 0) {
+                strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
+                if (tid == 0) sSeen = seen;         // read at the top of later tiles
+            }
             __syncthreads();
 
-            if (PIPE) {                             // written by another block: only after the wait above
+            if (late) {                             // only after the wait above
                 if (I + 1 < geo.nCY && lvalid) {
                     const float *src = gdown + (int64_t)J * DN8;
 #pragma unroll
@@ -506,6 +519,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             sweep_half(std::integral_constant<int, 4>{}, hu + 4, hu[3], hmid, smid, Gd + 4, GRc);
             sweep_half(std::integral_constant<int, 0>{}, hu, hc, hlft, slft, Gd, gd_old4);
             GRc = gd_old0;
+            const bool hands_over = PIPE && I == I_lo && I > 0;   // top strip of a band: another block takes the row
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
                 float *dst = gdown + (int64_t)J * DN8;
                 if (PIPE) {
@@ -516,9 +530,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     ((float4 *)dst)[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
                 }
             }
-            if (PIPE && I > 0) strip_stores_done();
+            if (hands_over) strip_stores_done();
             __syncthreads();
-            if (PIPE && I > 0) strip_signal(progress + I);   // tile J is handed over to the strip above
+            if (hands_over) strip_signal(progress + I);   // tile J is handed over to the strip above
 
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
             {
@@ -601,7 +615,8 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
     constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = WPB;
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
-    const bool pipe = use_strip_pipeline(p.f.schedule, nPC, geo.nCY, p.workspace);
+    const int bands = bwd_band_count(p.f.schedule, nPC, geo.nCY, p.workspace);   // 0: one block per plane chunk
+    const bool pipe = bands > 0;
     // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
     static bool configured[2][64] = {};
     int dev = 0;
@@ -614,7 +629,10 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
     if (pipe) {
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
-        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE>), dim3((int)(nPC * geo.nCY)), dim3(16 * NP), lds, stream, p, geo);
+        Geo gb = geo;
+        gb.nBands = bands;
+        gb.nQueues = job_queues(sh.batch * sh.n_groups);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
         hipLaunchKernelGGL((bwd_kernel<T, NP, false, TE>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);

@@ -79,7 +79,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 103; }
+int snd_version(void) { return 104; }
 
 const char *snd_status_string(int status) {
     switch (status) {
@@ -129,7 +129,7 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols,
                 esize(params->out_dtype)))
         return SND_ERR_STRIDE;
-    if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
+    if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_BANDS) return SND_ERR_SHAPE;
     if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (params->workspace) {
         snd_plan plan;
@@ -161,7 +161,7 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
     if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
-    if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_STRIPS) return SND_ERR_SHAPE;
+    if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_BANDS) return SND_ERR_SHAPE;
     if (params->f.directions != SND_DIR_TOPLEFT && params->f.directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
                 params->f.shape.ncols, esize(params->dout_dtype)))

@@ -20,6 +20,8 @@ struct Geo {
     int nCX, nCY;                  // column tiles, row strips (of te)
     int Hp, Wp;                    // inner extents of the saved state: nCY*8, nCX*8
     int te;                        // tile extent
+    int nBands;                    // pipelined schedules: jobs per plane chunk (set by the launcher)
+    int nQueues;                   // and the number of job queues: 8 (one per XCD) or 1
 };
 __host__ __device__ inline Geo make_geo(int H, int W) {
     const long long c8 = (long long)((H + 7) / 8) * ((W + 7) / 8) * 64, c7 = (long long)((H + 6) / 7) * ((W + 6) / 7) * 49;
@@ -29,6 +31,8 @@ __host__ __device__ inline Geo make_geo(int H, int W) {
     g.nCY = (H + g.te - 1) / g.te;
     g.Hp = g.nCY * kRows;
     g.Wp = g.nCX * kCkX;
+    g.nBands = 0;
+    g.nQueues = 1;
     return g;
 }
 
@@ -192,12 +196,13 @@ __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8
 // strips of a plane then run as a pipeline, each one tile behind the strip it depends on.
 // Blocks take (plane chunk, strip) jobs from a ticket counter in dependency order, so the block a
 // job waits for always holds an earlier ticket and is already running or finished.
-// Sync words (int32, zeroed before the launch): [0] ticket, [1] error flag, [4 + job] per-strip count
-// of tiles whose hand-over row the strip's block has written.
+// Sync words (int32, zeroed before the launch): [1] error flag, [4..11] ticket counters (one per job
+// queue), [12 + plane chunk * strips + strip] count of tiles whose hand-over row the strip's block has
+// written.
 #ifndef SND_POLL_SLEEP
 #define SND_POLL_SLEEP 16                           // s_sleep units (64 cycles) between polls
 #endif
-constexpr int kSyncHeader = 4;
+constexpr int kErrorWord = 1, kTicketWord = 4, kSyncHeader = 12;
 constexpr int kSpinLimit = 1 << 21;                 // polls (a memory round trip each) before giving up
 __host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips) {
 #ifdef SND_PIPE_TRACE   // timing study only: 4 extra words per job (start, end, time spent waiting, -)
@@ -249,7 +254,7 @@ __device__ __forceinline__ void strip_wait(const int *count, int need, int &seen
         __builtin_amdgcn_s_sleep(SND_POLL_SLEEP);
         if (++polls > kSpinLimit) {
             dead = true;
-            __hip_atomic_store(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sync + kErrorWord, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
         }
     }
@@ -258,11 +263,44 @@ __device__ __forceinline__ void strip_wait(const int *count, int need, int &seen
     g_wait_ticks += (int)(wall_clock64() - t0_);
 #endif
 }
+// Take the next job.  Jobs are (plane chunk, band) in band-major order, so the job a block waits for
+// always holds an earlier ticket of the same queue: it is running or finished.  With many (batch, group)
+// pairs there is one queue per XCD (blocks are dealt round-robin to the XCDs, each with its own L2),
+// holding the pairs congruent to it, so that all chunks and bands of a pair - they stream the same B/C
+// planes - run on one XCD as in the whole-plane schedule; a block whose own queue is empty takes from
+// the next one.  Returns false when no job is left (every block makes at most nQueues draws).
+__device__ __forceinline__ bool draw_job(int *sync, int nPairs, int nChunks, int nBands, int nQ, int &pair, int &chunk,
+                                         int &band) {
+    __shared__ int sJob[2];
+    if (threadIdx.x == 0) {
+        int q = blockIdx.x & (nQ - 1), t = -1;
+        for (int k = 0; k < nQ; ++k) {
+            const int jobs = ((nPairs - q + nQ - 1) / nQ) * nChunks * nBands;
+            if (jobs > 0) {
+                const int got = __hip_atomic_fetch_add(sync + kTicketWord + q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (got < jobs) { t = got; break; }
+            }
+            q = (q + 1) & (nQ - 1);
+        }
+        sJob[0] = t;
+        sJob[1] = q;
+    }
+    __syncthreads();
+    const int t = sJob[0], q = sJob[1];
+    if (t < 0) return false;
+    const int per_band = ((nPairs - q + nQ - 1) / nQ) * nChunks;
+    band = t / per_band;
+    const int r = t - band * per_band;
+    pair = (r / nChunks) * nQ + q;
+    chunk = r - (r / nChunks) * nChunks;
+    return true;
+}
+__host__ inline int job_queues(int nPairs) { return nPairs >= 16 ? 8 : 1; }
 // Enqueue a fill kernel that zeroes n int32 words (defined with the C entry points).
 int zero_words(int *p, int64_t n, hipStream_t stream);
 // How a launch is scheduled (snd_fwd_params::schedule): one block per plane chunk walking all its
 // strips, or one block per strip with the strips of a plane pipelined.
-enum { kSchedAuto = 0, kSchedPlane = 1, kSchedStrips = 2 };
+enum { kSchedAuto = 0, kSchedPlane = 1, kSchedStrips = 2, kSchedBands = 3 };
 // Strip pipelining pays when there are fewer whole-plane blocks than CUs (256): a strip waits for
 // the strip above at every tile, which costs more than it gains once the planes alone fill the chip
 // (measured at 768 plane blocks of 7x7 tiles: 2.2x slower forward, 1.3x slower backward).
@@ -270,6 +308,27 @@ __host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int n
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return false;
     if (schedule == kSchedStrips) return true;
     return planeBlocks < 128 || (planeBlocks < 256 && nStrips >= 16);
+}
+
+// The backward holds two blocks per CU (512 slots on 256 CUs).  With more plane chunks than slots
+// the last round of whole-plane blocks leaves slots idle (768 chunks: two rounds, the second half
+// empty); cutting every plane into a few bands of strips, handed over like strips but only at band
+// ends, lets the ticket order pack them (768 x 2 bands: three rounds of half the length).  Returns the
+// number of jobs per plane chunk: 0 = whole planes, nStrips = one strip per job.
+__host__ inline int bwd_band_count(int schedule, int64_t planeBlocks, int nStrips, const void *sync) {
+    if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return 0;
+    if (schedule == kSchedStrips) return nStrips;
+    if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync)) return nStrips;
+    constexpr int64_t kSlots = 512;
+    int best = 1;
+    double best_cost = 0.0;
+    for (int nb = 1; nb <= 4 && nb <= nStrips; ++nb) {
+        // rounds of jobs of length 1/nb, a few percent per extra band for the hand-over
+        const double cost = (double)((planeBlocks * nb + kSlots - 1) / kSlots) / nb * (1.0 + 0.03 * (nb - 1));
+        if (nb == 1 || cost < best_cost * 0.95) { best = nb; best_cost = cost; }
+    }
+    if (schedule == kSchedBands) return best > 1 ? best : 2;
+    return (planeBlocks >= kSlots / 2 && best > 1) ? best : 0;
 }
 
 // Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging

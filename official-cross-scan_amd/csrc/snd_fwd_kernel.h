@@ -58,18 +58,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
     if (PIPE) {
-        __shared__ int sTicket;
-        if (threadIdx.x == 0) sTicket = __hip_atomic_fetch_add(sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        // tickets run strip-major (all plane chunks' strip 0, then every strip 1, ...): a job's
-        // predecessor holds an earlier ticket, and a strip only takes a slot about when it can start
+        // jobs are single strips, drawn top strip first
+        if (!draw_job(sync, sh.batch * G, nChunks, geo.nCY, geo.nQueues, pair, chunk, I_begin)) return;
         const int nPC = sh.batch * G * nChunks;
-        const int pc = sTicket % nPC;
-        I_begin = sTicket / nPC;
-        if (I_begin >= geo.nCY) return;
+        const int pc = pair * nChunks + chunk;
         I_end = I_begin + 1;
-        pair = pc / nChunks;
-        chunk = pc - pair * nChunks;
+        (void)nPC;
         progress = sync + kSyncHeader + pc * geo.nCY;
 #ifdef SND_PIPE_TRACE
         trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_begin);
@@ -390,10 +384,13 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
         const int grid = (int)(nPC * geo.nCY);
+        Geo gs = geo;
+        gs.nBands = geo.nCY;
+        gs.nQueues = job_queues(sh.batch * sh.n_groups);
         if (p.x != nullptr)
-            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
         else
-            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
         if (p.x != nullptr)

@@ -247,7 +247,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("dout"), py::arg("x"), py::arg("x_v"),
           py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0);
     m.def("set_schedule", [](int mode) {
-        TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_STRIPS, "schedule must be 0 (auto), 1 (plane) or 2 (strips)");
+        TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_BANDS, "schedule must be 0 (auto), 1 (plane), 2 (strips) or 3 (bands, backward)");
         g_schedule = mode;
     }, "Force how fwd/bwd map work to blocks: 0 auto, 1 one block per plane chunk, 2 pipelined row strips");
 }

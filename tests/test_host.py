@@ -59,7 +59,7 @@ def test_plan_geometry(H, W, ncx, ncy):
     planes = 2 * 8 * 16
     assert plan.x_elems == planes * ncx * plan.x_inner == plan.x_sd_elems
     assert plan.x_v_elems == planes * ncy * plan.xv_inner
-    sync_words = (4 + 2 * 4 * 1 * ncy + 3) // 4 * 4         # header + (batch * groups * chunks) * strips
+    sync_words = (12 + 2 * 4 * 1 * ncy + 3) // 4 * 4        # header + (batch * groups * chunks) * strips
     assert plan.fwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
     assert plan.auto_schedule == (capi.SCHED_STRIPS if ncy > 1 else capi.SCHED_PLANE)   # 8 plane chunks only
     assert plan.bwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
@@ -108,7 +108,7 @@ def test_address_range_limits_are_status_codes():
             setattr(fp, k, v)
         return fp
 
-    assert lib.snd_fwd(C.byref(params(schedule=3)), None) == -2                  # unknown schedule
+    assert lib.snd_fwd(C.byref(params(schedule=4)), None) == -2                  # unknown schedule
     assert lib.snd_fwd(C.byref(params(directions=2)), None) == -2                # unknown directions
     assert lib.snd_fwd(C.byref(params(u_h_stride=2)), None) == -4                # rows overlap
     assert lib.snd_fwd(C.byref(params(u_h_stride=1 << 21)), None) == -4          # row pitch >= 2^23 bytes
