@@ -44,6 +44,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     __shared__ __align__(16) float sDl[CB * DLP];
     __shared__ __align__(16) float sDu[CB * kTile];  // delta' * u
     __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s + bu/4)
+    // out of up to four consecutive tiles of a strip (two in the 8-state kernels, whose blocks have
+    // less LDS each), flushed together: a 32-byte run per tile row is a partial line write (measured:
+    // 13 % of the kernel for 154 MB at c1), four tiles make whole lines
+    constexpr int QT = NP == 16 ? 4 : 2, QC = QT * kCkX;
+    constexpr int OROW = NP == 16 ? QC + 8 : QC, OCH = kRows * OROW + (NP == 16 ? 16 : 8);   // padded against bank conflicts
+    __shared__ float sOut[CB * OCH];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -104,7 +110,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     // row pitches / state strides in bytes
     constexpr int ESZ = (int)sizeof(T);
     const uint32_t cUb = (uint32_t)(p.u_shared ? cc - g * rg : cc) * (uint32_t)p.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)p.delta_d_stride * ESZ;
-    const uint32_t cOb = (uint32_t)cc * (uint32_t)p.out_d_stride * esz_out;
     const int BhB = (int)p.B_h_stride * ESZ, ChB = (int)p.C_h_stride * ESZ, UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ;
     const int OhB = (int)p.out_h_stride * esz_out;
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
@@ -347,17 +352,44 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             __syncthreads();
             if (PIPE) strip_signal(progress + I);   // tile J is handed over to the strip below
 
-            // ---- out = D*u + y, written by the thread that staged the pixel
+            // ---- out = D*u + y: finished by the thread that staged the pixel, parked in LDS
             SND_THREAD_MAPS(NP);
+            const int jq = J % QT;
+            if (geo.nCX <= 2) {                     // narrow planes: nothing to gather, write directly
+                const uint32_t cOb = (uint32_t)cc * (uint32_t)p.out_d_stride * esz_out;
+#pragma unroll
+                for (int k = 0; k < NPX; ++k) {
+                    const int pp = n + NP * k;
+                    const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
+                    if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
+                        st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                }
+                return;
+            }
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
-                const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-                if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
-                    st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                if ((pp >> 3) < TE && (pp & 7) < TE)
+                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = sY[cl * kTile + pp] + dukeep[k];
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
+            if (jq == QT - 1 || J == geo.nCX - 1) {
+                // ---- and written out once per QT tiles: consecutive lanes, consecutive columns
+                __syncthreads();
+                const int c0 = (J - jq) * TE, ncols = min((jq + 1) * TE, W - c0);
+                constexpr int PER_CH = kRows * QC;
+#pragma unroll 4
+                for (int idx = tid; idx < CB * PER_CH; idx += 16 * NP) {
+                    const int ch = idx / PER_CH, rr = (idx / QC) & 7, c32 = idx & (QC - 1);
+                    const int row = r0 + rr;
+                    if (rr < TE && row < H && c32 < ncols && cbase + ch < cend) {
+                        const uint32_t o = (uint32_t)(cbase + ch) * (uint32_t)p.out_d_stride * esz_out;
+                        st_f32_b(outb, o + mad24(mrow(row), OhB, mcol(c0 + c32) << sh_out), p.out_dtype, sOut[ch * OCH + rr * OROW + c32]);
+                    }
+                }
+                // the next write of sOut is behind the next tile's barriers
+            }
         };
         if (PAIR) {
             for (int J = 0; J < geo.nCX; J += 2) {
