@@ -73,7 +73,8 @@ typedef struct snd_plan {
                                                   (16-byte aligned, uninitialised; one row per plane) */
     int32_t auto_schedule;                     /* what SND_SCHED_AUTO resolves to in the forward for this shape
                                                   (PLANE or STRIPS): a caller may skip the fwd workspace for PLANE */
-    int32_t reserved_;
+    int32_t auto_bwd_jobs;                     /* jobs per plane chunk SND_SCHED_AUTO gives the backward: 0 = one
+                                                  block per plane chunk, n_chunks_y = one per strip, 2-4 = bands */
 } snd_plan;
 
 /* How a launch maps work to blocks.  The reference has one fixed mapping (one block per

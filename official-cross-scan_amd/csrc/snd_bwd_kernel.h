@@ -615,7 +615,7 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
     constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = WPB;
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
-    const int bands = bwd_band_count(p.f.schedule, nPC, geo.nCY, p.workspace);   // 0: one block per plane chunk
+    const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace);   // 0: one block per plane chunk
     const bool pipe = bands > 0;
     // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
     static bool configured[2][64] = {};

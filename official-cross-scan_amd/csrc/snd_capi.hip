@@ -116,7 +116,8 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
     plan->auto_schedule = snd::use_strip_pipeline(SND_SCHED_AUTO, plane_chunks(*shape), g.nCY, plan) ? SND_SCHED_STRIPS
                                                                                                    : SND_SCHED_PLANE;
-    plan->reserved_ = 0;
+    plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
+                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan);
     return SND_OK;
 }
 

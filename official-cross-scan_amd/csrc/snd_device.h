@@ -315,20 +315,25 @@ __host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int n
 // empty); cutting every plane into a few bands of strips, handed over like strips but only at band
 // ends, lets the ticket order pack them (768 x 2 bands: three rounds of half the length).  Returns the
 // number of jobs per plane chunk: 0 = whole planes, nStrips = one strip per job.
-__host__ inline int bwd_band_count(int schedule, int64_t planeBlocks, int nStrips, const void *sync) {
+__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync) {
+    const int64_t planeBlocks = nPairs * nChunks;
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return 0;
     if (schedule == kSchedStrips) return nStrips;
     if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync)) return nStrips;
     constexpr int64_t kSlots = 512;
+    // whole planes: every (batch, group) pair is pinned to one XCD (64 slots), so the rounds are those of
+    // the fullest XCD (340 pairs x 3 chunks: 129 blocks there, three rounds for 1020 blocks)
     int best = 1;
-    double best_cost = 0.0;
-    for (int nb = 1; nb <= 4 && nb <= nStrips; ++nb) {
-        // rounds of jobs of length 1/nb, a few percent per extra band for the hand-over
-        const double cost = (double)((planeBlocks * nb + kSlots - 1) / kSlots) / nb * (1.0 + 0.03 * (nb - 1));
-        if (nb == 1 || cost < best_cost * 0.95) { best = nb; best_cost = cost; }
+    double best_cost = (double)(((nPairs + 7) / 8 * nChunks + kSlots / 8 - 1) / (kSlots / 8));
+    for (int nb = 2; nb <= 4 && nb <= nStrips; ++nb) {
+        // rounds of jobs of length 1/nb (drawn from queues that balance the XCDs), never less than the
+        // chain of one plane's bands, and a few percent per extra band for the hand-over
+        double cost = (double)((planeBlocks * nb + kSlots - 1) / kSlots) / nb;
+        cost = (cost < 1.0 ? 1.0 : cost) * (1.0 + 0.03 * (nb - 1));
+        if (cost < best_cost * 0.95) { best = nb; best_cost = cost; }
     }
     if (schedule == kSchedBands) return best > 1 ? best : 2;
-    return (planeBlocks >= kSlots / 2 && best > 1) ? best : 0;
+    return best > 1 ? best : 0;
 }
 
 // Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging

@@ -29,7 +29,7 @@ def test_struct_layouts_match_header_sizes():
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
-    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule"]),
+    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs"]),
               ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared"]),
               ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
@@ -156,6 +156,24 @@ def test_cross_scan_host_helpers():
     assert torch.allclose(cs.cross_merge(xs, w), 10 * x)
     wc = torch.arange(12, dtype=torch.float32).reshape(4, 3)
     assert torch.allclose(cs.cross_merge(xs, wc), x * wc.sum(0).reshape(1, 3, 1, 1))
+
+
+def test_backward_job_split():
+    """What AUTO gives the backward: whole planes, one job per strip (few plane chunks), or a few bands
+    of strips when the plane chunks do not fill the chip's 512 block slots evenly."""
+    def jobs(Bt, Dm, H, W, K=4):
+        st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, 16, K, Dm, capi.SND_F32))
+        assert st == 0
+        return plan.auto_bwd_jobs, plan.n_chunks_y
+    assert jobs(64, 192, 56, 56) == (2, 7)        # 768 plane chunks: two rounds, the second half empty -> two bands
+    assert jobs(64, 768, 14, 14) == (0, 2)        # 3072 chunks = six full rounds
+    assert jobs(2, 192, 200, 336) == (25, 25)     # 24 chunks: one job per strip
+    assert jobs(1, 256, 512, 512) == (64, 64)
+    assert jobs(43, 192, 56, 56) == (3, 7)        # 516 chunks: 4 rounds of a third instead of 2 whole ones
+    assert jobs(64, 192, 8, 56) == (0, 1)         # a single strip cannot be split
+    assert jobs(32, 192, 56, 56) == (0, 7)        # 384 chunks are all resident at once: a plane's bands are a chain
+    assert jobs(85, 192, 56, 56) == (2, 7)        # 1020 chunks, but 129 of them pinned to each of four XCDs: 3 rounds
+    assert jobs(128, 192, 56, 56) == (0, 7)       # 1536 chunks: three full rounds
 
 
 def test_tile_extent_choice():
