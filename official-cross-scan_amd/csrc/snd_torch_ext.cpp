@@ -194,13 +194,20 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     const auto f32 = u.options().dtype(at::ScalarType::Float);
     at::Tensor du = torch::empty({batch_size, dim, nrows, ncols}, u.options());
     at::Tensor ddelta = torch::empty({batch_size, dim, nrows, ncols}, u.options());
-    at::Tensor dA = torch::zeros({dim, dstate}, f32);
-    at::Tensor dB = torch::zeros(B.sizes(), f32);
-    at::Tensor dC = torch::zeros(C.sizes(), f32);
+    // the accumulated gradients (zero-filled as host.cpp:395-403 does) are carved out of one buffer,
+    // so that one fill kernel clears them all
+    const int64_t nA = (int64_t)dim * dstate, nBC = B.numel();
+    auto round64 = [](int64_t v) { return (v + 63) / 64 * 64; };
+    const int64_t oB = round64(nA), oC = oB + round64(nBC), oD = oC + round64(nBC), oBias = oD + round64(dim),
+                  oDec = oBias + round64(dim);
+    at::Tensor acc = torch::zeros({oDec + 64}, f32);
+    at::Tensor dA = acc.narrow(0, 0, nA).view({dim, dstate});
+    at::Tensor dB = acc.narrow(0, oB, nBC).view(B.sizes());
+    at::Tensor dC = acc.narrow(0, oC, nBC).view(C.sizes());
     at::Tensor dD, ddelta_bias, dA_decay;
-    if (D_.has_value()) dD = torch::zeros({dim}, f32);
-    if (delta_bias_.has_value()) ddelta_bias = torch::zeros({dim}, f32);
-    if (A_decay_.has_value()) dA_decay = torch::zeros({1}, f32);
+    if (D_.has_value()) dD = acc.narrow(0, oD, dim);
+    if (delta_bias_.has_value()) ddelta_bias = acc.narrow(0, oBias, dim);
+    if (A_decay_.has_value()) dA_decay = acc.narrow(0, oDec, 1);
     at::Tensor ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
 
     snd_bwd_params p;
