@@ -72,7 +72,7 @@ typedef struct snd_plan {
     int64_t fwd_workspace_bytes;               /* scratch fwd uses when it splits planes into strips
                                                   (16-byte aligned, uninitialised; one row per plane) */
     int32_t auto_schedule;                     /* what SND_SCHED_AUTO resolves to in the forward for this shape
-                                                  (PLANE or STRIPS): a caller may skip the fwd workspace for PLANE */
+                                                  (PLANE, STRIPS or BANDS): a caller may skip the fwd workspace for PLANE */
     int32_t auto_bwd_jobs;                     /* jobs per plane chunk SND_SCHED_AUTO gives the backward: 0 = one
                                                   block per plane chunk, n_chunks_y = one per strip, 2-4 = bands */
 } snd_plan;
@@ -82,10 +82,10 @@ typedef struct snd_plan {
  *   PLANE   one block per (batch, group, 16-channel chunk) walks the whole plane;
  *   STRIPS  one block per 8-row strip of such a chunk, the strips of a plane pipelined one tile
  *           apart (for few, large planes: c3/c4-like shapes).  Needs the workspace.
- *   BANDS   backward only (the forward treats it as AUTO): one block per band of consecutive strips,
- *           2-4 bands per plane, handed over like strips but only at band ends.  For more plane
- *           chunks than the chip holds blocks at once (c1: 768 chunks, 512 slots), where whole-plane
- *           blocks leave the last round half empty. */
+ *   BANDS   one block per band of consecutive strips, 2-4 bands per plane, handed over like strips but
+ *           only at band ends.  For more plane chunks than the chip holds blocks at once (c1 backward:
+ *           768 chunks, 512 slots), where whole-plane blocks leave the last round half empty.  Needs
+ *           the workspace. */
 typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2, SND_SCHED_BANDS = 3 } snd_schedule;
 
 /* Scan origin per group.  The reference scans every group from the top-left corner and leaves the

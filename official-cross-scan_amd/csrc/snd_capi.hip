@@ -114,8 +114,9 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);
     plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
-    plan->auto_schedule = snd::use_strip_pipeline(SND_SCHED_AUTO, plane_chunks(*shape), g.nCY, plan) ? SND_SCHED_STRIPS
-                                                                                                   : SND_SCHED_PLANE;
+    const int fwd_jobs = snd::fwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
+                                             (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
+    plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
     plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
                                               (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan);
     return SND_OK;
@@ -137,7 +138,7 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
         snd_make_plan(&params->shape, &plan);
         if (params->workspace_bytes < plan.fwd_workspace_bytes) return SND_ERR_WORKSPACE;
         if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
-    } else if (params->schedule == SND_SCHED_STRIPS) {
+    } else if (params->schedule == SND_SCHED_STRIPS || params->schedule == SND_SCHED_BANDS) {
         return SND_ERR_WORKSPACE;
     }
     switch (params->shape.in_dtype) {

@@ -310,30 +310,36 @@ __host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int n
     return planeBlocks < 128 || (planeBlocks < 256 && nStrips >= 16);
 }
 
-// The backward holds two blocks per CU (512 slots on 256 CUs).  With more plane chunks than slots
-// the last round of whole-plane blocks leaves slots idle (768 chunks: two rounds, the second half
-// empty); cutting every plane into a few bands of strips, handed over like strips but only at band
-// ends, lets the ticket order pack them (768 x 2 bands: three rounds of half the length).  Returns the
-// number of jobs per plane chunk: 0 = whole planes, nStrips = one strip per job.
-__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync) {
+// Jobs per plane chunk: 0 = one block walks the whole plane, nStrips = one strip per job, 2-4 = bands of
+// strips.  A kernel holds `slots` blocks at once on the 256 CUs (backward 512; forward 768, or 1536 with
+// the 128-thread blocks of the 8-state kernels).  With more plane chunks than slots the last round of
+// whole-plane blocks leaves slots idle (backward, 768 chunks: two rounds, the second half empty);
+// cutting every plane into a few bands of strips, handed over like strips but only at band ends, lets
+// the ticket order pack them (768 x 2 bands: three rounds of half the length).
+__host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int64_t slots) {
     const int64_t planeBlocks = nPairs * nChunks;
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return 0;
     if (schedule == kSchedStrips) return nStrips;
     if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync)) return nStrips;
-    constexpr int64_t kSlots = 512;
-    // whole planes: every (batch, group) pair is pinned to one XCD (64 slots), so the rounds are those of
-    // the fullest XCD (340 pairs x 3 chunks: 129 blocks there, three rounds for 1020 blocks)
+    // whole planes: every (batch, group) pair is pinned to one XCD (an eighth of the slots), so the rounds
+    // are those of the fullest XCD (backward, 340 pairs x 3 chunks: 129 blocks there, three rounds)
     int best = 1;
-    double best_cost = (double)(((nPairs + 7) / 8 * nChunks + kSlots / 8 - 1) / (kSlots / 8));
+    double best_cost = (double)(((nPairs + 7) / 8 * nChunks + slots / 8 - 1) / (slots / 8));
     for (int nb = 2; nb <= 4 && nb <= nStrips; ++nb) {
         // rounds of jobs of length 1/nb (drawn from queues that balance the XCDs), never less than the
         // chain of one plane's bands, and a few percent per extra band for the hand-over
-        double cost = (double)((planeBlocks * nb + kSlots - 1) / kSlots) / nb;
+        double cost = (double)((planeBlocks * nb + slots - 1) / slots) / nb;
         cost = (cost < 1.0 ? 1.0 : cost) * (1.0 + 0.03 * (nb - 1));
         if (cost < best_cost * 0.95) { best = nb; best_cost = cost; }
     }
     if (schedule == kSchedBands) return best > 1 ? best : 2;
     return best > 1 ? best : 0;
+}
+__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync) {
+    return band_count(schedule, nPairs, nChunks, nStrips, sync, 512);
+}
+__host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate) {
+    return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 768 : 1536);
 }
 
 // Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging

@@ -64,11 +64,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
     if (PIPE) {
-        // jobs are single strips, drawn top strip first
-        if (!draw_job(sync, sh.batch * G, nChunks, geo.nCY, geo.nQueues, pair, chunk, I_begin)) return;
+        // A job is a band of consecutive strips (one strip each in the fully pipelined case), drawn
+        // top band first; band k covers strips ceil(k*nCY/nBands) .. ceil((k+1)*nCY/nBands)-1.
+        int band;
+        if (!draw_job(sync, sh.batch * G, nChunks, geo.nBands, geo.nQueues, pair, chunk, band)) return;
         const int nPC = sh.batch * G * nChunks;
         const int pc = pair * nChunks + chunk;
-        I_end = I_begin + 1;
+        I_begin = (band * geo.nCY + geo.nBands - 1) / geo.nBands;
+        I_end = ((band + 1) * geo.nCY + geo.nBands - 1) / geo.nBands;
         (void)nPC;
         progress = sync + kSyncHeader + pc * geo.nCY;
 #ifdef SND_PIPE_TRACE
@@ -180,9 +183,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         load_tile(st0, I, J);
         if (PAIR && J + 1 < geo.nCX) load_tile(st1, I, J + 1);
     };
-    // h of the row above tile (I, J), one tile ahead (whole-plane schedule)
+    // h of the row above tile (I, J), one tile ahead, where this block wrote it itself (whole-plane
+    // schedule; every strip of a pipelined band but its first)
     auto prefetch_xv = [&](int I, int J) {
-        if (!PIPE && I > 0 && geo.nCX > 1) {        // with one column tile the row comes from registers
+        if ((!PIPE || I > I_begin) && I > 0 && geo.nCX > 1) {   // with one column tile the row comes from registers
             const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
             const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
@@ -202,13 +206,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                              (int64_t)b * geo.nCX * DN8 + ((int64_t)cc * N + nn) * 2
                        : nullptr;
     float xv_last = 0.f;
-    auto fetch_row_above = [&](int I, int J) {
-        if (I == 0) return;
+    auto fetch_row_above = [&](int J, float (&row)[kCkX]) {
         const float *src = hrow + (int64_t)J * DN8;
-        qcorner = J > 0 ? xv_last : 0.f;
 #pragma unroll
-        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, qxv[k], qxv[k + 1]);
-        xv_last = qxv[TE - 1];
+        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, row[k], row[k + 1]);
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&](const Stage &q) {
@@ -248,14 +249,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
         auto do_tile = [&](const int J, const Stage &mine, const bool last_of_pair) {
             const int j0 = J * TE;
             commit(mine);
-            if (PIPE && I > 0 && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
+            // first strip of a pipelined band: the row above comes from another block
+            const bool handed = PIPE && I == I_begin && I > 0;
+            if (handed && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
             __syncthreads();
             // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
-            // registers), handed over in registers, or - strip pipeline - fetched here
+            // registers), handed over in registers, or - from another block - fetched here
             float hup[kCkX], aup[kCkX];
             float corner = 0.f;                     // h[r0-1][j0-1]
-            if (PIPE) fetch_row_above(I, J);
-            if (!PIPE) {
+            if (handed) {
+                fetch_row_above(J, hup);
+            } else {
                 corner = (I > 0) ? qcorner : 0.f;
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
@@ -268,10 +272,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     if (last_of_pair) load_pair(In, Jn);
                 }
             }
-            if (PIPE) {
-                corner = (I > 0) ? qcorner : 0.f;
-#pragma unroll
-                for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
+            if (handed) {                           // the corner is the previous fetch's last column
+                corner = J > 0 ? xv_last : 0.f;
+                xv_last = hup[TE - 1];
             }
 
             // ---- per-lane tile walk
@@ -324,7 +327,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     }
                 }
             }
-            if (!PIPE && geo.nCX == 1) {            // the next strip's row above is this tile's last row
+            if (geo.nCX == 1 && I + 1 < I_end) {    // the next strip's row above is this tile's last row
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];
                 qcorner = 0.f;
@@ -334,13 +337,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
                 st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
                 st4_stream(dst + 4, hup[4], hup[5], hup[6], hup[7]);
-                if (PIPE && I + 1 < geo.nCY) {      // and the hand-over copy for the strip below
+                if (PIPE && I + 1 == I_end && I + 1 < geo.nCY) {   // and the hand-over copy for the block of the strip below
                     float *ho = hrow + (int64_t)J * DN8;
 #pragma unroll
                     for (int k = 0; k < kCkX; k += 2) st2_coherent(ho + (k >> 1) * DN2, hup[k], hup[k + 1]);
                 }
             }
-            if (PIPE) strip_stores_done();
+            const bool hands_over = PIPE && I + 1 == I_end && I + 1 < geo.nCY;
+            if (hands_over) strip_stores_done();
             if (lvalid && SAVE && J + 1 < geo.nCX) {   // column checkpoints: only if a tile follows
                 float *dh = xh + ((int64_t)J * geo.nCY + I) * DN8;
                 float *ds = xs + ((int64_t)J * geo.nCY + I) * DN8;
@@ -350,7 +354,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 st4_stream(ds + 4, sl[4], sl[5], sl[6], sl[7]);
             }
             __syncthreads();
-            if (PIPE) strip_signal(progress + I);   // tile J is handed over to the strip below
+            if (hands_over) strip_signal(progress + I);   // tile J is handed over to the strip below
 
             // ---- out = D*u + y: finished by the thread that staged the pixel, parked in LDS
             SND_THREAD_MAPS(NP);
@@ -412,12 +416,13 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
-    if (use_strip_pipeline(p.schedule, nPC, geo.nCY, p.workspace)) {
+    const int bands = fwd_band_count(p.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate);
+    if (bands > 0) {
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
-        const int grid = (int)(nPC * geo.nCY);
+        const int grid = (int)(nPC * bands);
         Geo gs = geo;
-        gs.nBands = geo.nCY;
+        gs.nBands = bands;
         gs.nQueues = job_queues(sh.batch * sh.n_groups);
         if (p.x != nullptr)
             hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);

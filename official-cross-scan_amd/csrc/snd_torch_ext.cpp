@@ -150,7 +150,8 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     // allocator in stream order
     p.schedule = g_schedule;
     at::Tensor ws;
-    if (g_schedule == SND_SCHED_STRIPS || (g_schedule == SND_SCHED_AUTO && c.plan.auto_schedule == SND_SCHED_STRIPS)) {
+    if (g_schedule == SND_SCHED_STRIPS || g_schedule == SND_SCHED_BANDS ||
+        (g_schedule == SND_SCHED_AUTO && c.plan.auto_schedule != SND_SCHED_PLANE)) {
         ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
         p.workspace = ws.data_ptr();
         p.workspace_bytes = c.plan.fwd_workspace_bytes;

@@ -50,10 +50,8 @@ def test_strips_match_plane_and_oracle(gpu_device, Bt, Dm, H, W, N, K, dtype):
         b.ws.view(torch.int32)[:16] = 0x7fffffff
         b.launch()
         torch.cuda.synchronize()
-        if sched == capi.SCHED_STRIPS:
-            assert sync_error(f.ws) == 0, "a strip wait ran into its poll limit"
         if sched != capi.SCHED_PLANE:
-            assert sync_error(b.ws) == 0, "a strip wait ran into its poll limit"
+            assert sync_error(f.ws) == 0 and sync_error(b.ws) == 0, "a strip wait ran into its poll limit"
         res[sched] = (f.out, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias], (f.x, f.x_v, f.x_sd))
     out_p, g_p, st_p = res[capi.SCHED_PLANE]
     out_s, g_s, st_s = res[capi.SCHED_STRIPS]
