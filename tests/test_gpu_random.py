@@ -21,7 +21,7 @@ def draw(seed):
     rg = int(r.choice([1, 3, 4, 16, 20]))
     c = dict(Bt=int(r.randint(1, 4)), K=K, Dm=K * rg, H=int(r.randint(1, MAX_HW + 1)), W=int(r.randint(1, MAX_HW + 1)),
              N=int(r.choice([1, 2, 3, 4, 7, 8, 9, 12, 16])), dt=int(r.choice([0, 0, 1, 2])),
-             sched=int(r.choice([0, 1, 2])), dirs=int(r.choice([0, 1])), softplus=bool(r.randint(2)),
+             sched=int(r.choice([0, 1, 2, 3])), dirs=int(r.choice([0, 1])), softplus=bool(r.randint(2)),
              has_D=bool(r.randint(2)), has_bias=bool(r.randint(2)), has_decay=bool(r.randint(4) == 0),
              out_float=bool(r.randint(2)), share_delta=bool(r.randint(3) == 0))
     if not c["softplus"]:
@@ -57,7 +57,7 @@ def test_random_case(gpu_device, seed):
     g = capi.bwd(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, dout, f.x, f.x_v, c["softplus"], dec, f.x_sd,
                  None, c["sched"], c["dirs"])
     torch.cuda.synchronize()
-    strips = c["sched"] == capi.SCHED_STRIPS or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule == capi.SCHED_STRIPS)
+    strips = c["sched"] in (capi.SCHED_STRIPS, capi.SCHED_BANDS) or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule != capi.SCHED_PLANE)
     if strips and f.plan.n_chunks_y > 1:                   # a single strip always runs as a whole plane
         assert int(f.ws.view(torch.int32)[1]) == 0         # no strip wait gave up
 
