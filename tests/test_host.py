@@ -176,6 +176,20 @@ def test_backward_job_split():
     assert jobs(128, 192, 56, 56) == (0, 7)       # 1536 chunks: three full rounds
 
 
+def test_forward_job_split():
+    """The forward holds 768 blocks at once (1536 with the 8-state kernels' smaller blocks)."""
+    def sched(Bt, Dm, H, W, N=16, K=4):
+        st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, N, K, Dm, capi.SND_F32))
+        assert st == 0
+        return plan.auto_schedule
+    assert sched(64, 192, 56, 56) == capi.SCHED_PLANE     # 768 plane chunks on 768 slots
+    assert sched(70, 192, 56, 56) == capi.SCHED_BANDS     # 840: a second round for 72 blocks otherwise
+    assert sched(128, 192, 56, 56) == capi.SCHED_PLANE    # 1536: two full rounds
+    assert sched(70, 192, 56, 56, N=8) == capi.SCHED_PLANE   # 840 of 1536 slots
+    assert sched(2, 192, 200, 336) == capi.SCHED_STRIPS
+    assert sched(70, 192, 8, 56) == capi.SCHED_PLANE      # one strip
+
+
 def test_tile_extent_choice():
     """7x7 tiles where they leave clearly fewer padded cells (the 14 / 28 / 7 stage sizes), else 8x8."""
     def tiles(H, W):
