@@ -170,15 +170,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const int64_t HW4 = (int64_t)H * W * 4;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the wave index as a scalar
 
-    // saved state and scratch, tile-major with the lane's 8 values innermost (as the forward writes):
-    //   x_v [b][I][J][c][n][8 cols]   x, x_sd [b][J][I][c][n][8 rows]   scratch G row [b][J][c][n][8 cols]
+    // saved state and scratch, tile-major; inside a tile the lanes' values 0-3, then the lanes' values
+    // 4-7 (as the forward writes: a wave's 16-byte accesses cover whole lines):
+    //   x_v [b][I][J][half][c][n][4 cols]   x, x_sd [b][J][I][half][c][n][4 rows]   scratch G row [b][J][half][c][n][4 cols]
     const int64_t DN8 = (int64_t)Dm * N * 8;
-    const int64_t lane_off = ((int64_t)cc * N + nn) * 8;
+    const int64_t DN4 = DN8 / 2;
+    const int64_t lane_off = ((int64_t)cc * N + nn) * 4;
     const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
     const float *xh = f.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
     const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
-    // whole-plane schedule: [J][c][n][8 cols]; strip schedule: [J][pair k][c][n][2], so that a wave's
-    // 8-byte coherent accesses cover whole lines
+    // hand-over between blocks (pipelined schedules): [J][pair k][c][n][2], so that a wave's 8-byte
+    // coherent accesses cover whole lines too
     const int64_t DN2 = (int64_t)Dm * N * 2;
     float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + (PIPE ? ((int64_t)cc * N + nn) * 2 : lane_off);
 
@@ -296,18 +298,19 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             float Gd[kCkX];                                        // G of the row below
             if (I > 0) {
                 const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
-                const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                const float4 v0 = *(const float4 *)src, v1 = *(const float4 *)(src + DN4);
                 hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
                 hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
-                if (J > 0) hc = src[TE - 1 - DN8];          // last column of the tile on the left
+                if (J > 0) hc = src[((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8];   // last column of the tile on the left
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
             if (J > 0) {
-                const float4 *sh_ = (const float4 *)(xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
-                const float4 *ss_ = (const float4 *)(xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8);
-                const float4 h0 = sh_[0], h1 = sh_[1], s0 = ss_[0], s1 = ss_[1];
+                const float *sh_ = xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8;
+                const float *ss_ = xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8;
+                const float4 h0 = *(const float4 *)sh_, h1 = *(const float4 *)(sh_ + DN4);
+                const float4 s0 = *(const float4 *)ss_, s1 = *(const float4 *)(ss_ + DN4);
                 hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
                 hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
                 slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                         for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
                     } else {
-                        const float4 v0 = ((const float4 *)src)[0], v1 = ((const float4 *)src)[1];
+                        const float4 v0 = *(const float4 *)src, v1 = *(const float4 *)(src + DN4);
                         Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
                         Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
                     }
@@ -526,8 +529,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                     for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
                 } else {
-                    ((float4 *)dst)[0] = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
-                    ((float4 *)dst)[1] = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
+                    *(float4 *)dst = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
+                    *(float4 *)(dst + DN4) = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
                 }
             }
             if (hands_over) strip_stores_done();

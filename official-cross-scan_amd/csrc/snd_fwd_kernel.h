@@ -118,11 +118,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the wave index as a scalar
 
-    // saved state, tile-major with the lane's 8 values innermost, so that each lane moves 32
-    // contiguous bytes and a wave's 64 planes one contiguous 2 KB run:
-    //   x_v  [b][strip I][col tile J][c][n][8 cols]     x, x_sd  [b][J][I][c][n][8 rows]
+    // saved state, tile-major; inside a tile the lanes' values 0-3, then the lanes' values 4-7, so that
+    // each 16-byte store or load instruction of a wave covers one contiguous 1 KB run (whole lines):
+    //   x_v  [b][strip I][col tile J][half][c][n][4 cols]     x, x_sd  [b][J][I][half][c][n][4 rows]
     const int64_t DN8 = (int64_t)Dm * N * 8;
-    const int64_t lane_off = ((int64_t)cc * N + nn) * 8;
+    const int64_t DN4 = DN8 / 2;                    // the lane's values 0-3 of every lane, then values 4-7
+    const int64_t lane_off = ((int64_t)cc * N + nn) * 4;
     float *xv = p.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
     float *xh = SAVE ? p.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off : nullptr;
     float *xs = SAVE ? p.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off : nullptr;
@@ -188,10 +189,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     auto prefetch_xv = [&](int I, int J) {
         if ((!PIPE || I > I_begin) && I > 0 && geo.nCX > 1) {   // with one column tile the row comes from registers
             const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
-            const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + 4);
+            const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + DN4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
             qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
-            qcorner = J > 0 ? src[TE - 1 - DN8] : 0.f;      // last column of the tile on the left
+            qcorner = J > 0 ? src[((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8] : 0.f;   // last column of the tile on the left
         }
     };
     // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
@@ -336,7 +337,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
                 st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
-                st4_stream(dst + 4, hup[4], hup[5], hup[6], hup[7]);
+                st4_stream(dst + DN4, hup[4], hup[5], hup[6], hup[7]);
                 if (PIPE && I + 1 == I_end && I + 1 < geo.nCY) {   // and the hand-over copy for the block of the strip below
                     float *ho = hrow + (int64_t)J * DN8;
 #pragma unroll
@@ -349,9 +350,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                 float *dh = xh + ((int64_t)J * geo.nCY + I) * DN8;
                 float *ds = xs + ((int64_t)J * geo.nCY + I) * DN8;
                 st4_stream(dh, hl[0], hl[1], hl[2], hl[3]);
-                st4_stream(dh + 4, hl[4], hl[5], hl[6], hl[7]);
+                st4_stream(dh + DN4, hl[4], hl[5], hl[6], hl[7]);
                 st4_stream(ds, sl[0], sl[1], sl[2], sl[3]);
-                st4_stream(ds + 4, sl[4], sl[5], sl[6], sl[7]);
+                st4_stream(ds + DN4, sl[4], sl[5], sl[6], sl[7]);
             }
             __syncthreads();
             if (hands_over) strip_signal(progress + I);   // tile J is handed over to the strip below
