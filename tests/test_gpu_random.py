@@ -94,5 +94,10 @@ def test_random_case(gpu_device, seed):
         if nm == "ddelta_bias" and c["dirs"] and rep > 1:
             want = want.reshape(c["Dd"], rep).sum(1)
         tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 3e-4
+        if nm == "dA_decay" and c["H"] == 1:
+            # a single row makes h = s, so out does not depend on a: the reference is zero and relerr
+            # measures the fp32 rounding noise of a sum over every cell of every plane on its absolute
+            # scale of 1e-2 (seed 1092: 6e-6 over 11264 cells)
+            tol = 5e-3
         e = relerr(g[i].float().cpu().numpy(), np.asarray(want))
         assert e <= tol, (nm, e)
