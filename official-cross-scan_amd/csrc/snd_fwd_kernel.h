@@ -43,7 +43,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     __shared__ __align__(16) float sC[NP * NSTR];
     __shared__ __align__(16) float sDl[CB * DLP];
     __shared__ __align__(16) float sDu[CB * kTile];  // delta' * u
-    __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s + bu/4)
+    __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s)
+    // The bu/4 term of the output, sum_n C*B*delta'*u/4, is delta'*u times a per-pixel sum that all
+    // channels share: S/4 = sum_n B*C / 4 is built once per tile (per-wave partial sums at staging, added
+    // up by one wave) instead of one multiply-add per state cell.
+    __shared__ float sSp[(NP / 4) * kTile], sS[kTile];
     // out of up to four consecutive tiles of a strip (two in the 8-state kernels, whose blocks have
     // less LDS each), flushed together: a 32-byte run per tile row is a partial line write (measured:
     // 13 % of the kernel for 154 MB at c1), four tiles make whole lines
@@ -221,6 +225,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             sB[sn * NSTR + px] = q.qb[k];
             sC[sn * NSTR + px] = q.qc[k];
         }
+        {
+            float part = 0.f;
+#pragma unroll
+            for (int k = 0; k < NBC; ++k) part = fmaf(q.qb[k], q.qc[k], part);
+            sSp[wave * kTile + px] = part;
+        }
         float dsp;
 #pragma unroll
         for (int k = 0; k < NPX; ++k) {
@@ -254,6 +264,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             const bool handed = PIPE && I == I_begin && I > 0;
             if (handed && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
             __syncthreads();
+            if (wave == 0) {                        // read by the output phase, behind the next barrier
+                float t = 0.f;
+#pragma unroll
+                for (int w = 0; w < WPB; ++w) t += sSp[w * kTile + (tid & 63)];
+                sS[tid & 63] = 0.25f * t;
+            }
             // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
             // registers), handed over in registers, or - from another block - fetched here
             float hup[kCkX], aup[kCkX];
@@ -307,7 +323,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                         const float X = fmaf(-0.5f * (aup[j] + aleft), diag, hup[j]);
                         const float h = fmaf(a, left + X, bu);
                         const float s = fmaf(a, sleft, bu);
-                        y[j] = ac[q] * fmaf(0.25f, bu, h - s);
+                        y[j] = ac[q] * (h - s);
                         diag = hup[j];
                         hup[j] = h; aup[j] = a;
                         left = h; aleft = a; sleft = s;
@@ -367,7 +383,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
                     const int pp = n + NP * k;
                     const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                     if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
-                        st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype, sY[cl * kTile + pp] + dukeep[k]);
+                        st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype,
+                                 fmaf(sDu[cl * kTile + pp], sS[pp], sY[cl * kTile + pp] + dukeep[k]));
                 }
                 return;
             }
@@ -375,7 +392,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 if ((pp >> 3) < TE && (pp & 7) < TE)
-                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = sY[cl * kTile + pp] + dukeep[k];
+                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = fmaf(sDu[cl * kTile + pp], sS[pp], sY[cl * kTile + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
