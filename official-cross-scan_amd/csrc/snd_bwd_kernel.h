@@ -501,11 +501,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     }
                     {
                         // sum over the wave's channels: lane bits 4-5 by a swap reduce-scatter (the
-                        // 16-lane row q ends with column C0+q), bit 3 (8-state layout) by a row rotate
+                        // 16-lane row q ends with column C0+q), bits 3 and 2 (8- and 4-lane layouts) by row rotates
                         rows_scatter4x2(vB[0], vB[1], vB[2], vB[3], vC[0], vC[1], vC[2], vC[3]);
                         float tb = vB[0], tc = vC[0];
-                        if (NP == 8) { tb += dpp_mov<0x128>(tb); tc += dpp_mov<0x128>(tc); }   // row_ror:8
-                        if (NP == 16 || (tid & 8) == 0) {
+                        if (NP <= 8) { tb += dpp_mov<0x128>(tb); tc += dpp_mov<0x128>(tc); }   // row_ror:8
+                        if (NP <= 4) { tb += dpp_mov<0x124>(tb); tc += dpp_mov<0x124>(tc); }   // row_ror:4
+                        if ((tid & (16 - NP)) == 0) {
                             mydB[r * kCkX + C0 + qrow] = tb;
                             mydC[r * kCkX + C0 + qrow] = tc;
                         }
@@ -618,7 +619,7 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
     constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = WPB;
     constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
-    const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace);   // 0: one block per plane chunk
+    const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate);   // 0: one block per plane chunk
     const bool pipe = bands > 0;
     // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
     static bool configured[2][64] = {};
@@ -652,7 +653,8 @@ static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
 // One instantiation per input dtype, each in its own translation unit.
 template <typename T>
 int launch_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
-    return p.f.shape.dstate > 8 ? launch_bwd_np<T, 16>(p, stream) : launch_bwd_np<T, 8>(p, stream);
+    const int N = p.f.shape.dstate;
+    return N > 8 ? launch_bwd_np<T, 16>(p, stream) : N > 4 ? launch_bwd_np<T, 8>(p, stream) : launch_bwd_np<T, 4>(p, stream);
 }
 
 }  // namespace snd

@@ -118,7 +118,7 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
     plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
     plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
-                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan);
+                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
     return SND_OK;
 }
 

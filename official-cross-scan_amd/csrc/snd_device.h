@@ -153,6 +153,9 @@ template <int NP> __device__ __forceinline__ void group_sum4(float &a, float &b,
     else if (NP == 8)
         asm("s_nop 1\n\t" SND_DPP4("quad_perm:[1,0,3,2]") SND_DPP4("quad_perm:[2,3,0,1]") SND_DPP4("row_half_mirror")
             : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    else if (NP == 4)
+        asm("s_nop 1\n\t" SND_DPP4("quad_perm:[1,0,3,2]") SND_DPP4("quad_perm:[2,3,0,1]")
+            : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
     else { a = group_sum<NP>(a); b = group_sum<NP>(b); c = group_sum<NP>(c); d = group_sum<NP>(d); }
 }
 
@@ -335,8 +338,10 @@ __host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nS
     if (schedule == kSchedBands) return best > 1 ? best : 2;
     return best > 1 ? best : 0;
 }
-__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync) {
-    return band_count(schedule, nPairs, nChunks, nStrips, sync, 512);
+// Blocks per CU by the state-lane count of the kernels (16, 8 or 4 lanes per channel): the backward is held
+// to 2, 3, 4 by its LDS, the forward to 3, 6, 6.
+__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate) {
+    return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 512 : dstate > 4 ? 768 : 1024);
 }
 __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate) {
     return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 768 : 1536);

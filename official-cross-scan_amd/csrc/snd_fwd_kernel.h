@@ -31,7 +31,7 @@
 namespace snd {
 
 template <typename T, int NP, bool SAVE, bool PIPE, int TE>
-__global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
+__global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8 ? 3 : 2, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
     constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;                 // per-state pitch: lane n hits banks 4n..4n+3
@@ -143,7 +143,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
     // flight: a line is fetched from HBM twice per strip instead of four times.
     // (Only where it pays and fits: the 16-state whole-plane kernels, which are bandwidth-bound.)
     constexpr bool PAIR = NP == 16;
-    struct Stage { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo; };
+    constexpr int NHL = (kCkX + NP - 1) / NP;       // halo-row elements per thread (1; 2 with four lanes per channel)
+    struct Stage { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; };
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto load_tile = [&](Stage &q, int I, int J) {
@@ -176,11 +177,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             q.qdl[k] = ok ? vd : 0.f;
             q.qu[k] = ok ? vu : 0.f;
         }
-        q.qhalo = 0.f;
-        if (n < TE) {     // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
-            const int row = r0 - 1, col = j0 + n;
-            const float vd = ldg_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
-            q.qhalo = (cvalid && row >= 0 && col < W) ? vd : 0.f;
+#pragma unroll
+        for (int k = 0; k < NHL; ++k) {     // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
+            const int hj = n + NP * k;
+            q.qhalo[k] = 0.f;
+            if (hj < TE) {
+                const int row = r0 - 1, col = j0 + hj;
+                const float vd = ldg_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
+                q.qhalo[k] = (cvalid && row >= 0 && col < W) ? vd : 0.f;
+            }
         }
     };
     // the pair of tiles that starts at (I, J), J even (or the single tile when not pairing)
@@ -241,9 +246,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(3, 4)))
             sDu[cl * kTile + pp] = dl * q.qu[k];
             dukeep[k] = Dv * q.qu[k];
         }
-        if (n < kCkX) {
-            const float raw = q.qhalo + bias;
-            sDl[cl * DLP + n] = softplus ? softplus20(raw, dsp) : raw;
+#pragma unroll
+        for (int k = 0; k < NHL; ++k) {
+            const int hj = n + NP * k;
+            if (hj < kCkX) {
+                const float raw = q.qhalo[k] + bias;
+                sDl[cl * DLP + hj] = softplus ? softplus20(raw, dsp) : raw;
+            }
         }
     };
 
@@ -465,6 +474,8 @@ static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
 // One instantiation per input dtype, each in its own translation unit.
 template <typename T>
 int launch_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
+    // (four lanes per channel for N <= 4 work here too, but measure slower than eight: one-wave blocks
+    // with 16 staged pixels per thread; the backward does use them)
     return p.shape.dstate > 8 ? launch_fwd_np<T, 16>(p, stream) : launch_fwd_np<T, 8>(p, stream);
 }
 
