@@ -81,9 +81,9 @@ typedef struct snd_plan {
  * (batch, channel), fwd.cuh:359-392); here the library picks by shape unless told otherwise:
  *   PLANE   one block per (batch, group, 16-channel chunk) walks the whole plane;
  *   STRIPS  one block per 8-row strip of such a chunk, the strips of a plane pipelined one tile
- *           apart (for few, large planes: c3/c4-like shapes).  Needs the workspace.
+ *           apart (for few, large planes, e.g. 2 x 192 channels of 200x336 or 256 of 512x512).  Needs the workspace.
  *   BANDS   one block per band of consecutive strips, 2-4 bands per plane, handed over like strips but
- *           only at band ends.  For more plane chunks than the chip holds blocks at once (c1 backward:
+ *           only at band ends.  For more plane chunks than the chip holds blocks at once (backward at B=64, D=192, 56x56, N=16:
  *           768 chunks, 512 slots), where whole-plane blocks leave the last round half empty.  Needs
  *           the workspace. */
 typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2, SND_SCHED_BANDS = 3 } snd_schedule;

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     __shared__ float sSp[(NP / 4) * kTile], sS[kTile];
     // out of up to four consecutive tiles of a strip (two in the 8-state kernels, whose blocks have
     // less LDS each), flushed together: a 32-byte run per tile row is a partial line write (measured:
-    // 13 % of the kernel for 154 MB at c1), four tiles make whole lines
+    // 13 % of the kernel for the 154 MB of out at B=64, D=192, 56x56), four tiles make whole lines
     constexpr int QT = NP == 16 ? 4 : 2, QC = QT * kCkX;
     constexpr int OROW = NP == 16 ? QC + 8 : QC, OCH = kRows * OROW + (NP == 16 ? 16 : 8);   // padded against bank conflicts
     __shared__ float sOut[CB * OCH];
