@@ -109,6 +109,8 @@ def test_address_range_limits_are_status_codes():
         return fp
 
     assert lib.snd_fwd(C.byref(params(schedule=4)), None) == -2                  # unknown schedule
+    assert lib.snd_fwd(C.byref(params(schedule=capi.SCHED_STRIPS)), None) == -6  # pipelined schedules need the workspace
+    assert lib.snd_fwd(C.byref(params(schedule=capi.SCHED_BANDS)), None) == -6
     assert lib.snd_fwd(C.byref(params(directions=2)), None) == -2                # unknown directions
     assert lib.snd_fwd(C.byref(params(u_h_stride=2)), None) == -4                # rows overlap
     assert lib.snd_fwd(C.byref(params(u_h_stride=1 << 21)), None) == -4          # row pitch >= 2^23 bytes
