@@ -45,7 +45,9 @@ typedef enum snd_status {
     SND_ERR_STRIDE = -4,           /* a stride is negative / zero where a dense walk is required */
     SND_ERR_LAUNCH = -5,           /* hipLaunchKernel reported an error */
     SND_ERR_WORKSPACE = -6,        /* checkpoint / workspace buffer missing or too small */
-    SND_ERR_ALIGN = -7             /* checkpoint / workspace pointer not 16-byte aligned */
+    SND_ERR_ALIGN = -7,            /* checkpoint / workspace pointer not 16-byte aligned */
+    SND_ERR_RESERVED_ = -8,
+    SND_ERR_PIPELINE = -9          /* snd_workspace_error: a hand-over wait between blocks timed out (outputs are NaN) */
 } snd_status;
 
 /* Problem sizes; replaces the size fields of SSMParamsBase
@@ -171,6 +173,30 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream);
 /* Backward: replaces selective_scan_bwd_cuda<input_t, weight_t, output_t>(params, stream)
  * (selective_scan_oflex.cpp:34-35,424-430; kernel bwd.cuh:91-902).  Asynchronous on `stream`. */
 int snd_bwd(const snd_bwd_params *params, snd_stream_t stream);
+
+/* Per-device set-up: raises the dynamic-LDS limit of the backward kernels and on `device`
+ * (replaces the cudaFuncSetAttribute calls the reference makes inside every launch,
+ * bwd.cuh:913-915, fwd.cuh:368-370).  Optional: the first snd_bwd on a device does the same,
+ * but these runtime calls are not stream-ordered, so a host that captures launches into a HIP graph, or
+ * launches from several threads at once, calls snd_init(device) once beforehand.  Thread-safe. */
+int snd_init(int device);
+
+/* The pipelined schedules (STRIPS, BANDS; what the plan's auto_schedule / auto_bwd_jobs say AUTO picks)
+ * hand rows from block to block through the workspace.  Its first 12 int32 words are the launch's sync
+ * header, cleared by the launch itself: word [1] is an error flag that a block sets when a wait for another
+ * block's row exceeds its poll limit (2^21 polls: a stalled producer, e.g. on a preempted GPU).  Such a
+ * block replaces the missing row by NaN, so out / du / ddelta / dA / dB / dC downstream of it are NaN,
+ * never plausible numbers, and the launch still drains.  snd_fwd / snd_bwd have returned SND_OK long
+ * before; this call is how a host learns the reason: it copies word [1] back and WAITS for `stream`
+ * (the only synchronising call of the library).  Returns SND_OK, SND_ERR_PIPELINE, or another error.
+ * Meaningful only after a pipelined launch on that workspace (a whole-plane launch leaves the header
+ * alone).  No counterpart in the reference, whose blocks never wait for each other. */
+int snd_workspace_error(const void *workspace, snd_stream_t stream);
+
+/* Test hook: poll limit of the hand-over waits for later launches (<= 0 restores the default 2^21).
+ * With a limit of a few polls the time-out path above can be exercised from the host while every
+ * kernel still runs to completion. */
+void snd_debug_set_spin_limit(int polls);
 
 #ifdef __cplusplus
 }

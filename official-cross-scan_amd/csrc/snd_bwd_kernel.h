@@ -106,8 +106,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
     __shared__ int sSeen;                           // (pipelined) progress count of the strip below, as last polled
+    __shared__ int sDead;                           // (pipelined) a hand-over wait of this block has timed out
     if (PIPE) {
-        if (threadIdx.x == 0) sSeen = 0;            // ordered before its readers by the barrier in draw_job
+        if (threadIdx.x == 0) { sSeen = 0; sDead = 0; }   // ordered before their readers by the barrier in draw_job
         // A job is a band of consecutive strips (one strip each in the fully pipelined case), drawn
         // bottom band first; band k from the bottom covers strips ceil(k*nCY/nBands) ..
         // ceil((k+1)*nCY/nBands)-1, counted from the bottom.
@@ -345,8 +346,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
             if (handed && wave == 0) {
-                strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead SND_TRACE_PASS);
-                if (tid == 0) sSeen = seen;         // read at the top of later tiles
+                strip_wait(progress + I + 1, geo.nCX - J, seen, sync, dead, geo.spinLimit SND_TRACE_PASS);
+                if (tid == 0) { sSeen = seen; if (dead) sDead = 1; }   // read at the top of later tiles
             }
             __syncthreads();
 
@@ -359,6 +360,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
                     for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
                 }
+            }
+            if (handed && *(volatile int *)&sDead) {   // the wait timed out: poison everything downstream
+#pragma unroll
+                for (int j = 0; j < kCkX; ++j) Gd[j] = __builtin_nanf("");
             }
             const float gd_old0 = Gd[0];            // G[r0+8][j0]: the corner of the tile on the left
 
@@ -611,29 +616,40 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     }
 }
 
+// Dynamic LDS of one backward block (more than the 64 KB a kernel gets without asking).
+template <int NP> constexpr size_t bwd_lds_bytes() {
+    return sizeof(float) * ((2 + 2 * (NP / 4)) * NP * (kTile + 4) + 16 * 100 + 6 * 16 * kTile + NP / 4);
+}
+// Raise the dynamic LDS limit of every backward instantiation of one input dtype on the current device.
+// hipFuncSetAttribute is not stream-ordered and must not run under a stream capture, which is why it is
+// done once per device at set-up and not inside the launch path.
+template <typename T, int NP, int TE> static bool configure_bwd_one() {
+    const int lds = (int)bwd_lds_bytes<NP>();
+    return hipFuncSetAttribute((const void *)bwd_kernel<T, NP, true, TE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
+           hipFuncSetAttribute((const void *)bwd_kernel<T, NP, false, TE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
+}
+template <typename T> int configure_bwd_t() {
+    const bool ok = configure_bwd_one<T, 16, 8>() && configure_bwd_one<T, 16, 7>() && configure_bwd_one<T, 8, 8>() &&
+                    configure_bwd_one<T, 8, 7>() && configure_bwd_one<T, 4, 8>() && configure_bwd_one<T, 4, 7>();
+    return ok ? SND_OK : SND_ERR_LAUNCH;
+}
+
 template <typename T, int NP, int TE>
 static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
-    constexpr int WPB = NP / 4, NSTR = kTile + 4, NPART = WPB;
-    constexpr size_t lds = sizeof(float) * ((2 + 2 * NPART) * NP * NSTR + 16 * 100 + 6 * 16 * kTile + WPB);
+    constexpr size_t lds = bwd_lds_bytes<NP>();
     const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate);   // 0: one block per plane chunk
     const bool pipe = bands > 0;
-    // raise the dynamic LDS limit once per kernel and device (the call costs tens of microseconds)
-    static bool configured[2][64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SND_ERR_LAUNCH;
-    if (!configured[pipe][dev]) {
-        const void *fn = pipe ? (const void *)bwd_kernel<T, NP, true, TE> : (const void *)bwd_kernel<T, NP, false, TE>;
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return SND_ERR_LAUNCH;
-        configured[pipe][dev] = true;
-    }
+    // the dynamic LDS limit of these kernels is raised by snd_init() / on the first launch on a device
+    if (int st = ensure_device_ready(); st != SND_OK) return st;
     if (pipe) {
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
         Geo gb = geo;
+        gb.spinLimit = spin_limit();
         gb.nBands = bands;
         gb.nQueues = job_queues(sh.batch * sh.n_groups);
         hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);

@@ -1,6 +1,9 @@
 // C ABI of the gfx950 selective_nd_scan library: validation, planning and dispatch.
 // Mirrors the checks of the reference host binding
 // (kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:188-245,298-361) as status codes.
+#include <atomic>
+#include <mutex>
+
 #include "snd_device.h"
 
 namespace snd {
@@ -10,7 +13,11 @@ int launch_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
 int launch_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
+int configure_bwd_f32();
+int configure_bwd_bf16();
+int configure_bwd_f16();
 }  // namespace snd
+
 
 namespace snd {
 __global__ void zero_words_kernel(int *p, int64_t n) {
@@ -20,6 +27,25 @@ __global__ void zero_words_kernel(int *p, int64_t n) {
 int zero_words(int *p, int64_t n, hipStream_t stream) {
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_setup_mutex;
+static std::atomic<bool> g_ready[kMaxDevices];
+static std::atomic<int> g_spin_limit{kSpinLimit};
+
+int spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
+
+// Set-up of the current device: done once, by whichever of snd_init() and the first launch comes first.
+int ensure_device_ready() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SND_ERR_LAUNCH;
+    if (g_ready[dev].load(std::memory_order_acquire)) return SND_OK;
+    std::lock_guard<std::mutex> lock(g_setup_mutex);
+    if (g_ready[dev].load(std::memory_order_relaxed)) return SND_OK;
+    if (configure_bwd_f32() != SND_OK || configure_bwd_bf16() != SND_OK || configure_bwd_f16() != SND_OK) return SND_ERR_LAUNCH;
+    g_ready[dev].store(true, std::memory_order_release);
+    return SND_OK;
 }
 }  // namespace snd
 
@@ -79,7 +105,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 104; }
+int snd_version(void) { return 200; }
 
 const char *snd_status_string(int status) {
     switch (status) {
@@ -91,6 +117,7 @@ const char *snd_status_string(int status) {
         case SND_ERR_LAUNCH: return "kernel launch failed";
         case SND_ERR_WORKSPACE: return "saved state (x, x_v, x_sd) or workspace missing or too small";
         case SND_ERR_ALIGN: return "saved state / workspace pointers must be 16-byte aligned";
+        case SND_ERR_PIPELINE: return "a hand-over wait between blocks timed out in an earlier launch on this workspace: its outputs are NaN";
         default: return "unknown status";
     }
 }
@@ -148,7 +175,7 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     }
 }
 
-int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
+static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
     if (!params) return SND_ERR_NULL;
     int st = check_fwd(params->f, true);
     if (st != SND_OK) return st;
@@ -174,5 +201,27 @@ int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) {
         default: return snd::launch_bwd_f16(*params, (hipStream_t)stream);
     }
 }
+
+int snd_bwd(const snd_bwd_params *params, snd_stream_t stream) { return bwd_checked(params, stream); }
+
+int snd_init(int device) {
+    int cur = 0;
+    if (hipGetDevice(&cur) != hipSuccess) return SND_ERR_LAUNCH;
+    if (device != cur && hipSetDevice(device) != hipSuccess) return SND_ERR_LAUNCH;
+    const int st = snd::ensure_device_ready();
+    if (device != cur && hipSetDevice(cur) != hipSuccess) return SND_ERR_LAUNCH;
+    return st;
+}
+
+int snd_workspace_error(const void *workspace, snd_stream_t stream) {
+    if (!workspace) return SND_ERR_NULL;
+    int word = 0;
+    if (hipMemcpyAsync(&word, (const int *)workspace + snd::kErrorWord, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+        return SND_ERR_LAUNCH;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return SND_ERR_LAUNCH;
+    return word != 0 ? SND_ERR_PIPELINE : SND_OK;
+}
+
+void snd_debug_set_spin_limit(int polls) { snd::g_spin_limit.store(polls > 0 ? polls : snd::kSpinLimit, std::memory_order_relaxed); }
 
 }  // extern "C"

@@ -22,6 +22,7 @@ struct Geo {
     int te;                        // tile extent
     int nBands;                    // pipelined schedules: jobs per plane chunk (set by the launcher)
     int nQueues;                   // and the number of job queues: 8 (one per XCD) or 1
+    int spinLimit;                 // polls a hand-over wait makes before it gives up (set by the launcher)
 };
 __host__ __device__ inline Geo make_geo(int H, int W) {
     const long long c8 = (long long)((H + 7) / 8) * ((W + 7) / 8) * 64, c7 = (long long)((H + 6) / 7) * ((W + 6) / 7) * 49;
@@ -33,6 +34,7 @@ __host__ __device__ inline Geo make_geo(int H, int W) {
     g.Wp = g.nCX * kCkX;
     g.nBands = 0;
     g.nQueues = 1;
+    g.spinLimit = 1 << 21;
     return g;
 }
 
@@ -206,7 +208,9 @@ __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8
 #define SND_POLL_SLEEP 16                           // s_sleep units (64 cycles) between polls
 #endif
 constexpr int kErrorWord = 1, kTicketWord = 4, kSyncHeader = 12;
-constexpr int kSpinLimit = 1 << 21;                 // polls (a memory round trip each) before giving up
+constexpr int kSpinLimit = 1 << 21;                 // default polls (a memory round trip each) before giving up
+// The limit launches use: kSpinLimit unless snd_debug_set_spin_limit() lowered it (tests of the time-out path).
+int spin_limit();
 __host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips) {
 #ifdef SND_PIPE_TRACE   // timing study only: 4 extra words per job (start, end, time spent waiting, -)
     return (kSyncHeader + 5 * nPlaneChunks * nStrips + 3) / 4 * 4;
@@ -217,6 +221,23 @@ __host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips)
 
 // Data handed from one block to another inside a launch is written and read with agent-scope
 // relaxed atomics (they go through to the coherence point and are never served from a stale line).
+//
+// Why no release / acquire fence is needed around the hand-over on gfx950:
+//   * producer: the row is written with agent-scope atomic stores, which are performed at the agent's
+//     coherence point and not held back in a wave-private or CU-private cache.  Every wave then executes
+//     `s_waitcnt vmcnt(0)` (strip_stores_done): it does not pass this point before the coherence point has
+//     acknowledged all of its stores.  The block barrier that follows makes that true for all waves of the
+//     block, and only then does thread 0 move the count with an agent-scope atomic add.  So whoever can
+//     observe the new count can observe the row: the count is issued after every store of the row has
+//     completed, which is what a release fence would have waited for as well (it would in addition write
+//     back the whole L2 working set of the block, which nothing here needs).
+//   * consumer: the count is polled with agent-scope atomic loads, and the row is read with agent-scope
+//     atomic loads (ld2_coherent) that are issued only after a poll has returned the expected value (the
+//     loop exit is a branch on the loaded value, so the wave has waited for it).  Coherent loads are not
+//     served from lines cached before the hand-over, which is what an acquire fence (a cache invalidate)
+//     would have guaranteed for ordinary loads; no ordinary load ever touches the hand-over rows or counts.
+//   * the compiler barrier at the end of strip_wait keeps the compiler from moving the row loads above the
+//     poll; the hardware issues a wave's memory instructions in program order.
 __device__ __forceinline__ void st2_coherent(float *dst, float a, float b) {
     const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
     __hip_atomic_store((uint64_t *)dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -245,9 +266,11 @@ __device__ __forceinline__ void strip_signal(int *count) {
 #endif
 // Wait until *count >= need.  `seen` caches the last value read (counts only grow), so a consumer
 // that runs well behind its producer polls once per strip, not once per tile.  Bounded: after
-// kSpinLimit polls the error word is set and the wave goes on (with wrong data) so that the grid
-// always drains; `dead` then disables further waits.
-__device__ __forceinline__ void strip_wait(const int *count, int need, int &seen, int *sync, bool &dead SND_TRACE_ARG) {
+// `limit` polls the error word (sync word kErrorWord) is set and the wave goes on so that the grid
+// always drains; `dead` then disables further waits.  A block that gave up replaces every row it
+// should have been handed by NaN (see the callers), so the outputs downstream of a timed-out wait are
+// NaN and never plausible-looking numbers; the error word says why (snd_workspace_error reads it).
+__device__ __forceinline__ void strip_wait(const int *count, int need, int &seen, int *sync, bool &dead, int limit SND_TRACE_ARG) {
     if (dead || seen >= need) return;
 #ifdef SND_PIPE_TRACE
     const long long t0_ = wall_clock64();
@@ -255,7 +278,7 @@ __device__ __forceinline__ void strip_wait(const int *count, int need, int &seen
     int polls = 0;
     while ((seen = __hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) < need) {
         __builtin_amdgcn_s_sleep(SND_POLL_SLEEP);
-        if (++polls > kSpinLimit) {
+        if (++polls > limit) {
             dead = true;
             __hip_atomic_store(sync + kErrorWord, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
@@ -301,6 +324,9 @@ __device__ __forceinline__ bool draw_job(int *sync, int nPairs, int nChunks, int
 __host__ inline int job_queues(int nPairs) { return nPairs >= 16 ? 8 : 1; }
 // Enqueue a fill kernel that zeroes n int32 words (defined with the C entry points).
 int zero_words(int *p, int64_t n, hipStream_t stream);
+// Per-device set-up (kernel attributes, the address of the static scratch array), done by snd_init() or
+// by the first call that needs it on a device.  Returns an snd_status.
+int ensure_device_ready();
 // How a launch is scheduled (snd_fwd_params::schedule): one block per plane chunk walking all its
 // strips, or one block per strip with the strips of a plane pipelined.
 enum { kSchedAuto = 0, kSchedPlane = 1, kSchedStrips = 2, kSchedBands = 3 };

@@ -67,7 +67,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
 #ifdef SND_PIPE_TRACE
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
+    __shared__ int sDead;                           // (pipelined) a hand-over wait of this block has timed out
     if (PIPE) {
+        if (threadIdx.x == 0) sDead = 0;            // ordered before its readers by the barrier in draw_job
         // A job is a band of consecutive strips (one strip each in the fully pipelined case), drawn
         // top band first; band k covers strips ceil(k*nCY/nBands) .. ceil((k+1)*nCY/nBands)-1.
         int band;
@@ -271,7 +273,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             commit(mine);
             // first strip of a pipelined band: the row above comes from another block
             const bool handed = PIPE && I == I_begin && I > 0;
-            if (handed && wave == 0) strip_wait(progress + I - 1, J + 1, seen, sync, dead SND_TRACE_PASS);
+            if (handed && wave == 0) {
+                strip_wait(progress + I - 1, J + 1, seen, sync, dead, geo.spinLimit SND_TRACE_PASS);
+                if (dead && tid == 0) sDead = 1;
+            }
             __syncthreads();
             if (wave == 0) {                        // read by the output phase, behind the next barrier
                 float t = 0.f;
@@ -285,6 +290,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             float corner = 0.f;                     // h[r0-1][j0-1]
             if (handed) {
                 fetch_row_above(J, hup);
+                if (*(volatile int *)&sDead) {      // the wait timed out: poison everything downstream
+#pragma unroll
+                    for (int j = 0; j < kCkX; ++j) hup[j] = __builtin_nanf("");
+                }
             } else {
                 corner = (I > 0) ? qcorner : 0.f;
 #pragma unroll
@@ -449,6 +458,7 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;
         const int grid = (int)(nPC * bands);
         Geo gs = geo;
+        gs.spinLimit = spin_limit();
         gs.nBands = bands;
         gs.nQueues = job_queues(sh.batch * sh.n_groups);
         if (p.x != nullptr)

@@ -13,6 +13,8 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
+#include <atomic>
+#include <cstdlib>
 #include <vector>
 
 #include "snd_scan.h"
@@ -101,8 +103,23 @@ Checked check_inputs(const at::Tensor &u, const at::Tensor &delta, const at::Ten
     return c;
 }
 
-// snd_schedule used by fwd and bwd (0 = chosen by shape); set_schedule() is for tests and tuning.
-int g_schedule = SND_SCHED_AUTO;
+// Default snd_schedule of fwd and bwd (0 = chosen by shape) when a call does not name one; set_schedule()
+// is for tests and tuning.  Calls that pass `schedule` themselves never read it.
+std::atomic<int> g_schedule{SND_SCHED_AUTO};
+// Opt-in check of the pipelined schedules' error word after every launch (costs a stream sync):
+// SND_CHECK_PIPELINE=1 in the environment, or set_debug(True).
+std::atomic<bool> g_check_pipeline{[] { const char *e = std::getenv("SND_CHECK_PIPELINE"); return e && e[0] && e[0] != '0'; }()};
+
+int resolve_schedule(int64_t schedule) {
+    if (schedule < 0) return g_schedule.load();
+    TORCH_CHECK(schedule >= SND_SCHED_AUTO && schedule <= SND_SCHED_BANDS, "schedule must be 0 (auto), 1 (plane), 2 (strips) or 3 (bands)");
+    return (int)schedule;
+}
+void check_pipeline(const at::Tensor &ws, hipStream_t stream, const char *what) {
+    if (!ws.defined() || !g_check_pipeline.load()) return;
+    const int st = snd_workspace_error(ws.data_ptr(), (snd_stream_t)stream);
+    TORCH_CHECK(st == SND_OK, "selective_nd_scan ", what, ": ", snd_status_string(st), " (status ", st, ")");
+}
 
 void fill_fwd(snd_fwd_params &p, const Checked &c, const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
               const at::Tensor &B, const at::Tensor &C, const c10::optional<at::Tensor> &D_,
@@ -129,7 +146,7 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
                                            const c10::optional<at::Tensor> &D_,
                                            const c10::optional<at::Tensor> &delta_bias_, bool delta_softplus,
                                            bool out_float, const c10::optional<at::Tensor> &A_decay_,
-                                           int64_t directions) {
+                                           int64_t directions, int64_t schedule) {
     TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
     at::hip::HIPGuardMasqueradingAsCUDA device_guard{u.device()};
@@ -148,10 +165,11 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     p.x = x.data_ptr<float>(); p.x_v = x_v.data_ptr<float>(); p.x_sd = x_sd.data_ptr<float>();
     // scratch for the strip-pipelined schedule (only when it will be used); released to the caching
     // allocator in stream order
-    p.schedule = g_schedule;
+    const int sched = resolve_schedule(schedule);
+    p.schedule = sched;
     at::Tensor ws;
-    if (g_schedule == SND_SCHED_STRIPS || g_schedule == SND_SCHED_BANDS ||
-        (g_schedule == SND_SCHED_AUTO && c.plan.auto_schedule != SND_SCHED_PLANE)) {
+    if (sched == SND_SCHED_STRIPS || sched == SND_SCHED_BANDS ||
+        (sched == SND_SCHED_AUTO && c.plan.auto_schedule != SND_SCHED_PLANE)) {
         ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
         p.workspace = ws.data_ptr();
         p.workspace_bytes = c.plan.fwd_workspace_bytes;
@@ -159,6 +177,7 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     p.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");
+    check_pipeline(ws, stream, "fwd");
     return {out, x, x_v, x_sd};
 }
 
@@ -168,7 +187,7 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
                                            const c10::optional<at::Tensor> &delta_bias_, const at::Tensor &dout,
                                            const c10::optional<at::Tensor> &x_, const c10::optional<at::Tensor> &x_v_,
                                            bool delta_softplus, const c10::optional<at::Tensor> &A_decay_,
-                                           const c10::optional<at::Tensor> &x_sd_, int64_t directions) {
+                                           const c10::optional<at::Tensor> &x_sd_, int64_t directions, int64_t schedule) {
     TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
     const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate;
@@ -195,20 +214,21 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     const auto f32 = u.options().dtype(at::ScalarType::Float);
     at::Tensor du = torch::empty({batch_size, dim, nrows, ncols}, u.options());
     at::Tensor ddelta = torch::empty({batch_size, dim, nrows, ncols}, u.options());
-    // the accumulated gradients (zero-filled as host.cpp:395-403 does) are carved out of one buffer,
-    // so that one fill kernel clears them all
+    // the accumulated gradients are zero-filled as host.cpp:395-403 does.  dB and dC share one buffer (one
+    // fill kernel for the two large tensors); the small ones (dA, dD, ddelta_bias, dA_decay) share another,
+    // so that a parameter gradient kept by the optimizer never pins the large buffer.
     const int64_t nA = (int64_t)dim * dstate, nBC = B.numel();
     auto round64 = [](int64_t v) { return (v + 63) / 64 * 64; };
-    const int64_t oB = round64(nA), oC = oB + round64(nBC), oD = oC + round64(nBC), oBias = oD + round64(dim),
-                  oDec = oBias + round64(dim);
-    at::Tensor acc = torch::zeros({oDec + 64}, f32);
-    at::Tensor dA = acc.narrow(0, 0, nA).view({dim, dstate});
-    at::Tensor dB = acc.narrow(0, oB, nBC).view(B.sizes());
-    at::Tensor dC = acc.narrow(0, oC, nBC).view(C.sizes());
+    at::Tensor accBC = torch::zeros({2 * round64(nBC)}, f32);
+    at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
+    at::Tensor dC = accBC.narrow(0, round64(nBC), nBC).view(C.sizes());
+    const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim);
+    at::Tensor accP = torch::zeros({oDec + 64}, f32);
+    at::Tensor dA = accP.narrow(0, 0, nA).view({dim, dstate});
     at::Tensor dD, ddelta_bias, dA_decay;
-    if (D_.has_value()) dD = acc.narrow(0, oD, dim);
-    if (delta_bias_.has_value()) ddelta_bias = acc.narrow(0, oBias, dim);
-    if (A_decay_.has_value()) dA_decay = acc.narrow(0, oDec, 1);
+    if (D_.has_value()) dD = accP.narrow(0, oD, dim);
+    if (delta_bias_.has_value()) ddelta_bias = accP.narrow(0, oBias, dim);
+    if (A_decay_.has_value()) dA_decay = accP.narrow(0, oDec, 1);
     at::Tensor ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
 
     snd_bwd_params p;
@@ -225,10 +245,11 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     p.dA_decay = dA_decay.defined() ? dA_decay.data_ptr<float>() : nullptr;
     p.workspace = ws.data_ptr();
     p.workspace_bytes = c.plan.bwd_workspace_bytes;
-    p.f.schedule = g_schedule;
+    p.f.schedule = resolve_schedule(schedule);
     p.f.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
+    if (c.plan.auto_bwd_jobs != 0 || p.f.schedule == SND_SCHED_STRIPS || p.f.schedule == SND_SCHED_BANDS) check_pipeline(ws, stream, "bwd");
 
     // host.cpp:432-438: cast dB/dC to the input dtype, fold channel groups that share a delta
     std::vector<at::Tensor> result = {du, ddelta, dA, dB.to(B.dtype()), dC.to(C.dtype()), dD, ddelta_bias, dA_decay};
@@ -245,17 +266,22 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
-    // the reference's positional lists (selective_scan_oflex.cpp:179-187,286-297) plus one trailing
-    // optional argument: the per-group scan origin the reference leaves as a TODO (fwd.cuh:140)
+    // the reference's positional lists (selective_scan_oflex.cpp:179-187,286-297) plus two trailing
+    // optional arguments: the per-group scan origin the reference leaves as a TODO (fwd.cuh:140) and the
+    // block mapping of this call (-1: the module default)
     namespace py = pybind11;
     m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("delta_softplus"), py::arg("out_float"),
-          py::arg("A_decay"), py::arg("directions") = 0);
+          py::arg("A_decay"), py::arg("directions") = 0, py::arg("schedule") = -1);
     m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("dout"), py::arg("x"), py::arg("x_v"),
-          py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0);
+          py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0, py::arg("schedule") = -1);
     m.def("set_schedule", [](int mode) {
         TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_BANDS, "schedule must be 0 (auto), 1 (plane), 2 (strips) or 3 (bands, backward)");
-        g_schedule = mode;
-    }, "Force how fwd/bwd map work to blocks: 0 auto, 1 one block per plane chunk, 2 pipelined row strips");
+        g_schedule.store(mode);
+    }, "Default block mapping of calls that pass no schedule: 0 auto, 1 one block per plane chunk, 2 pipelined row strips, 3 bands");
+    m.def("set_debug", [](bool on) { g_check_pipeline.store(on); },
+          "Check the pipelined schedules' error word after every launch (a stream sync per call) and raise if a hand-over wait timed out");
+    m.def("init", [](int device) { check_status(snd_init(device), "init"); },
+          "Per-device set-up (kernel attributes); call once before capturing launches into a HIP graph");
 }

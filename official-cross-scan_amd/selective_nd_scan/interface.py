@@ -25,22 +25,36 @@ from ._ext import ext
 
 
 def fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
-        directions=0):
-    """Reference binding `fwd` -> [out, x, x_v, x_sd] (selective_scan_oflex.cpp:179-187,282)."""
-    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)
+        directions=0, schedule=-1):
+    """Reference binding `fwd` -> [out, x, x_v, x_sd] (selective_scan_oflex.cpp:179-187,282).
+    schedule: block mapping of this call (-1 = the module default, see set_schedule)."""
+    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions, schedule)
 
 
-def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions=0):
+def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions=0, schedule=-1):
     """Reference binding `bwd` -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
     (selective_scan_oflex.cpp:286-297,432-438)."""
-    return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions)
+    return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions,
+                     schedule)
 
 
 def set_schedule(mode):
-    """How fwd/bwd map work to blocks: 0 = chosen by shape, 1 = one block per (batch, group,
-    16-channel chunk) plane, 2 = one block per 8-row strip, strips pipelined.  Results do not
-    depend on it (only the order of the atomic sums in dA, dB, dC, dD, ddelta_bias does)."""
+    """Default block mapping of calls that name none: 0 = chosen by shape, 1 = one block per (batch,
+    group, 16-channel chunk) plane, 2 = one block per 8-row strip, strips pipelined, 3 = bands of strips.
+    Results do not depend on it (only the order of the atomic sums in dA, dB, dC, dD, ddelta_bias does)."""
     ext().set_schedule(int(mode))
+
+
+def set_debug(on=True):
+    """After every pipelined launch, read the workspace's error word (one stream sync per call) and raise
+    if a block-to-block wait timed out.  Also switched on by SND_CHECK_PIPELINE=1 in the environment."""
+    ext().set_debug(bool(on))
+
+
+def init(device=0):
+    """Per-device set-up (kernel attributes).  Optional; call it once before capturing launches into a
+    HIP graph or launching from several threads."""
+    ext().init(int(device))
 
 
 def _last_dim_contiguous(t):

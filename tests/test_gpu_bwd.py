@@ -133,4 +133,4 @@ def test_bwd_linearity_in_dout_at_scale(gpu_device):
     for a, b_, c_, name in zip(g1, g2, g12, NAMES):
         if a is None:
             continue
-        assert relerr(c_.cpu().numpy(), (2.0 * a - 3.0 * b_).cpu().numpy()) <= 2e-4, name
+        assert relerr(c_.cpu().numpy(), (2.0 * a - 3.0 * b_).cpu().numpy()) <= 1e-4, name

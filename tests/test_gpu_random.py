@@ -93,7 +93,14 @@ def test_random_case(gpu_device, seed):
                 want = want.reshape(c["Bt"], c["Dd"], rep, c["H"], c["W"]).sum(2)
         if nm == "ddelta_bias" and c["dirs"] and rep > 1:
             want = want.reshape(c["Dd"], rep).sum(1)
-        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 3e-4
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
+        if nm == "dA_decay":
+            # one scalar: the sum of a signed term over every cell of every plane, taken in fp32 by
+            # per-lane partial sums and atomics.  The terms cancel (|sum| is a few percent of sum |term|),
+            # so the fp32 rounding of the terms shows up amplified against the sum itself: seed 14
+            # (2 x 8 planes of 22 x 10, N = 2) measures 1.0e-4 to 1.2e-4 depending on the order the atomics
+            # land in.  Every other gradient keeps 1e-4.
+            tol = 5e-4
         if nm == "dA_decay" and c["H"] == 1:
             # a single row makes h = s, so out does not depend on a: the reference is zero and relerr
             # measures the fp32 rounding noise of a sum over every cell of every plane on its absolute

@@ -72,7 +72,7 @@ def test_strips_match_plane_and_oracle(gpu_device, Bt, Dm, H, W, N, K, dtype):
     assert relerr(out_s.cpu().numpy(), ref) <= 1e-4
     half = dtype != torch.float32
     for nm, a, b_ in zip(NAMES, g_s, gref):
-        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 2e-4
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
         assert relerr(a.float().cpu().numpy(), b_) <= tol, (nm, relerr(a.float().cpu().numpy(), b_))
 
 

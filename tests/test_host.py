@@ -11,11 +11,12 @@ import capi
 
 def test_library_exports_every_declared_symbol():
     names = capi.declared_symbols()
-    assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd"}
+    assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd", "snd_init",
+                          "snd_workspace_error", "snd_debug_set_spin_limit"}
     lib = capi.lib()
     for n in names:
         assert getattr(lib, n) is not None, n
-    assert lib.snd_version() >= 100
+    assert lib.snd_version() >= 200
 
 
 def test_struct_layouts_match_header_sizes():
@@ -108,7 +109,7 @@ def test_address_range_limits_are_status_codes():
             setattr(fp, k, v)
         return fp
 
-    assert lib.snd_fwd(C.byref(params(schedule=4)), None) == -2                  # unknown schedule
+    assert lib.snd_fwd(C.byref(params(schedule=9)), None) == -2                  # unknown schedule
     assert lib.snd_fwd(C.byref(params(schedule=capi.SCHED_STRIPS)), None) == -6  # pipelined schedules need the workspace
     assert lib.snd_fwd(C.byref(params(schedule=capi.SCHED_BANDS)), None) == -6
     assert lib.snd_fwd(C.byref(params(directions=2)), None) == -2                # unknown directions
@@ -201,3 +202,39 @@ def test_tile_extent_choice():
     assert tiles(14, 14) == (2, 2) and tiles(28, 28) == (4, 4) and tiles(7, 7) == (1, 1) and tiles(21, 35) == (3, 5)
     assert tiles(56, 56) == (7, 7) and tiles(64, 64) == (8, 8) and tiles(512, 512) == (64, 64) and tiles(200, 336) == (25, 42)
     assert tiles(1, 37) == (1, 5)                 # 294 vs 320 padded cells: not worth the smaller tile
+
+
+def test_pipeline_error_contract_on_the_host():
+    """The documented error query and status text exist and validate their arguments; the spin-limit
+    hook accepts any value (<= 0 restores the default)."""
+    lib = capi.lib()
+    assert lib.snd_workspace_error(None, None) == -1
+    assert b"timed out" in lib.snd_status_string(-9) and b"NaN" in lib.snd_status_string(-9)
+    lib.snd_debug_set_spin_limit(3)
+    lib.snd_debug_set_spin_limit(0)
+    header = open(capi.HEADER).read()
+    assert "word [1] is an error flag" in header and "snd_workspace_error" in header
+
+
+def test_init_without_a_gpu_is_a_status_not_a_crash():
+    torch = pytest.importorskip("torch")
+    if torch.cuda.is_available():
+        pytest.skip("needs a box without a GPU")
+    assert capi.lib().snd_init(0) == -5
+
+
+def test_reference_module_name_is_importable():
+    """Callers of the reference `import selective_nd_scan_cuda_oflex` (setup.py:80): the same name here is
+    the gfx950 extension, with the reference's two functions."""
+    pytest.importorskip("torch")
+    import selective_nd_scan_cuda_oflex as m
+    import selective_nd_scan_hip_oflex as h
+    assert m.fwd is h.fwd and m.bwd is h.bwd
+    assert "schedule" in m.fwd.__doc__ and "directions" in m.bwd.__doc__
+
+
+def test_packaging_names_match_the_reference():
+    """setup.py: distribution `selective_nd_scan` (reference setup.py:118), extension module
+    `selective_nd_scan_cuda_oflex` (:80)."""
+    text = open(os.path.join(capi.ROOT, "setup.py")).read()
+    assert 'name="selective_nd_scan"' in text and '"selective_nd_scan_cuda_oflex"' in text
