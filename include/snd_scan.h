@@ -46,7 +46,7 @@ typedef enum snd_status {
     SND_ERR_LAUNCH = -5,           /* hipLaunchKernel reported an error */
     SND_ERR_WORKSPACE = -6,        /* checkpoint / workspace buffer missing or too small */
     SND_ERR_ALIGN = -7,            /* checkpoint / workspace pointer not 16-byte aligned */
-    SND_ERR_RESERVED_ = -8,
+    SND_ERR_TOO_LARGE = -8,        /* snd_bwd_static: the shape needs more scratch than the static workspace holds */
     SND_ERR_PIPELINE = -9          /* snd_workspace_error: a hand-over wait between blocks timed out (outputs are NaN) */
 } snd_status;
 
@@ -174,9 +174,9 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream);
  * (selective_scan_oflex.cpp:34-35,424-430; kernel bwd.cuh:91-902).  Asynchronous on `stream`. */
 int snd_bwd(const snd_bwd_params *params, snd_stream_t stream);
 
-/* Per-device set-up: raises the dynamic-LDS limit of the backward kernels and on `device`
- * (replaces the cudaFuncSetAttribute calls the reference makes inside every launch,
- * bwd.cuh:913-915, fwd.cuh:368-370).  Optional: the first snd_bwd on a device does the same,
+/* Per-device set-up: raises the dynamic-LDS limit of the backward kernels and looks up the static
+ * workspace on `device` (replaces the cudaFuncSetAttribute calls the reference makes inside every launch,
+ * bwd.cuh:913-915, fwd.cuh:368-370).  Optional: the first snd_bwd / snd_bwd_static on a device does the same,
  * but these runtime calls are not stream-ordered, so a host that captures launches into a HIP graph, or
  * launches from several threads at once, calls snd_init(device) once beforehand.  Thread-safe. */
 int snd_init(int device);
@@ -197,6 +197,19 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream);
  * With a limit of a few polls the time-out path above can be exercised from the host while every
  * kernel still runs to completion. */
 void snd_debug_set_spin_limit(int polls);
+
+/* snd_bwd for callers that cannot allocate device memory (code under HIP-graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, which allocates its scratch with
+ * torch::empty / torch::zeros inside every call (selective_scan_oflex.cpp:393-403).  Identical to
+ * snd_bwd except that params->workspace / workspace_bytes are ignored: the scratch is a static device
+ * array of snd_static_workspace_bytes() bytes (64 MiB per GPU, held until the process ends) that the
+ * library owns.  Shapes whose plan.bwd_workspace_bytes exceeds it are refused with SND_ERR_TOO_LARGE.
+ * The caller still passes every input, output and saved-state buffer.  Allocates nothing, frees nothing.
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
+ * calls on one stream are ordered.  The sync header is cleared by a fill kernel at the start of each
+ * launch; nothing else in the array needs to start at zero. */
+int snd_bwd_static(const snd_bwd_params *params, snd_stream_t stream);
+int64_t snd_static_workspace_bytes(void);
 
 #ifdef __cplusplus
 }

@@ -18,6 +18,11 @@ int configure_bwd_bf16();
 int configure_bwd_f16();
 }  // namespace snd
 
+// Scratch of snd_bwd_static(): one array per GPU the library runs on, held until the process ends.
+// Host code never uses the array's name as an address: ensure_device_ready() asks the runtime for the
+// array's device address on each GPU and every later use goes through that pointer.
+#define SND_STATIC_WORKSPACE_BYTES (64ll << 20)
+static __device__ __align__(256) unsigned char scratch[SND_STATIC_WORKSPACE_BYTES];
 
 namespace snd {
 __global__ void zero_words_kernel(int *p, int64_t n) {
@@ -32,6 +37,7 @@ int zero_words(int *p, int64_t n, hipStream_t stream) {
 constexpr int kMaxDevices = 64;
 static std::mutex g_setup_mutex;
 static std::atomic<bool> g_ready[kMaxDevices];
+static void *g_scratch[kMaxDevices];                // device address of `scratch` on each GPU
 static std::atomic<int> g_spin_limit{kSpinLimit};
 
 int spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
@@ -43,9 +49,17 @@ int ensure_device_ready() {
     if (g_ready[dev].load(std::memory_order_acquire)) return SND_OK;
     std::lock_guard<std::mutex> lock(g_setup_mutex);
     if (g_ready[dev].load(std::memory_order_relaxed)) return SND_OK;
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return SND_ERR_LAUNCH;
+    g_scratch[dev] = ptr;
     if (configure_bwd_f32() != SND_OK || configure_bwd_bf16() != SND_OK || configure_bwd_f16() != SND_OK) return SND_ERR_LAUNCH;
     g_ready[dev].store(true, std::memory_order_release);
     return SND_OK;
+}
+static void *device_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    return g_ready[dev].load(std::memory_order_acquire) ? g_scratch[dev] : nullptr;
 }
 }  // namespace snd
 
@@ -117,6 +131,7 @@ const char *snd_status_string(int status) {
         case SND_ERR_LAUNCH: return "kernel launch failed";
         case SND_ERR_WORKSPACE: return "saved state (x, x_v, x_sd) or workspace missing or too small";
         case SND_ERR_ALIGN: return "saved state / workspace pointers must be 16-byte aligned";
+        case SND_ERR_TOO_LARGE: return "the problem needs more scratch than the static workspace holds (snd_static_workspace_bytes); use snd_bwd with a caller workspace";
         case SND_ERR_PIPELINE: return "a hand-over wait between blocks timed out in an earlier launch on this workspace: its outputs are NaN";
         default: return "unknown status";
     }
@@ -211,6 +226,24 @@ int snd_init(int device) {
     const int st = snd::ensure_device_ready();
     if (device != cur && hipSetDevice(cur) != hipSuccess) return SND_ERR_LAUNCH;
     return st;
+}
+
+int64_t snd_static_workspace_bytes(void) { return SND_STATIC_WORKSPACE_BYTES; }
+
+int snd_bwd_static(const snd_bwd_params *params, snd_stream_t stream) {
+    if (!params) return SND_ERR_NULL;
+    snd_plan plan;
+    int st = snd_make_plan(&params->f.shape, &plan);
+    if (st != SND_OK) return st;
+    if (plan.bwd_workspace_bytes > SND_STATIC_WORKSPACE_BYTES) return SND_ERR_TOO_LARGE;
+    st = snd::ensure_device_ready();                // no allocation: symbol lookup and kernel attributes, once per device
+    if (st != SND_OK) return st;
+    void *ws = snd::device_scratch();
+    if (!ws) return SND_ERR_LAUNCH;
+    snd_bwd_params q = *params;
+    q.workspace = ws;
+    q.workspace_bytes = SND_STATIC_WORKSPACE_BYTES;
+    return bwd_checked(&q, stream);
 }
 
 int snd_workspace_error(const void *workspace, snd_stream_t stream) {

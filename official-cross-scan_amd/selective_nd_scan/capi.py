@@ -70,6 +70,8 @@ def lib():
         _lib.snd_make_plan.argtypes = [C.POINTER(Shape), C.POINTER(Plan)]
         _lib.snd_fwd.argtypes = [C.POINTER(FwdParams), vp]
         _lib.snd_bwd.argtypes = [C.POINTER(BwdParams), vp]
+        _lib.snd_bwd_static.argtypes = [C.POINTER(BwdParams), vp]
+        _lib.snd_static_workspace_bytes.restype = C.c_int64
         _lib.snd_init.argtypes = [C.c_int]
         _lib.snd_workspace_error.argtypes = [vp, vp]
         _lib.snd_debug_set_spin_limit.argtypes = [C.c_int]
@@ -149,50 +151,6 @@ class FwdCall:
                   self.x, self.x_v, self.x_sd, schedule, directions)
         self.ws = torch.empty(plan.fwd_workspace_bytes // 4 + 4, **f32)
         self.params.workspace, self.params.workspace_bytes = self.ws.data_ptr(), plan.fwd_workspace_bytes
-
-    def launch(self, stream=None):
-        check(lib().snd_fwd(C.byref(self.params), _stream(stream)))
-
-
-class BwdCall:
-    """Gradient buffers, scratch and the filled snd_bwd_params of one backward.  launch() zero-fills
-    the accumulated gradients (as the reference host does, selective_scan_oflex.cpp:395-403) and
-    enqueues the kernel; launch_kernel_only() skips the zero-fill (timing)."""
-
-    def __init__(self, u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd,
-                 schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
-        import torch
-        self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, dout, x, x_v, x_sd)
-        shape = make_shape(u, delta, A, B)
-        st, plan = make_plan(shape)
-        check(st)
-        Dm = A.shape[0]
-        f32 = dict(device=u.device, dtype=torch.float32)
-        self.du = torch.empty((u.shape[0], Dm, u.shape[2], u.shape[3]), device=u.device, dtype=u.dtype)
-        self.ddelta = torch.empty_like(self.du)
-        self.dA = torch.zeros_like(A)
-        self.dB, self.dC = torch.zeros(B.shape, **f32), torch.zeros(Cc.shape, **f32)
-        self.dD = torch.zeros_like(D) if D is not None else None
-        self.dbias = torch.zeros(Dm, **f32) if delta_bias is not None else None
-        self.ddec = torch.zeros_like(A_decay) if A_decay is not None else None
-        self.ws = torch.empty(plan.bwd_workspace_bytes // 4 + 4, **f32)
-        bp = self.params = BwdParams()
-        _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd,
-                  schedule, directions)
-        bp.dout, bp.dout_dtype = dout.data_ptr(), _dt(dout)
-        bp.dout_batch_stride, bp.dout_d_stride, bp.dout_h_stride = dout.stride(0), dout.stride(1), dout.stride(2)
-        bp.du, bp.ddelta = self.du.data_ptr(), self.ddelta.data_ptr()
-        bp.dA, bp.dB, bp.dC = self.dA.data_ptr(), self.dB.data_ptr(), self.dC.data_ptr()
-        bp.dD, bp.ddelta_bias, bp.dA_decay = _ptr(self.dD), _ptr(self.dbias), _ptr(self.ddec)
-        bp.workspace, bp.workspace_bytes = self.ws.data_ptr(), plan.bwd_workspace_bytes
-
-    def zero(self):
-        for t in (self.dA, self.dB, self.dC, self.dD, self.dbias, self.ddec):
-            if t is not None:
-                t.zero_()
-
-    def launch_kernel_only(self, stream=None):
-        check(lib().snd_bwd(C.byref(self.params), _stream(stream)))
 
     def launch(self, stream=None):
         check(lib().snd_fwd(C.byref(self.params), _stream(stream)))

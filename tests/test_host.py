@@ -12,7 +12,8 @@ import capi
 def test_library_exports_every_declared_symbol():
     names = capi.declared_symbols()
     assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd", "snd_init",
-                          "snd_workspace_error", "snd_debug_set_spin_limit"}
+                          "snd_workspace_error", "snd_debug_set_spin_limit", "snd_bwd_static",
+                          "snd_static_workspace_bytes"}
     lib = capi.lib()
     for n in names:
         assert getattr(lib, n) is not None, n
@@ -202,6 +203,27 @@ def test_tile_extent_choice():
     assert tiles(14, 14) == (2, 2) and tiles(28, 28) == (4, 4) and tiles(7, 7) == (1, 1) and tiles(21, 35) == (3, 5)
     assert tiles(56, 56) == (7, 7) and tiles(64, 64) == (8, 8) and tiles(512, 512) == (64, 64) and tiles(200, 336) == (25, 42)
     assert tiles(1, 37) == (1, 5)                 # 294 vs 320 padded cells: not worth the smaller tile
+
+
+def test_static_workspace_entry_point_validates_on_the_host():
+    """snd_bwd_static refuses bad calls before it touches a GPU: null parameters, bad shapes, and shapes
+    whose scratch does not fit the static workspace (with the status code and text that say so)."""
+    lib = capi.lib()
+    limit = lib.snd_static_workspace_bytes()
+    assert limit == 64 << 20
+    assert lib.snd_bwd_static(None, None) == -1
+    bp = capi.BwdParams()
+    bp.f.shape = capi.Shape(1, 6, 4, 4, 16, 4, 6, capi.SND_F32)          # dim % n_groups != 0
+    assert lib.snd_bwd_static(C.byref(bp), None) == -2
+    big = capi.Shape(64, 768, 56, 56, 16, 4, 768, capi.SND_F32)          # needs 176 MB of adjoint rows
+    st, plan = capi.make_plan(big)
+    assert st == 0 and plan.bwd_workspace_bytes > limit
+    bp.f.shape = big
+    assert lib.snd_bwd_static(C.byref(bp), None) == -8
+    assert b"static workspace" in lib.snd_status_string(-8)
+    for cfg in [(64, 192, 56, 56, 16, 4), (64, 768, 14, 14, 16, 4), (2, 192, 200, 336, 16, 4), (1, 256, 512, 512, 16, 4)]:
+        st, plan = capi.make_plan(capi.Shape(*cfg, cfg[1], capi.SND_F32))
+        assert st == 0 and plan.bwd_workspace_bytes <= limit, cfg        # every benchmark configuration fits
 
 
 def test_pipeline_error_contract_on_the_host():
