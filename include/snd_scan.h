@@ -64,6 +64,7 @@ typedef struct snd_shape {
  *     x     [batch, dim, dstate, n_chunks_x, x_inner]     (h at the right edge of every column tile)
  *     x_sd  [batch, dim, dstate, n_chunks_x, x_inner]     (row-only scan s at the same places)
  *     x_v   [batch, dim, dstate, n_chunks_y, xv_inner]    (h at the last row of every row strip)
+ * (sized so that either kernel family fits where both apply).
  * Their contents are private to this library; bwd does NOT modify them (a second backward over
  * the same saved state is valid, unlike the reference, bwd.cuh:489-491,614-619,725-727). */
 typedef struct snd_plan {
@@ -74,9 +75,12 @@ typedef struct snd_plan {
     int64_t fwd_workspace_bytes;               /* scratch fwd uses when it splits planes into strips
                                                   (16-byte aligned, uninitialised; one row per plane) */
     int32_t auto_schedule;                     /* what SND_SCHED_AUTO resolves to in the forward for this shape
-                                                  (PLANE, STRIPS or BANDS): a caller may skip the fwd workspace for PLANE */
+                                                  (PLANE, STRIPS, BANDS or WAVEFRONT): a caller may skip the fwd
+                                                  workspace for PLANE and WAVEFRONT */
     int32_t auto_bwd_jobs;                     /* jobs per plane chunk SND_SCHED_AUTO gives the backward: 0 = one
-                                                  block per plane chunk, n_chunks_y = one per strip, 2-4 = bands */
+                                                  block per plane chunk (also when auto_schedule is WAVEFRONT: then
+                                                  the backward runs WAVEFRONT too and needs no workspace),
+                                                  n_chunks_y = one per strip, 2-4 = bands */
 } snd_plan;
 
 /* How a launch maps work to blocks.  The reference has one fixed mapping (one block per
@@ -87,8 +91,13 @@ typedef struct snd_plan {
  *   BANDS   one block per band of consecutive strips, 2-4 bands per plane, handed over like strips but
  *           only at band ends.  For more plane chunks than the chip holds blocks at once (backward at B=64, D=192, 56x56, N=16:
  *           768 chunks, 512 slots), where whole-plane blocks leave the last round half empty.  Needs
- *           the workspace. */
-typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2, SND_SCHED_BANDS = 3 } snd_schedule;
+ *           the workspace.
+ *   WAVEFRONT  the second kernel family, for 1-4 states per channel and planes up to 512 columns wide: a
+ *           block per (batch, channel), a wave per 64-column row segment, the segments of a plane advancing
+ *           as an anti-diagonal wavefront (what AUTO picks whenever it applies).  Its saved state has a
+ *           layout of its own: fwd and bwd of one call pair must both run WAVEFRONT or both run one of the
+ *           three tile schedules above (AUTO decides by shape alone, so AUTO on both sides always agrees). */
+typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2, SND_SCHED_BANDS = 3, SND_SCHED_WAVEFRONT = 4 } snd_schedule;
 
 /* Scan origin per group.  The reference scans every group from the top-left corner and leaves the
  * per-group order as a TODO (fwd.cuh:140); its callers build the four corner directions of the

@@ -13,6 +13,12 @@ int launch_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
 int launch_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
+int launch_wave_fwd_f32(const snd_fwd_params &p, hipStream_t stream);
+int launch_wave_fwd_bf16(const snd_fwd_params &p, hipStream_t stream);
+int launch_wave_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
+int launch_wave_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
+int launch_wave_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
+int launch_wave_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
 int configure_bwd_f32();
 int configure_bwd_bf16();
 int configure_bwd_f16();
@@ -82,6 +88,15 @@ int check_shape(const snd_shape &s) {
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+// Which kernel family a call runs: the row-segment wavefront when asked for, or under AUTO whenever the
+// shape qualifies (1-4 states, at most 512 columns); the tile kernels otherwise.  -1: WAVEFRONT asked for a
+// shape it does not cover.
+int use_wavefront(const snd_shape &s, int schedule) {
+    const bool fits = snd::wave_family_fits(s.ncols, s.dstate);
+    if (schedule == SND_SCHED_WAVEFRONT) return fits ? 1 : -1;
+    return schedule == SND_SCHED_AUTO && fits ? 1 : 0;
+}
+
 // The kernels address inside one batch image with unsigned 32-bit BYTE offsets from a scalar base
 // and form row offsets with 24-bit multiplies: a (count x stride) walk plus rows must stay below
 // 2^32 bytes and a row pitch below 2^23 bytes.
@@ -147,13 +162,21 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->n_chunks_y = g.nCY;
     plan->x_inner = g.Hp;
     plan->xv_inner = g.Wp;
-    plan->x_elems = planes * g.nCX * g.Hp;
+    const bool wave = snd::wave_family_fits(shape->ncols, shape->dstate);
+    if (wave) {
+        // either family may run on this shape: the inner extents grow until the wavefront layout fits too
+        const snd::WaveGeo wg = snd::make_wave_geo(shape->nrows, shape->ncols, shape->dstate);
+        const int64_t need_x = (snd::wave_x_plane(wg) + g.nCX - 1) / g.nCX, need_xv = (snd::wave_xv_plane(wg) + g.nCY - 1) / g.nCY;
+        if (need_x > plan->x_inner) plan->x_inner = (int32_t)((need_x + 3) / 4 * 4);
+        if (need_xv > plan->xv_inner) plan->xv_inner = (int32_t)((need_xv + 3) / 4 * 4);
+    }
+    plan->x_elems = planes * g.nCX * plan->x_inner;
     plan->x_sd_elems = plan->x_elems;
-    plan->x_v_elems = planes * g.nCY * g.Wp;
+    plan->x_v_elems = planes * g.nCY * plan->xv_inner;
     // strip-pipeline sync words, then one row per plane: forward, h handed from a strip to the strip
     // below (strip schedule only); backward, the adjoint G = a*g handed to the strip above
     const int64_t sync_bytes = snd::sync_words(plane_chunks(*shape), g.nCY) * (int64_t)sizeof(int);
-    const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);
+    const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);   // (tile layout: Wp = nCX * 8)
     plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
     const int fwd_jobs = snd::fwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
@@ -161,6 +184,10 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
     plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
                                               (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
+    if (wave) {
+        plan->auto_schedule = SND_SCHED_WAVEFRONT;
+        plan->auto_bwd_jobs = 0;
+    }
     return SND_OK;
 }
 
@@ -173,8 +200,17 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols,
                 esize(params->out_dtype)))
         return SND_ERR_STRIDE;
-    if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_BANDS) return SND_ERR_SHAPE;
+    if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_WAVEFRONT) return SND_ERR_SHAPE;
     if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
+    const int wave = use_wavefront(params->shape, params->schedule);
+    if (wave < 0) return SND_ERR_SHAPE;
+    if (wave) {                                     // needs no workspace
+        switch (params->shape.in_dtype) {
+            case SND_F32: return snd::launch_wave_fwd_f32(*params, (hipStream_t)stream);
+            case SND_BF16: return snd::launch_wave_fwd_bf16(*params, (hipStream_t)stream);
+            default: return snd::launch_wave_fwd_f16(*params, (hipStream_t)stream);
+        }
+    }
     if (params->workspace) {
         snd_plan plan;
         snd_make_plan(&params->shape, &plan);
@@ -203,13 +239,22 @@ static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
     snd_plan plan;
     st = snd_make_plan(&params->f.shape, &plan);
     if (st != SND_OK) return st;
-    if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
-    if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
-    if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_BANDS) return SND_ERR_SHAPE;
+    if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_WAVEFRONT) return SND_ERR_SHAPE;
     if (params->f.directions != SND_DIR_TOPLEFT && params->f.directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
     if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
                 params->f.shape.ncols, esize(params->dout_dtype)))
         return SND_ERR_STRIDE;
+    const int wave = use_wavefront(params->f.shape, params->f.schedule);
+    if (wave < 0) return SND_ERR_SHAPE;
+    if (wave) {                                     // needs no workspace
+        switch (params->f.shape.in_dtype) {
+            case SND_F32: return snd::launch_wave_bwd_f32(*params, (hipStream_t)stream);
+            case SND_BF16: return snd::launch_wave_bwd_bf16(*params, (hipStream_t)stream);
+            default: return snd::launch_wave_bwd_f16(*params, (hipStream_t)stream);
+        }
+    }
+    if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
+    if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
     switch (params->f.shape.in_dtype) {
         case SND_F32: return snd::launch_bwd_f32(*params, (hipStream_t)stream);
         case SND_BF16: return snd::launch_bwd_bf16(*params, (hipStream_t)stream);

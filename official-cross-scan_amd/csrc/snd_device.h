@@ -373,6 +373,76 @@ __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, in
     return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 768 : 1536);
 }
 
+
+// ---------------------------------------------------------------- row-segment wavefront (1-4 states per channel)
+// With one to four states per channel a lane-per-(channel, state) mapping leaves most of the machine idle
+// (256 channels x 1 state of a 512x512 plane are 256 lanes of work).  The second kernel family turns the
+// plane itself into the parallel axis: the 64 lanes of a wave are 64 consecutive columns of one row (a
+// row segment), the states of the channel live in registers of the lane, rows are taken one after the
+// other, and the segments of a plane - one wave each, up to eight per block - advance as an anti-diagonal
+// wavefront: wave w works on row i while wave w+1 works on row i-2 (forward; mirrored in the backward).
+// Inside a segment the recurrence along the row, h_j = a_j*h_{j-1} + y_j, is resolved by a wave-wide
+// inclusive scan of the affine maps (a_j, y_j) in six DPP steps (row_shr 1, 2, 4, 8, row_bcast 15, 31);
+// neighbours in the row come from wave_shr:1 / wave_shl:1; the state at a segment's last column goes to
+// the next wave through a few LDS words per row.
+struct WaveGeo {
+    int nseg;                      // row segments (waves per plane): ceil(W / 64)
+    int R;                         // rows per band: row-checkpoint spacing = rows the backward holds in registers
+    int nBands;                    // ceil(H / R)
+    int Hp, Wp;                    // nBands * R, nseg * 64
+};
+constexpr int kSeg = 64;
+constexpr int kMaxSeg = 8;
+__host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 && W <= kSeg * kMaxSeg; }
+__host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
+    WaveGeo g;
+    g.nseg = (W + kSeg - 1) / kSeg;
+    g.R = N <= 2 ? 8 : 4;
+    g.nBands = (H + g.R - 1) / g.R;
+    g.Hp = g.nBands * g.R;
+    g.Wp = g.nseg * kSeg;
+    return g;
+}
+// Saved state of this family, per (batch, channel, state) plane, fp32:
+//   x    [segment w][2][Hp]   h, then a, at column 64w-1 of every row (what segment w needs from its left)
+//   x_sd [segment w][2][Hp]   s at the same places (second half unused)
+//   x_v  [band][2][Wp]        h, then a, on the last row of every band
+__host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
+__host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
+
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_old(float old, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+// v of the lane below (lane 0 keeps `edge`): the left neighbour when lanes run along the scan direction
+__device__ __forceinline__ float from_prev_lane(float v, float edge) { return dpp_old<0x138, 0xF>(edge, v); }   // wave_shr:1
+// v of the lane above (lane 63 keeps `edge`)
+__device__ __forceinline__ float from_next_lane(float v, float edge) { return dpp_old<0x130, 0xF>(edge, v); }   // wave_shl:1
+
+// Inclusive scan over the 64 lanes of the affine maps t -> a*t + y (and t -> a*t + s, sharing a):
+// afterwards lane j holds a = prod_{k<=j} a_k, y = sum_{k<=j} (prod_{k<m<=j} a_m) y_k, s likewise, so that
+// with a value c entering lane 0 from the left the recurrence's solution is a*c + y.
+// Three interleaved chains per level keep two instructions between a VALU write and the DPP read of the
+// same register (the hazard distance); lanes without a source (and rows masked off) keep their values.
+#define SND_SCAN3_LVL(ctrl, rm)                                                  \
+    "v_fmac_f32_dpp %0, %0, %2 " ctrl " row_mask:" rm " bank_mask:0xf\n\t"        \
+    "v_fmac_f32_dpp %1, %1, %2 " ctrl " row_mask:" rm " bank_mask:0xf\n\t"        \
+    "v_mul_f32_dpp %2, %2, %2 " ctrl " row_mask:" rm " bank_mask:0xf\n\t"
+__device__ __forceinline__ void wave_scan3(float &y, float &s, float &a) {
+    asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
+            SND_SCAN3_LVL("row_shr:8", "0xf") SND_SCAN3_LVL("row_bcast:15", "0xa") SND_SCAN3_LVL("row_bcast:31", "0xc")
+        : "+v"(y), "+v"(s), "+v"(a));
+}
+// Sum over the 64 lanes; the total ends in lane 63.
+__device__ __forceinline__ float wave_sum_to_last(float v) {
+    v += dpp_old<0x111, 0xF>(0.f, v);
+    v += dpp_old<0x112, 0xF>(0.f, v);
+    v += dpp_old<0x114, 0xF>(0.f, v);
+    v += dpp_old<0x118, 0xF>(0.f, v);
+    v += dpp_old<0x142, 0xA>(0.f, v);
+    v += dpp_old<0x143, 0xC>(0.f, v);
+    return v;
+}
+
 // Re-derive a thread's element maps from an opaque copy of its id.  Used at the top of each staging
 // section so that the compiler recomputes a few integer ops per tile instead of hoisting dozens of
 // loop-invariant addresses out of the tile loop and keeping (or spilling) them across it.

@@ -112,8 +112,17 @@ std::atomic<bool> g_check_pipeline{[] { const char *e = std::getenv("SND_CHECK_P
 
 int resolve_schedule(int64_t schedule) {
     if (schedule < 0) return g_schedule.load();
-    TORCH_CHECK(schedule >= SND_SCHED_AUTO && schedule <= SND_SCHED_BANDS, "schedule must be 0 (auto), 1 (plane), 2 (strips) or 3 (bands)");
+    TORCH_CHECK(schedule >= SND_SCHED_AUTO && schedule <= SND_SCHED_WAVEFRONT,
+                "schedule must be 0 (auto), 1 (plane), 2 (strips), 3 (bands) or 4 (row-segment wavefront)");
     return (int)schedule;
+}
+// whether a call with this schedule runs one of the pipelined tile schedules (they need the workspace)
+bool pipelined(int sched, int auto_choice) {
+    const int s = sched == SND_SCHED_AUTO ? auto_choice : sched;
+    return s == SND_SCHED_STRIPS || s == SND_SCHED_BANDS;
+}
+bool wavefront(int sched, const snd_plan &plan) {
+    return sched == SND_SCHED_WAVEFRONT || (sched == SND_SCHED_AUTO && plan.auto_schedule == SND_SCHED_WAVEFRONT);
 }
 void check_pipeline(const at::Tensor &ws, hipStream_t stream, const char *what) {
     if (!ws.defined() || !g_check_pipeline.load()) return;
@@ -168,8 +177,7 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     const int sched = resolve_schedule(schedule);
     p.schedule = sched;
     at::Tensor ws;
-    if (sched == SND_SCHED_STRIPS || sched == SND_SCHED_BANDS ||
-        (sched == SND_SCHED_AUTO && c.plan.auto_schedule != SND_SCHED_PLANE)) {
+    if (pipelined(sched, c.plan.auto_schedule)) {
         ws = torch::empty({(c.plan.fwd_workspace_bytes + 3) / 4}, f32);
         p.workspace = ws.data_ptr();
         p.workspace_bytes = c.plan.fwd_workspace_bytes;
@@ -229,7 +237,9 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     if (D_.has_value()) dD = accP.narrow(0, oD, dim);
     if (delta_bias_.has_value()) ddelta_bias = accP.narrow(0, oBias, dim);
     if (A_decay_.has_value()) dA_decay = accP.narrow(0, oDec, 1);
-    at::Tensor ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
+    const int sched = resolve_schedule(schedule);
+    at::Tensor ws;                                  // the wavefront kernels need none
+    if (!wavefront(sched, c.plan)) ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
 
     snd_bwd_params p;
     memset(&p, 0, sizeof(p));
@@ -243,13 +253,14 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     p.dD = dD.defined() ? dD.data_ptr<float>() : nullptr;
     p.ddelta_bias = ddelta_bias.defined() ? ddelta_bias.data_ptr<float>() : nullptr;
     p.dA_decay = dA_decay.defined() ? dA_decay.data_ptr<float>() : nullptr;
-    p.workspace = ws.data_ptr();
-    p.workspace_bytes = c.plan.bwd_workspace_bytes;
-    p.f.schedule = resolve_schedule(schedule);
+    p.workspace = ws.defined() ? ws.data_ptr() : nullptr;
+    p.workspace_bytes = ws.defined() ? c.plan.bwd_workspace_bytes : 0;
+    p.f.schedule = sched;
     p.f.directions = (int32_t)directions;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
-    if (c.plan.auto_bwd_jobs != 0 || p.f.schedule == SND_SCHED_STRIPS || p.f.schedule == SND_SCHED_BANDS) check_pipeline(ws, stream, "bwd");
+    if (sched == SND_SCHED_STRIPS || sched == SND_SCHED_BANDS || (sched == SND_SCHED_AUTO && c.plan.auto_bwd_jobs != 0))
+        check_pipeline(ws, stream, "bwd");
 
     // host.cpp:432-438: cast dB/dC to the input dtype, fold channel groups that share a delta
     std::vector<at::Tensor> result = {du, ddelta, dA, dB.to(B.dtype()), dC.to(C.dtype()), dD, ddelta_bias, dA_decay};
@@ -277,7 +288,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("dout"), py::arg("x"), py::arg("x_v"),
           py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0, py::arg("schedule") = -1);
     m.def("set_schedule", [](int mode) {
-        TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_BANDS, "schedule must be 0 (auto), 1 (plane), 2 (strips) or 3 (bands, backward)");
+        TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_WAVEFRONT, "schedule must be 0 (auto), 1 (plane), 2 (strips), 3 (bands) or 4 (row-segment wavefront)");
         g_schedule.store(mode);
     }, "Default block mapping of calls that pass no schedule: 0 auto, 1 one block per plane chunk, 2 pipelined row strips, 3 bands");
     m.def("set_debug", [](bool on) { g_check_pipeline.store(on); },

@@ -1,0 +1,7 @@
+// Row-segment wavefront backward (1-4 states per channel): instantiations for the three input dtypes.
+#include "snd_wave_bwd_kernel.h"
+namespace snd {
+int launch_wave_bwd_f32(const snd_bwd_params &p, hipStream_t stream) { return launch_wave_bwd_t<float>(p, stream); }
+int launch_wave_bwd_bf16(const snd_bwd_params &p, hipStream_t stream) { return launch_wave_bwd_t<bf16_t>(p, stream); }
+int launch_wave_bwd_f16(const snd_bwd_params &p, hipStream_t stream) { return launch_wave_bwd_t<f16_t>(p, stream); }
+}  // namespace snd

@@ -1,0 +1,299 @@
+// Backward kernel of the 2D-CrossScan selective scan for one to four states per channel (gfx950):
+// the row-segment wavefront, run in reverse.
+//
+// Same gradients as snd_bwd_kernel.h (reference: selective_scan_bwd_kernel_oflex.cuh:91-902).  With
+// G = a*g, Gs = a*gs and every out-of-range term zero, per (batch, channel, state) plane:
+//     g[i,j]  = dout*C + G[i,j+1] + G[i+1,j] - 0.5*(a[i,j+1] + a[i+1,j])*G[i+1,j+1]
+//     gs[i,j] = -dout*C + Gs[i,j+1]
+//     dbu     = g + gs + 0.25*dout*C
+//     da*a    = g*(h - bu) + gs*(s - bu) - 0.5*a*(G[i+1,j]*h[i,j-1] + G[i,j+1]*h[i-1,j])
+// and from these du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay as listed in snd_bwd_kernel.h.
+//
+// Mapping as in snd_wave_fwd_kernel.h: a block per (batch, channel), a wave per 64-column row segment, the
+// states in registers.  Along a row the adjoint is first order towards the left,
+//     G_j = a_j*G_{j+1} + a_j*z_j,   z_j = dout*C + G[i+1,j] - 0.5*(a[i,j+1] + a[i+1,j])*G[i+1,j+1],
+// so a wave resolves a row with one DPP scan, exactly like the forward - provided its lanes run against
+// the columns.  Every load, store and the whole adjoint sweep therefore use the mirrored order (lane l =
+// column 64w + 63 - l); only the recomputation of h and s, which runs with the columns, sees its inputs and
+// leaves its results through a lane reversal (ds_bpermute: a register crossbar move, no LDS memory).
+// A wave handles its segment band by band (R rows), bottom band first: recompute h, s of the band's rows
+// from the forward's checkpoints (row above the band from x_v, what entered the segment on every row from
+// x / x_sd: no wave waits for another here), then sweep the band's rows bottom-up.  The sweep needs G, Gs, a
+// of the segment on the right at its first column: wave w runs one band behind wave w+1 and finds them in
+// LDS (one block barrier per band, no polling).  dB, dC leave as one global atomic per element and channel
+// (a wave-wide instruction covers 256 consecutive bytes), du / ddelta as whole row segments.
+#pragma once
+#include "snd_device.h"
+
+namespace snd {
+
+__device__ __forceinline__ void wave_glb_add(float *p, float v) {
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, int NS>
+__global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
+    constexpr int R = NS <= 2 ? 8 : 4;               // rows per band
+    // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and state
+    __shared__ float4 sHO[2][kMaxSeg][R][NS];
+
+    const snd_fwd_params &f = p.f;
+    const snd_shape &sh = f.shape;
+    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
+    const int rg = Dm / G, rd = Dm / sh.delta_dim;
+    int pair, chunk;
+    if (!xcd_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
+    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nseg = wg.nseg;
+    const bool multi = nseg > 1;
+
+    const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
+    const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
+    const int jm = w * kSeg + 63 - lane;             // this lane's column (mirrored order)
+    const bool jin = jm < W;
+    const int jc = jin ? jm : W - 1;
+    const int mc = fh ? W - 1 - jc : jc;
+    const int jn = w * kSeg + lane;                  // natural order (row checkpoints, recomputation)
+    const int rev_addr = (63 - lane) * 4;
+    auto mirror = [&](float v) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(rev_addr, __builtin_bit_cast(int, v)));
+    };
+    auto bcast = [](float v, int src_lane) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
+    };
+
+    float Av[NS], A2[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+        Av[n] = n < N ? f.A[(int64_t)c * f.A_d_stride + (int64_t)n * f.A_dstate_stride] : 0.f;
+        A2[n] = Av[n] * kLog2e;
+    }
+    const float ld = f.A_decay ? __log2f(f.A_decay[0]) : 0.f;
+    const float Dv = f.D ? f.D[c] : 0.f;
+    const float bias = f.delta_bias ? f.delta_bias[c / rd] : 0.f;
+    const bool softplus = f.delta_softplus != 0;
+    const bool want_decay = p.dA_decay != nullptr;
+
+    constexpr int ESZ = (int)sizeof(T);
+    const T *Bb = (const T *)f.B + (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
+    const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
+    const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chunk : c) * f.u_d_stride;
+    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(c / rd) * f.delta_d_stride;
+    const int sh_do = p.dout_dtype == SND_F32 ? 2 : 1;
+    const void *dob = (const char *)p.dout + (((int64_t)b * p.dout_batch_stride + (int64_t)c * p.dout_d_stride) << sh_do);
+    T *dub = (T *)p.du + ((int64_t)b * Dm + c) * H * W;                 // du, ddelta: dense [b, c, H, W]
+    T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + c) * H * W;
+    float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;               // dense [b, g, N, H, W]
+    float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
+    const int UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ, BhB = (int)f.B_h_stride * ESZ,
+              ChB = (int)f.C_h_stride * ESZ, DohB = (int)p.dout_h_stride << sh_do, WB = W * ESZ, W4 = W * 4;
+    const int64_t BsB = f.B_dstate_stride * ESZ, CsB = f.C_dstate_stride * ESZ, HW4 = (int64_t)H * W * 4;
+    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc << sh_do, col4 = (uint32_t)mc * 4;
+
+    // saved state of this plane set (layouts in snd_device.h)
+    const int64_t plane0 = ((int64_t)b * Dm + c) * N;
+    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn;
+    const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
+    const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
+
+    // inputs of one band: rows in mirrored lane order; the row above the band (h0, a0) in natural order;
+    // what entered the segment from the left on rows i0-1 .. i0+R-1, one row per lane (ch, cs, ca)
+    struct In { float u[R], d[R], o[R], b[R][NS], c[R][NS], h0[NS], a0[NS], ch[NS], cs[NS], ca[NS]; };
+    auto load_band = [&](In &q, int band) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = min(band * R + r, H - 1);                      // always in bounds
+            const int mr = mad24(i, rs, r0m);
+            q.u[r] = jin ? ldg_b(ub, mad24(mr, UhB, colB)) : 0.f;
+            q.d[r] = ldg_b(db, mad24(mr, DhB, colB));
+            q.o[r] = jin ? ld_f32_b(dob, mad24(mr, DohB, colO), p.dout_dtype) : 0.f;
+#pragma unroll
+            for (int n = 0; n < NS; ++n) {
+                const int sn = n < N ? n : 0;
+                const float vb = ldg_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
+                const float vc = ldg_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
+                q.b[r][n] = (jin && n < N) ? vb : 0.f;
+                q.c[r][n] = (jin && n < N) ? vc : 0.f;
+            }
+        }
+        const int row = band * R - 1 + lane;
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+            q.h0[n] = 0.f; q.a0[n] = 0.f; q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
+            if (n < N) {
+                if (band > 0) {
+                    const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
+                    q.h0[n] = __builtin_nontemporal_load(src);
+                    q.a0[n] = __builtin_nontemporal_load(src + wg.Wp);
+                }
+                if (w > 0 && lane <= R && row >= 0) {
+                    const int64_t o = (int64_t)n * wave_x_plane(wg) + row;
+                    q.ch[n] = xh[o];
+                    q.ca[n] = xh[o + wg.Hp];
+                    q.cs[n] = xs[o];
+                }
+            }
+        }
+    };
+
+    float Gd[NS], ad[NS], GdEdge[NS];               // G, a of the row below at this column; G[i+1, 64(w+1)]
+    float dA_acc[NS];
+    float dec_acc = 0.f, dD_acc = 0.f, dbias_acc = 0.f;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) { Gd[n] = 0.f; ad[n] = 0.f; GdEdge[n] = 0.f; dA_acc[n] = 0.f; }
+
+    In cur, nxt;
+    load_band(cur, wg.nBands - 1);
+    int step = nseg - 1 - w;                         // the waves on the right go first
+    if (multi)
+        for (int e = 0; e < nseg - 1 - w; ++e) __syncthreads();
+
+    for (int band = wg.nBands - 1; band >= 0; --band) {
+        if (band > 0) load_band(nxt, band - 1);
+
+        // ---- recompute h, s on the band's rows (with the columns), results back in mirrored order
+        float hT[R][NS], sT[R][NS], dl[R], dsp[R], hTop[NS];
+        {
+            float hp[NS], ap[NS], hdiag[NS];
+#pragma unroll
+            for (int n = 0; n < NS; ++n) {
+                hp[n] = cur.h0[n];
+                ap[n] = cur.a0[n];
+                hdiag[n] = bcast(cur.ch[n], 0);
+                hTop[n] = mirror(cur.h0[n]);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float raw = cur.d[r] + bias;
+                float sg = 1.f;
+                dl[r] = softplus ? softplus20(raw, sg) : raw;
+                dsp[r] = sg;
+                if (band * R + r < H) {
+                    const float dl_n = mirror(dl[r]), dlu_n = mirror(dl[r] * cur.u[r]);
+#pragma unroll
+                    for (int n = 0; n < NS; ++n) {
+                        const float hin = bcast(cur.ch[n], r + 1), sin_ = bcast(cur.cs[n], r + 1), ain = bcast(cur.ca[n], r + 1);
+                        const float a = fast_exp2(fmaf(dl_n, A2[n], ld));
+                        const float bu = mirror(cur.b[r][n]) * dlu_n;
+                        const float a_l = from_prev_lane(a, ain);              // a[i, j-1]
+                        const float h_d = from_prev_lane(hp[n], hdiag[n]);     // h[i-1, j-1]
+                        const float X = fmaf(-0.5f * (ap[n] + a_l), h_d, hp[n]);
+                        float Y = fmaf(a, X, bu), S = bu, Ap = a;
+                        wave_scan3(Y, S, Ap);
+                        const float h = fmaf(Ap, hin, Y);
+                        const float s = fmaf(Ap, sin_, S);
+                        hT[r][n] = mirror(h);
+                        sT[r][n] = mirror(s);
+                        hp[n] = h;
+                        ap[n] = a;
+                        hdiag[n] = hin;
+                    }
+                } else {
+#pragma unroll
+                    for (int n = 0; n < NS; ++n) { hT[r][n] = 0.f; sT[r][n] = 0.f; }
+                }
+            }
+        }
+
+        // ---- adjoint sweep over the band's rows, bottom-up (against the columns)
+#pragma unroll
+        for (int r = R - 1; r >= 0; --r) {
+            const int i = band * R + r;
+            if (i < H) {
+                const float dov = cur.o[r], uv = cur.u[r], dlv = dl[r];
+                const float dlu = dlv * uv;
+                const int mr = mad24(i, rs, r0m);
+                float qsum = 0.f, psum = 0.f;
+#pragma unroll
+                for (int n = 0; n < NS; ++n) {
+                    // what the segment on the right left for this row: G, Gs, a at column 64(w+1)
+                    float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (w + 1 < nseg) in = sHO[(step + 1) & 1][w + 1][r][n];
+                    const float hin = bcast(cur.ch[n], r + 1);                 // h[i, 64w-1]
+                    const float Bv = cur.b[r][n], Cv = cur.c[r][n];
+                    const float a = fast_exp2(fmaf(dlv, A2[n], ld));
+                    const float bu = Bv * dlu;
+                    const float dyC = dov * Cv;
+                    const float a_r = from_prev_lane(a, in.z);                 // a[i, j+1]
+                    const float Gdiag = from_prev_lane(Gd[n], GdEdge[n]);      // G[i+1, j+1]
+                    const float z = fmaf(-0.5f * (a_r + ad[n]), Gdiag, dyC + Gd[n]);
+                    float Y = a * z, S = -a * dyC, Ap = a;
+                    wave_scan3(Y, S, Ap);
+                    const float Gt = fmaf(Ap, in.x, Y), Gst = fmaf(Ap, in.y, S);   // G[i,j], Gs[i,j]
+                    const float Gr = from_prev_lane(Gt, in.x), Gsr = from_prev_lane(Gst, in.y);
+                    const float g_ = Gr + z, gs = Gsr - dyC;
+                    const float dbu = fmaf(0.25f, dyC, g_ + gs);
+                    const float hv = hT[r][n], sv = sT[r][n];
+                    const float h_l = from_next_lane(hv, hin);                 // h[i, j-1]
+                    const float h_u = r > 0 ? hT[r > 0 ? r - 1 : 0][n] : hTop[n];
+                    const float hs = hv - sv, sb = sv - bu;
+                    const float cross = fmaf(Gd[n], h_l, Gr * h_u);
+                    const float da = fmaf(-0.5f * a, cross, fmaf(g_, hs, (g_ + gs) * sb));
+                    dA_acc[n] = fmaf(dlv, da, dA_acc[n]);
+                    if (want_decay) dec_acc += da;
+                    qsum = fmaf(dbu, Bv, qsum);
+                    psum = fmaf(Av[n], da, psum);
+                    if (jin && n < N) {
+                        const int64_t o = (int64_t)n * HW4 + (uint32_t)mad24(mr, W4, col4);
+                        wave_glb_add((float *)((char *)dBg + o), dbu * dlu);
+                        wave_glb_add((float *)((char *)dCg + o), dov * fmaf(0.25f, bu, hs));
+                    }
+                    GdEdge[n] = in.x;
+                    Gd[n] = Gt;
+                    ad[n] = a;
+                    if (multi && lane == 63 && w > 0) sHO[step & 1][w][r][n] = make_float4(Gt, Gst, a, 0.f);
+                }
+                const float duv = fmaf(Dv, dov, dlv * qsum);
+                const float ddl = fmaf(uv, qsum, psum) * dsp[r];
+                if (jin) {
+                    dD_acc = fmaf(dov, uv, dD_acc);
+                    dbias_acc += ddl;
+                    const uint32_t o = mad24(mr, WB, colB);
+                    stg_b(dub, o, duv);
+                    stg_b(ddb, o, ddl);
+                }
+            }
+        }
+        if (multi) { __syncthreads(); ++step; }
+        cur = nxt;
+    }
+    if (multi)
+        for (int e = 0; e < w; ++e) __syncthreads();
+
+    // ---- per-channel sums leave the kernel: one atomic per wave and value
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+        const float t = wave_sum_to_last(dA_acc[n]);
+        if (lane == 63 && n < N) wave_glb_add(p.dA + (int64_t)c * N + n, t);
+    }
+    {
+        const float td = wave_sum_to_last(dD_acc), tb = wave_sum_to_last(dbias_acc);
+        if (lane == 63) {
+            if (p.dD) wave_glb_add(p.dD + c, td);
+            if (p.ddelta_bias) wave_glb_add(p.ddelta_bias + c, tb);
+        }
+    }
+    if (want_decay) {
+        const float t = wave_sum_to_last(dec_acc);
+        if (lane == 63) wave_glb_add(p.dA_decay, t / f.A_decay[0]);
+    }
+}
+
+template <typename T, int NS>
+static int launch_wave_bwd_ns(const snd_bwd_params &p, hipStream_t stream) {
+    const snd_shape &sh = p.f.shape;
+    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
+    const int grid = xcd_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    hipLaunchKernelGGL((wave_bwd_kernel<T, NS>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
+    return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
+    const int N = p.f.shape.dstate;
+    return N == 1 ? launch_wave_bwd_ns<T, 1>(p, stream) : N == 2 ? launch_wave_bwd_ns<T, 2>(p, stream)
+                                                                  : launch_wave_bwd_ns<T, 4>(p, stream);
+}
+
+}  // namespace snd

@@ -1,0 +1,7 @@
+// Row-segment wavefront forward (1-4 states per channel): instantiations for the three input dtypes.
+#include "snd_wave_fwd_kernel.h"
+namespace snd {
+int launch_wave_fwd_f32(const snd_fwd_params &p, hipStream_t stream) { return launch_wave_fwd_t<float>(p, stream); }
+int launch_wave_fwd_bf16(const snd_fwd_params &p, hipStream_t stream) { return launch_wave_fwd_t<bf16_t>(p, stream); }
+int launch_wave_fwd_f16(const snd_fwd_params &p, hipStream_t stream) { return launch_wave_fwd_t<f16_t>(p, stream); }
+}  // namespace snd

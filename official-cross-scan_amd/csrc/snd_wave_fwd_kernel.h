@@ -1,0 +1,193 @@
+// Forward kernel of the 2D-CrossScan selective scan for one to four states per channel (gfx950):
+// the row-segment wavefront.
+//
+// Same mathematics as snd_fwd_kernel.h (reference: selective_scan_fwd_kernel_oflex.cuh:189-346):
+//     delta' = softplus(delta + bias)          a = exp2(delta' * A * log2e) * A_decay          bu = B * delta' * u
+//     h[i,j] = a*(h[i,j-1] + h[i-1,j] - 0.5*(a[i-1,j] + a[i,j-1])*h[i-1,j-1]) + bu
+//     s[i,j] = a*s[i,j-1] + bu                 out = D*u + sum_n C*(h - s + 0.25*bu)
+// Mapping: a block owns one (batch, channel); wave w of the block owns columns 64w .. 64w+63 of the
+// plane (a row segment per row), lane = column, the channel's states are registers of the lane.
+// Along a row the recurrence is first order, h_j = a_j*h_{j-1} + y_j with
+//     y_j = a_j*(h[i-1,j] - 0.5*(a[i-1,j] + a[i,j-1])*h[i-1,j-1]) + bu_j
+// known from the row above, so a wave resolves its 64 cells of a row with one inclusive scan of the
+// affine maps (a_j, y_j) (and (a_j, bu_j) for s) in six DPP steps, then adds the value entering from
+// the segment on its left: h = Y + A*h[i, 64w-1].  h[i-1,j] and a[i-1,j] are the lane's own registers
+// from the previous row, h[i-1,j-1] and a[i,j-1] come from the lane below (wave_shr:1).
+// The segments of a plane form an anti-diagonal wavefront: in step e wave w works on rows 2(e-w),
+// 2(e-w)+1 and reads what wave w-1 left for those rows in LDS in step e-1 (h, s, a of its last column);
+// one block barrier per step, no polling.  Global loads are whole rows of 64 consecutive elements per
+// wave (one or two full memory lines per instruction), issued a band of rows ahead; nothing is staged
+// through LDS.  Saved for the backward: h, a on the last row of every band of R rows (x_v) and h, s, a
+// entering every segment on every row (x, x_sd), so that the backward can recompute any band of any
+// segment on its own.
+#pragma once
+#include "snd_device.h"
+
+namespace snd {
+
+template <typename T, int NS, bool SAVE>
+__global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
+    constexpr int R = NS <= 2 ? 8 : 4;               // rows per band = rows per load group
+    constexpr int RD = 2;                            // rows per wavefront step
+    static_assert(R % RD == 0, "a band is a whole number of steps");
+    // what a wave leaves for the wave on its right: {h, s, a, -} at its last column, per step parity, row and state
+    __shared__ float4 sHO[2][kMaxSeg][RD][NS];
+
+    const snd_shape &sh = p.shape;
+    const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
+    const int rg = Dm / G, rd = Dm / sh.delta_dim;
+    int pair, chunk;
+    if (!xcd_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;      // all channels of a (batch, group) on one XCD
+    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nseg = wg.nseg;
+    const bool multi = nseg > 1;
+
+    // scan origin of this group: memory row = r0m + rs*i, memory column = c0m + cs*j
+    const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
+    const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
+    const int j = w * kSeg + lane;
+    const bool jin = j < W;
+    const int jc = jin ? j : W - 1;
+    const int mc = fh ? W - 1 - jc : jc;
+
+    float A2[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) A2[n] = n < N ? p.A[(int64_t)c * p.A_d_stride + (int64_t)n * p.A_dstate_stride] * kLog2e : 0.f;
+    const float ld = p.A_decay ? __log2f(p.A_decay[0]) : 0.f;
+    const float Dv = p.D ? p.D[c] : 0.f;
+    const float bias = p.delta_bias ? p.delta_bias[c / rd] : 0.f;
+    const bool softplus = p.delta_softplus != 0;
+
+    constexpr int ESZ = (int)sizeof(T);
+    const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
+    const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
+    const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chunk : c) * p.u_d_stride;
+    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(c / rd) * p.delta_d_stride;
+    const int sh_out = p.out_dtype == SND_F32 ? 2 : 1;
+    void *outb = (char *)p.out + (((int64_t)b * p.out_batch_stride + (int64_t)c * p.out_d_stride) << sh_out);
+    const int UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ, BhB = (int)p.B_h_stride * ESZ,
+              ChB = (int)p.C_h_stride * ESZ, OhB = (int)p.out_h_stride << sh_out;
+    const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
+    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc << sh_out;
+
+    // saved state of this plane set
+    const int64_t plane0 = ((int64_t)b * Dm + c) * N;
+    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j;
+    float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
+    float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
+
+    struct Stage { float u[R], d[R], b[R][NS], c[R][NS]; };
+    auto load_band = [&](Stage &q, int band) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = min(band * R + r, H - 1);                      // always in bounds
+            const int mr = mad24(i, rs, r0m);
+            q.u[r] = jin ? ldg_b(ub, mad24(mr, UhB, colB)) : 0.f;
+            q.d[r] = ldg_b(db, mad24(mr, DhB, colB));
+#pragma unroll
+            for (int n = 0; n < NS; ++n) {
+                const int sn = n < N ? n : 0;
+                const float vb = ldg_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
+                const float vc = ldg_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
+                q.b[r][n] = (jin && n < N) ? vb : 0.f;
+                q.c[r][n] = (jin && n < N) ? vc : 0.f;
+            }
+        }
+    };
+
+    float hprev[NS], aprev[NS], hdiag[NS];          // h, a of the row above at this column; h[i-1, 64w-1]
+    float ch[NS], cs[NS], ca[NS];                   // (SAVE) what entered this segment on row band*R + lane
+#pragma unroll
+    for (int n = 0; n < NS; ++n) { hprev[n] = 0.f; aprev[n] = 0.f; hdiag[n] = 0.f; ch[n] = 0.f; cs[n] = 0.f; ca[n] = 0.f; }
+
+    Stage cur, nxt;
+    load_band(cur, 0);
+    int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
+    if (multi)
+        for (int e = 0; e < w; ++e) __syncthreads(); // the waves on the left go first
+
+    for (int band = 0; band < wg.nBands; ++band) {
+        if (band + 1 < wg.nBands) load_band(nxt, band + 1);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = band * R + r;
+            if (i < H) {
+                const float u = cur.u[r];
+                const float raw = cur.d[r] + bias;
+                float dsp;
+                const float dl = softplus ? softplus20(raw, dsp) : raw;
+                const float du = dl * u;
+                float acc = 0.f;
+#pragma unroll
+                for (int n = 0; n < NS; ++n) {
+                    // what the segment on the left left for this row: h, s, a at column 64w-1
+                    float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (w > 0) in = sHO[(step + 1) & 1][w - 1][r % RD][n];
+                    const float a = fast_exp2(fmaf(dl, A2[n], ld));
+                    const float bu = cur.b[r][n] * du;
+                    const float a_l = from_prev_lane(a, in.z);                 // a[i, j-1]
+                    const float h_d = from_prev_lane(hprev[n], hdiag[n]);      // h[i-1, j-1]
+                    const float X = fmaf(-0.5f * (aprev[n] + a_l), h_d, hprev[n]);
+                    float Y = fmaf(a, X, bu), S = bu, Ap = a;
+                    wave_scan3(Y, S, Ap);
+                    const float h = fmaf(Ap, in.x, Y);
+                    const float s = fmaf(Ap, in.y, S);
+                    acc = fmaf(cur.c[r][n], fmaf(0.25f, bu, h - s), acc);
+                    hdiag[n] = in.x;
+                    hprev[n] = h;
+                    aprev[n] = a;
+                    if (multi && lane == 63 && w + 1 < nseg) sHO[step & 1][w][r % RD][n] = make_float4(h, s, a, 0.f);
+                    if (SAVE && lane == r) { ch[n] = in.x; cs[n] = in.y; ca[n] = in.z; }
+                }
+                if (jin) st_f32_b(outb, mad24(mad24(i, rs, r0m), OhB, colO), p.out_dtype, fmaf(Dv, u, acc));
+            }
+            if (multi && r % RD == RD - 1) { __syncthreads(); ++step; }
+        }
+        // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+            if (n < N) {
+                float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
+                __builtin_nontemporal_store(hprev[n], dst);
+                __builtin_nontemporal_store(aprev[n], dst + wg.Wp);
+            }
+        }
+        // column checkpoints: lanes 0..R-1 hold what entered the segment on the band's rows
+        if (SAVE && w > 0 && lane < R) {
+#pragma unroll
+            for (int n = 0; n < NS; ++n) {
+                if (n < N) {
+                    const int64_t o = (int64_t)n * wave_x_plane(wg) + band * R + lane;
+                    xh[o] = ch[n];
+                    xh[o + wg.Hp] = ca[n];
+                    xs[o] = cs[n];
+                }
+            }
+        }
+        cur = nxt;
+    }
+    if (multi)
+        for (int e = 0; e < nseg - 1 - w; ++e) __syncthreads();
+}
+
+template <typename T, int NS>
+static int launch_wave_fwd_ns(const snd_fwd_params &p, hipStream_t stream) {
+    const snd_shape &sh = p.shape;
+    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
+    const int grid = xcd_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    if (p.x != nullptr)
+        hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
+    else
+        hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
+    return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_wave_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
+    const int N = p.shape.dstate;
+    return N == 1 ? launch_wave_fwd_ns<T, 1>(p, stream) : N == 2 ? launch_wave_fwd_ns<T, 2>(p, stream)
+                                                                  : launch_wave_fwd_ns<T, 4>(p, stream);
+}
+
+}  // namespace snd

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(PKG, "libsnd_scan.so")
 HEADER = os.path.join(ROOT, "include", "snd_scan.h")
 
 SND_F32, SND_F16, SND_BF16 = 0, 1, 2
-SCHED_AUTO, SCHED_PLANE, SCHED_STRIPS, SCHED_BANDS = 0, 1, 2, 3
+SCHED_AUTO, SCHED_PLANE, SCHED_STRIPS, SCHED_BANDS, SCHED_WAVEFRONT = 0, 1, 2, 3, 4
 DIR_TOPLEFT, DIR_CORNERS = 0, 1
 i32, i64, vp = C.c_int32, C.c_int64, C.c_void_p
 

@@ -27,6 +27,8 @@ def draw(seed):
     if not c["softplus"]:
         c["has_bias"] = False                              # delta + (negative) bias must stay positive without softplus
     c["Dd"] = c["Dm"] // 2 if (c["share_delta"] and c["Dm"] % 2 == 0) else c["Dm"]
+    if c["N"] <= 4 and seed % 2 == 1:
+        c["sched"] = capi.SCHED_WAVEFRONT                  # half of the small-state cases name the wavefront kernels (AUTO picks them too)
     return c
 
 
@@ -57,7 +59,7 @@ def test_random_case(gpu_device, seed):
     g = capi.bwd(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, dout, f.x, f.x_v, c["softplus"], dec, f.x_sd,
                  None, c["sched"], c["dirs"])
     torch.cuda.synchronize()
-    strips = c["sched"] in (capi.SCHED_STRIPS, capi.SCHED_BANDS) or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule != capi.SCHED_PLANE)
+    strips = c["sched"] in (capi.SCHED_STRIPS, capi.SCHED_BANDS) or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule in (capi.SCHED_STRIPS, capi.SCHED_BANDS))
     if strips and f.plan.n_chunks_y > 1:                   # a single strip always runs as a whole plane
         assert int(f.ws.view(torch.int32)[1]) == 0         # no strip wait gave up
 

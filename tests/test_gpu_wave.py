@@ -1,0 +1,147 @@
+"""The row-segment wavefront kernels (1-4 states per channel, planes up to 512 columns wide) against the
+float64 oracle and against the tile kernels on the same inputs, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import capi
+from oracle import snd_oracle as O
+from oracle import snd_oracle_c as OC
+from test_gpu_fwd import relerr
+
+pytestmark = pytest.mark.gpu
+NAMES = ["du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias", "dA_decay"]
+
+SHAPES = [
+    # Bt, Dm, H, W, N, K, Dd, dtype
+    (1, 8, 9, 10, 1, 2, None, torch.float32),        # one segment, partly filled
+    (2, 8, 16, 64, 1, 4, None, torch.float32),       # exactly one full segment, two full bands
+    (1, 4, 17, 65, 1, 1, None, torch.float32),       # second segment holds one column; ragged last band
+    (1, 4, 1, 200, 2, 2, None, torch.float32),       # single row: 1D scan across four segments
+    (1, 4, 33, 1, 2, 1, None, torch.float32),        # single column
+    (1, 8, 30, 130, 2, 4, 4, torch.float32),         # three segments, shared delta groups
+    (2, 6, 21, 100, 3, 2, None, torch.float32),      # three states run on the four-state kernels
+    (1, 8, 13, 150, 4, 2, None, torch.float32),      # four states: bands of four rows
+    (1, 8, 40, 512, 1, 4, None, torch.float32),      # the widest plane: eight segments
+    (1, 8, 64, 512, 1, 4, None, torch.bfloat16),
+    (3, 12, 14, 14, 4, 4, None, torch.bfloat16),
+    (1, 4, 25, 90, 2, 2, None, torch.float16),
+    (2, 48, 56, 56, 1, 4, None, torch.float32),      # stage-1 plane, d_state = 1
+]
+
+
+def run(dev, Bt, Dm, H, W, N, K, Dd, dtype, sched, dirs=capi.DIR_TOPLEFT, softplus=True, decay=None, seed=3,
+        use_D=True, use_bias=True, out_float=True):
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=seed, Dd=Dd)
+    t = {k: torch.from_numpy(v).to(dev) for k, v in d.items()}
+    for k in ("u", "delta", "B", "C"):
+        t[k] = t[k].to(dtype)
+    if not softplus:                                  # a raw delta must be positive: pass the discretised step itself
+        t["delta"] = torch.nn.functional.softplus(t["delta"].float() + t["delta_bias"].view(1, -1, 1, 1).repeat_interleave(Dm // t["delta"].shape[1], 1)[:, :t["delta"].shape[1]]).to(dtype)
+        d["delta"] = t["delta"].float().cpu().numpy()
+        use_bias = False
+    D = t["D"] if use_D else None
+    bias = t["delta_bias"] if use_bias else None
+    dec = torch.tensor([decay], device=dev) if decay is not None else None
+    args = (t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias)
+    f = capi.FwdCall(*args, softplus, out_float, dec, True, sched, dirs)
+    f.launch()
+    b = capi.BwdCall(*args, t["dout"], f.x, f.x_v, softplus, dec, f.x_sd, sched, dirs)
+    b.launch()
+    torch.cuda.synchronize()
+    return d, t, f, b
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,Dd,dtype", SHAPES)
+def test_wavefront_matches_oracle_and_tiles(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype):
+    print("wavefront", Bt, Dm, H, W, N, K, Dd, dtype, flush=True)
+    d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_WAVEFRONT)
+    assert f.plan.auto_schedule == capi.SCHED_WAVEFRONT and f.plan.auto_bwd_jobs == 0
+    r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    o = (r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"])
+    ref = OC.fwd(*o, True, None, real="f64")
+    gref = OC.bwd(*o, d["dout"], True, None, real="f64")
+    assert relerr(f.out.cpu().numpy(), ref) <= 1e-4
+    half = dtype != torch.float32
+    Dmm = Dm
+    got = [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias]
+    if Dd is not None:                                # the C ABI returns ddelta / ddelta_bias per channel
+        got[1] = got[1].float().view(Bt, Dd, Dmm // Dd, H, W).sum(2)
+        got[6] = got[6].view(Dd, Dmm // Dd).sum(1)
+    for nm, a, w_ in zip(NAMES, got, gref):
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
+        e = relerr(a.float().cpu().numpy(), w_)
+        assert e <= tol, (nm, e)
+    # the tile kernels on the same inputs (their own saved state)
+    _, _, f2, b2 = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_PLANE)
+    assert relerr(f.out.cpu().numpy(), f2.out.cpu().numpy()) <= 1e-5
+    got2 = [b2.du, b2.ddelta, b2.dA, b2.dB, b2.dC, b2.dD, b2.dbias]
+    if Dd is not None:
+        got2[1] = got2[1].float().view(Bt, Dd, Dmm // Dd, H, W).sum(2)
+        got2[6] = got2[6].view(Dd, Dmm // Dd).sum(1)
+    for nm, a, w_, r_ in zip(NAMES, got, got2, gref):
+        # difference of the two kernel families on the scale of the true gradient (a single row makes dA
+        # identically zero: both families then return rounding noise of different sizes)
+        tol = 1e-2 if (half and nm in ("du", "ddelta")) else 1e-4
+        scale = max(float(np.abs(r_).max()), 1e-2 if float(np.abs(r_).max()) < 1e-12 else 0.0)
+        e = float(np.abs(a.float().cpu().numpy().astype(np.float64) - w_.float().cpu().numpy()).max()) / scale
+        assert e <= tol, (nm, e)
+
+
+@pytest.mark.parametrize("kw", [dict(softplus=False), dict(use_D=False, use_bias=False), dict(decay=0.9),
+                                dict(dirs=capi.DIR_CORNERS), dict(out_float=False)])
+def test_wavefront_options(gpu_device, kw):
+    print("wavefront options", kw, flush=True)
+    Bt, Dm, H, W, N, K = 2, 8, 19, 150, 2, 4
+    dtype = torch.bfloat16 if kw.get("out_float") is False else torch.float32
+    d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, None, dtype, capi.SCHED_WAVEFRONT, **kw)
+    _, _, f2, b2 = run(gpu_device, Bt, Dm, H, W, N, K, None, dtype, capi.SCHED_PLANE, **kw)
+    half = dtype != torch.float32
+    assert f.out.dtype == (torch.float32 if kw.get("out_float", True) else dtype)
+    assert relerr(f.out.float().cpu().numpy(), f2.out.float().cpu().numpy()) <= (1e-2 if half else 1e-5)
+    pairs = zip(NAMES, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias, b.ddec], [b2.du, b2.ddelta, b2.dA, b2.dB, b2.dC, b2.dD, b2.dbias, b2.ddec])
+    for nm, a, w_ in pairs:
+        assert (a is None) == (w_ is None), nm
+        if a is None:
+            continue
+        tol = 1e-2 if (half and nm in ("du", "ddelta")) else (5e-4 if nm == "dA_decay" else 1e-4)
+        assert relerr(a.float().cpu().numpy(), w_.float().cpu().numpy()) <= tol, (nm, relerr(a.float().cpu().numpy(), w_.float().cpu().numpy()))
+    if "dirs" not in kw and "decay" not in kw and dtype == torch.float32:
+        # and the oracle, for the options it takes directly
+        D = d["D"] if kw.get("use_D", True) else None
+        bias = d["delta_bias"] if (kw.get("use_bias", True) and kw.get("softplus", True)) else None
+        ref = OC.fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], D, bias, kw.get("softplus", True), None, real="f64")
+        assert relerr(f.out.cpu().numpy(), ref) <= 1e-4
+
+
+def test_wavefront_shared_u_and_second_backward(gpu_device):
+    """u with dim / n_groups channels shared by the four corner groups; the saved state is read-only."""
+    Bt, Cc_, H, W, N, K = 2, 6, 20, 70, 1, 4
+    d = O.make_inputs(Bt, K * Cc_, H, W, N=N, K=K, seed=8)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    u1 = t["u"][:, :Cc_].contiguous()
+    args = (u1, t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+    res = {}
+    for sched in (capi.SCHED_WAVEFRONT, capi.SCHED_PLANE):
+        f = capi.FwdCall(*args, True, True, None, True, sched, capi.DIR_CORNERS)
+        f.launch()
+        g1 = capi.bwd(*args, t["dout"], f.x, f.x_v, True, None, f.x_sd, schedule=sched, directions=capi.DIR_CORNERS)
+        g2 = capi.bwd(*args, t["dout"], f.x, f.x_v, True, None, f.x_sd, schedule=sched, directions=capi.DIR_CORNERS)
+        torch.cuda.synchronize()
+        for a, b_ in zip(g1, g2):
+            if a is not None:
+                assert relerr(b_.cpu().numpy(), a.cpu().numpy()) <= 1e-6
+        res[sched] = (f.out, g1)
+    assert res[capi.SCHED_WAVEFRONT][1][0].shape == u1.shape
+    assert relerr(res[capi.SCHED_WAVEFRONT][0].cpu().numpy(), res[capi.SCHED_PLANE][0].cpu().numpy()) <= 1e-5
+    for a, b_ in zip(res[capi.SCHED_WAVEFRONT][1], res[capi.SCHED_PLANE][1]):
+        if a is not None:
+            assert relerr(a.cpu().numpy(), b_.cpu().numpy()) <= 1e-4
+
+
+def test_wavefront_refuses_what_it_does_not_cover(gpu_device):
+    d = O.make_inputs(1, 4, 8, 600, N=1, K=1, seed=1)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], None, None, False, True, None, True, capi.SCHED_WAVEFRONT)
+    assert f.plan.auto_schedule != capi.SCHED_WAVEFRONT
+    assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -2
