@@ -410,6 +410,39 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
 
+// Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all
+// channels of a pair share an XCD (and its L2 copy of the pair's B / C planes) as in xcd_job; with few pairs
+// that would leave XCDs idle, so the channels are dealt over all of them (B / C of few pairs are small).
+__device__ __forceinline__ bool wave_job(int bid, int nPairs, int rg, int &pair, int &chunk) {
+    if (nPairs >= 16 || (nPairs & 7) == 0) return xcd_job(bid, nPairs, rg, pair, chunk);
+    pair = bid / rg;
+    chunk = bid - pair * rg;
+    return pair < nPairs;
+}
+__host__ inline int wave_grid(int nPairs, int rg) { return (nPairs >= 16 || (nPairs & 7) == 0) ? xcd_grid(nPairs, rg) : nPairs * rg; }
+// Row inputs of the wavefront kernels wait in registers as raw bits for a band of rows and are converted
+// where they are used (a conversion at the load would put the wait for the load there).  They are loaded
+// without any lane condition: a load whose result is only needed under a lane condition is sunk into that
+// condition by the compiler - a branch with a full wait behind every load.
+__device__ __forceinline__ uint32_t ldraw_b(const float *base, uint32_t off) { uint32_t v = *(const uint32_t *)((const char *)base + off); return v; }
+__device__ __forceinline__ uint32_t ldraw_b(const bf16_t *base, uint32_t off) { uint32_t v = *(const uint16_t *)((const char *)base + off); return v; }
+__device__ __forceinline__ uint32_t ldraw_b(const f16_t *base, uint32_t off) { uint32_t v = *(const uint16_t *)((const char *)base + off); return v; }
+__device__ __forceinline__ uint32_t ldraw_dt(const void *base, uint32_t off, int dt) {
+    return dt == SND_F32 ? *(const uint32_t *)((const char *)base + off) : (uint32_t) * (const uint16_t *)((const char *)base + off);
+}
+__device__ __forceinline__ float cvt_raw(const float *, uint32_t r) { return __builtin_bit_cast(float, r); }
+__device__ __forceinline__ float cvt_raw(const bf16_t *, uint32_t r) { return __builtin_bit_cast(float, r << 16); }
+__device__ __forceinline__ float cvt_raw(const f16_t *, uint32_t r) { return (float)__builtin_bit_cast(f16_t, (uint16_t)r); }
+__device__ __forceinline__ float cvt_raw_dt(uint32_t r, int dt) {
+    if (dt == SND_F32) return __builtin_bit_cast(float, r);
+    if (dt == SND_BF16) return __builtin_bit_cast(float, r << 16);
+    return (float)__builtin_bit_cast(f16_t, (uint16_t)r);
+}
+// Block barrier for hand-overs through LDS only: waits for this wave's LDS traffic, not for its global loads
+// and stores (the prefetched rows and the row just written stay in flight across it; __syncthreads would
+// drain them at every step).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_old(float old, float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
 }

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     int pair, chunk;
-    if (!xcd_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
+    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nseg = wg.nseg;
@@ -99,22 +99,23 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     // inputs of one band: rows in mirrored lane order; the row above the band (h0, a0) in natural order;
     // what entered the segment from the left on rows i0-1 .. i0+R-1, one row per lane (ch, cs, ca)
-    struct In { float u[R], d[R], o[R], b[R][NS], c[R][NS], h0[NS], a0[NS], ch[NS], cs[NS], ca[NS]; };
+    // Row inputs wait as raw bits.  Lanes beyond the last column read the last column (always in bounds); only
+    // their dout is masked to zero where it is used, which makes every adjoint there exactly zero.
+    struct In { uint32_t u[R], d[R], o[R], b[R][NS], c[R][NS]; float h0[NS], a0[NS], ch[NS], cs[NS], ca[NS]; };
+    const T *const tp = nullptr;                     // selects the conversion
     auto load_band = [&](In &q, int band) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int i = min(band * R + r, H - 1);                      // always in bounds
             const int mr = mad24(i, rs, r0m);
-            q.u[r] = jin ? ldg_b(ub, mad24(mr, UhB, colB)) : 0.f;
-            q.d[r] = ldg_b(db, mad24(mr, DhB, colB));
-            q.o[r] = jin ? ld_f32_b(dob, mad24(mr, DohB, colO), p.dout_dtype) : 0.f;
+            q.u[r] = ldraw_b(ub, mad24(mr, UhB, colB));
+            q.d[r] = ldraw_b(db, mad24(mr, DhB, colB));
+            q.o[r] = ldraw_dt(dob, mad24(mr, DohB, colO), p.dout_dtype);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 const int sn = n < N ? n : 0;
-                const float vb = ldg_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
-                const float vc = ldg_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
-                q.b[r][n] = (jin && n < N) ? vb : 0.f;
-                q.c[r][n] = (jin && n < N) ? vc : 0.f;
+                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
+                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
             }
         }
         const int row = band * R - 1 + lane;
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     load_band(cur, wg.nBands - 1);
     int step = nseg - 1 - w;                         // the waves on the right go first
     if (multi)
-        for (int e = 0; e < nseg - 1 - w; ++e) __syncthreads();
+        for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
 
     for (int band = wg.nBands - 1; band >= 0; --band) {
         if (band > 0) load_band(nxt, band - 1);
@@ -165,17 +166,17 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const float raw = cur.d[r] + bias;
+                const float raw = cvt_raw(tp, cur.d[r]) + bias;
                 float sg = 1.f;
                 dl[r] = softplus ? softplus20(raw, sg) : raw;
                 dsp[r] = sg;
                 if (band * R + r < H) {
-                    const float dl_n = mirror(dl[r]), dlu_n = mirror(dl[r] * cur.u[r]);
+                    const float dl_n = mirror(dl[r]), dlu_n = mirror(dl[r] * cvt_raw(tp, cur.u[r]));
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
                         const float hin = bcast(cur.ch[n], r + 1), sin_ = bcast(cur.cs[n], r + 1), ain = bcast(cur.ca[n], r + 1);
                         const float a = fast_exp2(fmaf(dl_n, A2[n], ld));
-                        const float bu = mirror(cur.b[r][n]) * dlu_n;
+                        const float bu = (n < N ? mirror(cvt_raw(tp, cur.b[r][n])) : 0.f) * dlu_n;
                         const float a_l = from_prev_lane(a, ain);              // a[i, j-1]
                         const float h_d = from_prev_lane(hp[n], hdiag[n]);     // h[i-1, j-1]
                         const float X = fmaf(-0.5f * (ap[n] + a_l), h_d, hp[n]);
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         for (int r = R - 1; r >= 0; --r) {
             const int i = band * R + r;
             if (i < H) {
-                const float dov = cur.o[r], uv = cur.u[r], dlv = dl[r];
+                const float dov = jin ? cvt_raw_dt(cur.o[r], p.dout_dtype) : 0.f, uv = cvt_raw(tp, cur.u[r]), dlv = dl[r];
                 const float dlu = dlv * uv;
                 const int mr = mad24(i, rs, r0m);
                 float qsum = 0.f, psum = 0.f;
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                     float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
                     if (w + 1 < nseg) in = sHO[(step + 1) & 1][w + 1][r][n];
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, 64w-1]
-                    const float Bv = cur.b[r][n], Cv = cur.c[r][n];
+                    const float Bv = n < N ? cvt_raw(tp, cur.b[r][n]) : 0.f, Cv = n < N ? cvt_raw(tp, cur.c[r][n]) : 0.f;
                     const float a = fast_exp2(fmaf(dlv, A2[n], ld));
                     const float bu = Bv * dlu;
                     const float dyC = dov * Cv;
@@ -255,11 +256,11 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                 }
             }
         }
-        if (multi) { __syncthreads(); ++step; }
+        if (multi) { lds_barrier(); ++step; }
         cur = nxt;
     }
     if (multi)
-        for (int e = 0; e < w; ++e) __syncthreads();
+        for (int e = 0; e < w; ++e) lds_barrier();
 
     // ---- per-channel sums leave the kernel: one atomic per wave and value
 #pragma unroll
@@ -284,7 +285,7 @@ template <typename T, int NS>
 static int launch_wave_bwd_ns(const snd_bwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
-    const int grid = xcd_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    const int grid = wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
     hipLaunchKernelGGL((wave_bwd_kernel<T, NS>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     int pair, chunk;
-    if (!xcd_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;      // all channels of a (batch, group) on one XCD
+    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;      // all channels of a (batch, group) on one XCD
     const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nseg = wg.nseg;
@@ -77,21 +77,22 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
     float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
 
-    struct Stage { float u[R], d[R], b[R][NS], c[R][NS]; };
+    // Raw bits of a band's rows.  Lanes beyond the last column read the last column (always in bounds): what they
+    // compute only feeds cells further right and is never stored.
+    struct Stage { uint32_t u[R], d[R], b[R][NS], c[R][NS]; };
+    const T *const tp = nullptr;                     // selects the conversion
     auto load_band = [&](Stage &q, int band) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int i = min(band * R + r, H - 1);                      // always in bounds
             const int mr = mad24(i, rs, r0m);
-            q.u[r] = jin ? ldg_b(ub, mad24(mr, UhB, colB)) : 0.f;
-            q.d[r] = ldg_b(db, mad24(mr, DhB, colB));
+            q.u[r] = ldraw_b(ub, mad24(mr, UhB, colB));
+            q.d[r] = ldraw_b(db, mad24(mr, DhB, colB));
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 const int sn = n < N ? n : 0;
-                const float vb = ldg_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
-                const float vc = ldg_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
-                q.b[r][n] = (jin && n < N) ? vb : 0.f;
-                q.c[r][n] = (jin && n < N) ? vc : 0.f;
+                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
+                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
             }
         }
     };
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     load_band(cur, 0);
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     if (multi)
-        for (int e = 0; e < w; ++e) __syncthreads(); // the waves on the left go first
+        for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
 
     for (int band = 0; band < wg.nBands; ++band) {
         if (band + 1 < wg.nBands) load_band(nxt, band + 1);
@@ -113,8 +114,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         for (int r = 0; r < R; ++r) {
             const int i = band * R + r;
             if (i < H) {
-                const float u = cur.u[r];
-                const float raw = cur.d[r] + bias;
+                const float u = cvt_raw(tp, cur.u[r]);
+                const float raw = cvt_raw(tp, cur.d[r]) + bias;
                 float dsp;
                 const float dl = softplus ? softplus20(raw, dsp) : raw;
                 const float du = dl * u;
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                     float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
                     if (w > 0) in = sHO[(step + 1) & 1][w - 1][r % RD][n];
                     const float a = fast_exp2(fmaf(dl, A2[n], ld));
-                    const float bu = cur.b[r][n] * du;
+                    const float bu = (n < N ? cvt_raw(tp, cur.b[r][n]) : 0.f) * du;
                     const float a_l = from_prev_lane(a, in.z);                 // a[i, j-1]
                     const float h_d = from_prev_lane(hprev[n], hdiag[n]);      // h[i-1, j-1]
                     const float X = fmaf(-0.5f * (aprev[n] + a_l), h_d, hprev[n]);
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                     wave_scan3(Y, S, Ap);
                     const float h = fmaf(Ap, in.x, Y);
                     const float s = fmaf(Ap, in.y, S);
-                    acc = fmaf(cur.c[r][n], fmaf(0.25f, bu, h - s), acc);
+                    acc = fmaf(cvt_raw(tp, cur.c[r][n]), fmaf(0.25f, bu, h - s), acc);
                     hdiag[n] = in.x;
                     hprev[n] = h;
                     aprev[n] = a;
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                 }
                 if (jin) st_f32_b(outb, mad24(mad24(i, rs, r0m), OhB, colO), p.out_dtype, fmaf(Dv, u, acc));
             }
-            if (multi && r % RD == RD - 1) { __syncthreads(); ++step; }
+            if (multi && r % RD == RD - 1) { lds_barrier(); ++step; }
         }
         // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
 #pragma unroll
@@ -168,14 +169,14 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         cur = nxt;
     }
     if (multi)
-        for (int e = 0; e < nseg - 1 - w; ++e) __syncthreads();
+        for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
 }
 
 template <typename T, int NS>
 static int launch_wave_fwd_ns(const snd_fwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
-    const int grid = xcd_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    const int grid = wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
     if (p.x != nullptr)
         hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
     else
