@@ -397,7 +397,7 @@ __host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 &
 __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     WaveGeo g;
     g.nseg = (W + kSeg - 1) / kSeg;
-    g.R = N <= 2 ? 8 : 4;
+    g.R = N <= 1 ? 8 : 4;             // (the backward keeps a band's h, s, a and inputs of every state in registers)
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
     g.Wp = g.nseg * kSeg;

@@ -23,6 +23,7 @@
 // LDS (one block barrier per band, no polling).  dB, dC leave as one global atomic per element and channel
 // (a wave-wide instruction covers 256 consecutive bytes), du / ddelta as whole row segments.
 #pragma once
+#include <type_traits>
 #include "snd_device.h"
 
 namespace snd {
@@ -31,11 +32,13 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename T, int NS>
+template <typename T, int NS, bool DO32>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
-    constexpr int R = NS <= 2 ? 8 : 4;               // rows per band
-    // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and state
-    __shared__ float4 sHO[2][kMaxSeg][R][NS];
+    constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
+    constexpr bool PF = NS <= 2;                     // load a band's inputs one band ahead (with four states the registers are needed elsewhere)
+    // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and
+    // state.  Wave w writes slot w and reads slot w+1; the slot after the last wave stays zero.
+    __shared__ float4 sHO[2][kMaxSeg + 1][R][NS];
 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
@@ -47,6 +50,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nseg = wg.nseg;
     const bool multi = nseg > 1;
+    if (threadIdx.x < 2 * R * NS) (&sHO[0][0][0][0])[((threadIdx.x / (R * NS)) * (kMaxSeg + 1) + nseg) * R * NS + threadIdx.x % (R * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
@@ -76,20 +80,22 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const bool want_decay = p.dA_decay != nullptr;
 
     constexpr int ESZ = (int)sizeof(T);
+    using DoT = typename std::conditional<DO32, float, T>::type;
+    constexpr int DSZ = (int)sizeof(DoT);
     const T *Bb = (const T *)f.B + (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
     const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
     const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chunk : c) * f.u_d_stride;
     const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(c / rd) * f.delta_d_stride;
-    const int sh_do = p.dout_dtype == SND_F32 ? 2 : 1;
-    const void *dob = (const char *)p.dout + (((int64_t)b * p.dout_batch_stride + (int64_t)c * p.dout_d_stride) << sh_do);
+    const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)c * p.dout_d_stride;
     T *dub = (T *)p.du + ((int64_t)b * Dm + c) * H * W;                 // du, ddelta: dense [b, c, H, W]
     T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + c) * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;               // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
-    const int UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ, BhB = (int)f.B_h_stride * ESZ,
-              ChB = (int)f.C_h_stride * ESZ, DohB = (int)p.dout_h_stride << sh_do, WB = W * ESZ, W4 = W * 4;
+    // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
+    const int UhB = (int)f.u_h_stride * ESZ * rs, DhB = (int)f.delta_h_stride * ESZ * rs, BhB = (int)f.B_h_stride * ESZ * rs,
+              ChB = (int)f.C_h_stride * ESZ * rs, DohB = (int)p.dout_h_stride * DSZ * rs, WB = W * ESZ * rs, W4 = W * 4 * rs;
     const int64_t BsB = f.B_dstate_stride * ESZ, CsB = f.C_dstate_stride * ESZ, HW4 = (int64_t)H * W * 4;
-    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc << sh_do, col4 = (uint32_t)mc * 4;
+    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc * DSZ, col4 = (uint32_t)mc * 4;
 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
@@ -97,32 +103,39 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
     const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
 
-    // inputs of one band: rows in mirrored lane order; the row above the band (h0, a0) in natural order;
-    // what entered the segment from the left on rows i0-1 .. i0+R-1, one row per lane (ch, cs, ca)
-    // Row inputs wait as raw bits.  Lanes beyond the last column read the last column (always in bounds); only
-    // their dout is masked to zero where it is used, which makes every adjoint there exactly zero.
+    // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
+    // last column (always in bounds) and only their dout is masked to zero where it is used, which makes every
+    // adjoint there exactly zero.  h0, a0: the row above the band in natural order.  ch, cs, ca: what entered
+    // the segment from the left on rows i0-1 .. i0+R-1, one row per lane.
     struct In { uint32_t u[R], d[R], o[R], b[R][NS], c[R][NS]; float h0[NS], a0[NS], ch[NS], cs[NS], ca[NS]; };
-    const T *const tp = nullptr;                     // selects the conversion
+    const T *const tp = nullptr;                     // selects the conversions
+    const DoT *const dp = nullptr;
+    // Every band issues the same loads on every path (the wait counters the compiler derives for the prefetch
+    // need that): rows past the end of a ragged last band read the last row again and are never used.
     auto load_band = [&](In &q, int band) {
+        const int i0 = band * R;
+        const int m0 = mad24(i0, rs, r0m);           // memory row of the band's first scan row
+        uint32_t ou = mad24(m0, UhB * rs, colB), od = mad24(m0, DhB * rs, colB), oo = mad24(m0, DohB * rs, colO),
+                 ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int i = min(band * R + r, H - 1);                      // always in bounds
-            const int mr = mad24(i, rs, r0m);
-            q.u[r] = ldraw_b(ub, mad24(mr, UhB, colB));
-            q.d[r] = ldraw_b(db, mad24(mr, DhB, colB));
-            q.o[r] = ldraw_dt(dob, mad24(mr, DohB, colO), p.dout_dtype);
+            q.u[r] = ldraw_b(ub, ou);
+            q.d[r] = ldraw_b(db, od);
+            q.o[r] = ldraw_b(dob, oo);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                const int sn = n < N ? n : 0;
-                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
-                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
+                const int sn = (NS == 4 && n >= N) ? 0 : n;
+                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), ob);
+                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), oc);
             }
+            const bool more = i0 + r + 1 < H;
+            ou += more ? UhB : 0; od += more ? DhB : 0; oo += more ? DohB : 0; ob += more ? BhB : 0; oc += more ? ChB : 0;
         }
-        const int row = band * R - 1 + lane;
+        const int row = i0 - 1 + lane;
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
             q.h0[n] = 0.f; q.a0[n] = 0.f; q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
-            if (n < N) {
+            if (NS != 4 || n < N) {
                 if (band > 0) {
                     const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
                     q.h0[n] = __builtin_nontemporal_load(src);
@@ -143,18 +156,17 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     float dec_acc = 0.f, dD_acc = 0.f, dbias_acc = 0.f;
 #pragma unroll
     for (int n = 0; n < NS; ++n) { Gd[n] = 0.f; ad[n] = 0.f; GdEdge[n] = 0.f; dA_acc[n] = 0.f; }
-
-    In cur, nxt;
-    load_band(cur, wg.nBands - 1);
     int step = nseg - 1 - w;                         // the waves on the right go first
-    if (multi)
-        for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
+    const bool hands_over = multi && w > 0;
 
-    for (int band = wg.nBands - 1; band >= 0; --band) {
-        if (band > 0) load_band(nxt, band - 1);
+    // one band from `cur`, with the loads of the band above issued into `nxt` first
+    auto do_band = [&](In &cur, In &nxt, int band) {
+        if (PF) { if (band > 0) load_band(nxt, band - 1); }
+        else load_band(cur, band);
+        const int i0 = band * R;
 
-        // ---- recompute h, s on the band's rows (with the columns), results back in mirrored order
-        float hT[R][NS], sT[R][NS], dl[R], dsp[R], hTop[NS];
+        // ---- recompute h, s on the band's rows (with the columns); results back in mirrored order
+        float hT[R][NS], sT[R][NS], aT[R][NS], dl[R], dsp[R], hTop[NS];
         {
             float hp[NS], ap[NS], hdiag[NS];
 #pragma unroll
@@ -166,17 +178,19 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const float raw = cvt_raw(tp, cur.d[r]) + bias;
-                float sg = 1.f;
-                dl[r] = softplus ? softplus20(raw, sg) : raw;
-                dsp[r] = sg;
-                if (band * R + r < H) {
+                dl[r] = 0.f;
+                dsp[r] = 0.f;
+                if (i0 + r < H) {
+                    const float raw = cvt_raw(tp, cur.d[r]) + bias;
+                    float sg = 1.f;
+                    dl[r] = softplus ? softplus20(raw, sg) : raw;
+                    dsp[r] = sg;
                     const float dl_n = mirror(dl[r]), dlu_n = mirror(dl[r] * cvt_raw(tp, cur.u[r]));
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
                         const float hin = bcast(cur.ch[n], r + 1), sin_ = bcast(cur.cs[n], r + 1), ain = bcast(cur.ca[n], r + 1);
                         const float a = fast_exp2(fmaf(dl_n, A2[n], ld));
-                        const float bu = (n < N ? mirror(cvt_raw(tp, cur.b[r][n])) : 0.f) * dlu_n;
+                        const float bu = ((NS == 4 && n >= N) ? 0.f : mirror(cvt_raw(tp, cur.b[r][n]))) * dlu_n;
                         const float a_l = from_prev_lane(a, ain);              // a[i, j-1]
                         const float h_d = from_prev_lane(hp[n], hdiag[n]);     // h[i-1, j-1]
                         const float X = fmaf(-0.5f * (ap[n] + a_l), h_d, hp[n]);
@@ -186,34 +200,36 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         const float s = fmaf(Ap, sin_, S);
                         hT[r][n] = mirror(h);
                         sT[r][n] = mirror(s);
+                        aT[r][n] = mirror(a);
                         hp[n] = h;
                         ap[n] = a;
                         hdiag[n] = hin;
                     }
                 } else {
 #pragma unroll
-                    for (int n = 0; n < NS; ++n) { hT[r][n] = 0.f; sT[r][n] = 0.f; }
+                    for (int n = 0; n < NS; ++n) { hT[r][n] = 0.f; sT[r][n] = 0.f; aT[r][n] = 0.f; }
                 }
             }
         }
 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns)
+        const int rows = min(R, H - i0);             // rows of this band inside the plane
+        const int mlast = mad24(i0 + rows - 1, rs, r0m);
+        uint32_t og = mad24(mlast, WB * rs, colB), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
 #pragma unroll
         for (int r = R - 1; r >= 0; --r) {
-            const int i = band * R + r;
-            if (i < H) {
-                const float dov = jin ? cvt_raw_dt(cur.o[r], p.dout_dtype) : 0.f, uv = cvt_raw(tp, cur.u[r]), dlv = dl[r];
+            if (i0 + r < H) {
+                const float dov = jin ? cvt_raw(dp, cur.o[r]) : 0.f, uv = cvt_raw(tp, cur.u[r]), dlv = dl[r];
                 const float dlu = dlv * uv;
-                const int mr = mad24(i, rs, r0m);
                 float qsum = 0.f, psum = 0.f;
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column 64(w+1)
-                    float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (w + 1 < nseg) in = sHO[(step + 1) & 1][w + 1][r][n];
+                    const float4 in = sHO[(step + 1) & 1][w + 1][r][n];
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, 64w-1]
-                    const float Bv = n < N ? cvt_raw(tp, cur.b[r][n]) : 0.f, Cv = n < N ? cvt_raw(tp, cur.c[r][n]) : 0.f;
-                    const float a = fast_exp2(fmaf(dlv, A2[n], ld));
+                    const bool live = NS != 4 || n < N;
+                    const float Bv = live ? cvt_raw(tp, cur.b[r][n]) : 0.f, Cv = live ? cvt_raw(tp, cur.c[r][n]) : 0.f;
+                    const float a = aT[r][n];
                     const float bu = Bv * dlu;
                     const float dyC = dov * Cv;
                     const float a_r = from_prev_lane(a, in.z);                 // a[i, j+1]
@@ -235,29 +251,43 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                     if (want_decay) dec_acc += da;
                     qsum = fmaf(dbu, Bv, qsum);
                     psum = fmaf(Av[n], da, psum);
-                    if (jin && n < N) {
-                        const int64_t o = (int64_t)n * HW4 + (uint32_t)mad24(mr, W4, col4);
-                        wave_glb_add((float *)((char *)dBg + o), dbu * dlu);
-                        wave_glb_add((float *)((char *)dCg + o), dov * fmaf(0.25f, bu, hs));
+                    if (jin && live) {
+                        wave_glb_add((float *)((char *)dBg + n * HW4 + o4), dbu * dlu);
+                        wave_glb_add((float *)((char *)dCg + n * HW4 + o4), dov * fmaf(0.25f, bu, hs));
                     }
                     GdEdge[n] = in.x;
                     Gd[n] = Gt;
                     ad[n] = a;
-                    if (multi && lane == 63 && w > 0) sHO[step & 1][w][r][n] = make_float4(Gt, Gst, a, 0.f);
+                    if (hands_over && lane == 63) sHO[step & 1][w][r][n] = make_float4(Gt, Gst, a, 0.f);
                 }
                 const float duv = fmaf(Dv, dov, dlv * qsum);
                 const float ddl = fmaf(uv, qsum, psum) * dsp[r];
                 if (jin) {
                     dD_acc = fmaf(dov, uv, dD_acc);
                     dbias_acc += ddl;
-                    const uint32_t o = mad24(mr, WB, colB);
-                    stg_b(dub, o, duv);
-                    stg_b(ddb, o, ddl);
+                    stg_b(dub, og, duv);
+                    stg_b(ddb, og, ddl);
                 }
+                og -= WB;
+                o4 -= W4;
             }
         }
         if (multi) { lds_barrier(); ++step; }
-        cur = nxt;
+    };
+
+    In sA;
+    if (PF) load_band(sA, wg.nBands - 1);
+    lds_barrier();                                   // the zeroed slot
+    if (multi)
+        for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
+    if (PF) {
+        In sB;
+        for (int band = wg.nBands - 1; band >= 0; band -= 2) {
+            do_band(sA, sB, band);
+            if (band > 0) do_band(sB, sA, band - 1);
+        }
+    } else {
+        for (int band = wg.nBands - 1; band >= 0; --band) do_band(sA, sA, band);
     }
     if (multi)
         for (int e = 0; e < w; ++e) lds_barrier();
@@ -285,8 +315,9 @@ template <typename T, int NS>
 static int launch_wave_bwd_ns(const snd_bwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
-    const int grid = wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
-    hipLaunchKernelGGL((wave_bwd_kernel<T, NS>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
+    const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
+    if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, true>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 

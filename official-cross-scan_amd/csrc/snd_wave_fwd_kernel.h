@@ -21,27 +21,36 @@
 // entering every segment on every row (x, x_sd), so that the backward can recompute any band of any
 // segment on its own.
 #pragma once
+#include <type_traits>
 #include "snd_device.h"
+
+// Timing studies only (-DSND_WAVE_ABLATE=<bits>, results wrong): 1 no out stores, 2 no block barriers,
+// 4 no softplus, 8 no scan, 16 no checkpoint stores, 32 no hand-over through LDS.
+#ifndef SND_WAVE_ABLATE
+#define SND_WAVE_ABLATE 0
+#endif
 
 namespace snd {
 
-template <typename T, int NS, bool SAVE>
+template <typename T, int NS, bool SAVE, bool OUT32>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
-    constexpr int R = NS <= 2 ? 8 : 4;               // rows per band = rows per load group
+    constexpr int R = NS <= 1 ? 8 : 4;               // rows per band = rows per load group
     constexpr int RD = 2;                            // rows per wavefront step
     static_assert(R % RD == 0, "a band is a whole number of steps");
-    // what a wave leaves for the wave on its right: {h, s, a, -} at its last column, per step parity, row and state
-    __shared__ float4 sHO[2][kMaxSeg][RD][NS];
+    // what a wave leaves for the wave on its right: {h, s, a, -} at its last column, per step parity, row and
+    // state.  Wave w writes slot w+1 and reads slot w; slot 0 stays zero (nothing enters the first segment).
+    __shared__ float4 sHO[2][kMaxSeg + 1][RD][NS];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;      // all channels of a (batch, group) on one XCD
+    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
     const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nseg = wg.nseg;
     const bool multi = nseg > 1;
+    if (threadIdx.x < 2 * RD * NS) (&sHO[0][0][0][0])[(threadIdx.x / (RD * NS)) * (kMaxSeg + 1) * RD * NS + threadIdx.x % (RD * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     // scan origin of this group: memory row = r0m + rs*i, memory column = c0m + cs*j
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
@@ -60,16 +69,18 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     const bool softplus = p.delta_softplus != 0;
 
     constexpr int ESZ = (int)sizeof(T);
+    using OutT = typename std::conditional<OUT32, float, T>::type;
+    constexpr int OSZ = (int)sizeof(OutT);
     const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
     const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chunk : c) * p.u_d_stride;
     const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(c / rd) * p.delta_d_stride;
-    const int sh_out = p.out_dtype == SND_F32 ? 2 : 1;
-    void *outb = (char *)p.out + (((int64_t)b * p.out_batch_stride + (int64_t)c * p.out_d_stride) << sh_out);
-    const int UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ, BhB = (int)p.B_h_stride * ESZ,
-              ChB = (int)p.C_h_stride * ESZ, OhB = (int)p.out_h_stride << sh_out;
+    OutT *outb = (OutT *)p.out + (int64_t)b * p.out_batch_stride + (int64_t)c * p.out_d_stride;
+    // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
+    const int UhB = (int)p.u_h_stride * ESZ * rs, DhB = (int)p.delta_h_stride * ESZ * rs, BhB = (int)p.B_h_stride * ESZ * rs,
+              ChB = (int)p.C_h_stride * ESZ * rs, OhB = (int)p.out_h_stride * OSZ * rs;
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
-    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc << sh_out;
+    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc * OSZ;
 
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
@@ -81,19 +92,25 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     // compute only feeds cells further right and is never stored.
     struct Stage { uint32_t u[R], d[R], b[R][NS], c[R][NS]; };
     const T *const tp = nullptr;                     // selects the conversion
+    // Byte offsets advance by one row step per load (one vector add each).  Every band issues the same loads on
+    // every path - the wait counters the compiler derives for the prefetch need that - so rows past the end of a
+    // ragged last band read the last row again (their step is zero) and are never used.
     auto load_band = [&](Stage &q, int band) {
+        const int i0 = band * R;
+        const int m0 = mad24(i0, rs, r0m);           // memory row of the band's first scan row
+        uint32_t ou = mad24(m0, UhB * rs, colB), od = mad24(m0, DhB * rs, colB), ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int i = min(band * R + r, H - 1);                      // always in bounds
-            const int mr = mad24(i, rs, r0m);
-            q.u[r] = ldraw_b(ub, mad24(mr, UhB, colB));
-            q.d[r] = ldraw_b(db, mad24(mr, DhB, colB));
+            q.u[r] = ldraw_b(ub, ou);
+            q.d[r] = ldraw_b(db, od);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                const int sn = n < N ? n : 0;
-                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), mad24(mr, BhB, colB));
-                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), mad24(mr, ChB, colB));
+                const int sn = (NS == 4 && n >= N) ? 0 : n;
+                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), ob);
+                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), oc);
             }
+            const bool more = i0 + r + 1 < H;
+            ou += more ? UhB : 0; od += more ? DhB : 0; ob += more ? BhB : 0; oc += more ? ChB : 0;
         }
     };
 
@@ -102,63 +119,62 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
     for (int n = 0; n < NS; ++n) { hprev[n] = 0.f; aprev[n] = 0.f; hdiag[n] = 0.f; ch[n] = 0.f; cs[n] = 0.f; ca[n] = 0.f; }
 
-    Stage cur, nxt;
-    load_band(cur, 0);
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
-    if (multi)
-        for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
+    const bool hands_over = multi && w + 1 < nseg;
 
-    for (int band = 0; band < wg.nBands; ++band) {
+    // one band of rows from `cur`, with the next band's loads issued into `nxt` first
+    auto do_band = [&](Stage &cur, Stage &nxt, int band) {
         if (band + 1 < wg.nBands) load_band(nxt, band + 1);
+        const int i0 = band * R;
+        uint32_t oo = mad24(mad24(i0, rs, r0m), OhB * rs, colO);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int i = band * R + r;
-            if (i < H) {
+            if (i0 + r < H) {
                 const float u = cvt_raw(tp, cur.u[r]);
                 const float raw = cvt_raw(tp, cur.d[r]) + bias;
                 float dsp;
-                const float dl = softplus ? softplus20(raw, dsp) : raw;
+                const float dl = (softplus && !(SND_WAVE_ABLATE & 4)) ? softplus20(raw, dsp) : raw;
                 const float du = dl * u;
                 float acc = 0.f;
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column 64w-1
-                    float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (w > 0) in = sHO[(step + 1) & 1][w - 1][r % RD][n];
+                    const float4 in = (SND_WAVE_ABLATE & 32) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][w][r % RD][n];
                     const float a = fast_exp2(fmaf(dl, A2[n], ld));
-                    const float bu = (n < N ? cvt_raw(tp, cur.b[r][n]) : 0.f) * du;
+                    const float bu = ((NS == 4 && n >= N) ? 0.f : cvt_raw(tp, cur.b[r][n])) * du;
                     const float a_l = from_prev_lane(a, in.z);                 // a[i, j-1]
                     const float h_d = from_prev_lane(hprev[n], hdiag[n]);      // h[i-1, j-1]
                     const float X = fmaf(-0.5f * (aprev[n] + a_l), h_d, hprev[n]);
                     float Y = fmaf(a, X, bu), S = bu, Ap = a;
-                    wave_scan3(Y, S, Ap);
+                    if (!(SND_WAVE_ABLATE & 8)) wave_scan3(Y, S, Ap);
                     const float h = fmaf(Ap, in.x, Y);
                     const float s = fmaf(Ap, in.y, S);
                     acc = fmaf(cvt_raw(tp, cur.c[r][n]), fmaf(0.25f, bu, h - s), acc);
                     hdiag[n] = in.x;
                     hprev[n] = h;
                     aprev[n] = a;
-                    if (multi && lane == 63 && w + 1 < nseg) sHO[step & 1][w][r % RD][n] = make_float4(h, s, a, 0.f);
+                    if (!(SND_WAVE_ABLATE & 32) && hands_over && lane == 63) sHO[step & 1][w + 1][r % RD][n] = make_float4(h, s, a, 0.f);
                     if (SAVE && lane == r) { ch[n] = in.x; cs[n] = in.y; ca[n] = in.z; }
                 }
-                if (jin) st_f32_b(outb, mad24(mad24(i, rs, r0m), OhB, colO), p.out_dtype, fmaf(Dv, u, acc));
+                if (jin && (!(SND_WAVE_ABLATE & 1) || acc == 1234.5f)) stg_b(outb, oo, fmaf(Dv, u, acc));
+                oo += OhB;
             }
-            if (multi && r % RD == RD - 1) { lds_barrier(); ++step; }
+            if (multi && r % RD == RD - 1) { if (!(SND_WAVE_ABLATE & 2)) lds_barrier(); ++step; }
         }
         // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
-            if (n < N) {
+            if ((NS != 4 || n < N) && !(SND_WAVE_ABLATE & 16)) {
                 float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
                 __builtin_nontemporal_store(hprev[n], dst);
                 __builtin_nontemporal_store(aprev[n], dst + wg.Wp);
             }
         }
         // column checkpoints: lanes 0..R-1 hold what entered the segment on the band's rows
-        if (SAVE && w > 0 && lane < R) {
+        if (SAVE && w > 0 && lane < R && !(SND_WAVE_ABLATE & 16)) {
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                if (n < N) {
+                if (NS != 4 || n < N) {
                     const int64_t o = (int64_t)n * wave_x_plane(wg) + band * R + lane;
                     xh[o] = ch[n];
                     xh[o + wg.Hp] = ca[n];
@@ -166,7 +182,16 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                 }
             }
         }
-        cur = nxt;
+    };
+
+    Stage sA, sB;
+    load_band(sA, 0);
+    lds_barrier();                                   // the zeroed slot
+    if (multi)
+        for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
+    for (int band = 0; band < wg.nBands; band += 2) {
+        do_band(sA, sB, band);
+        if (band + 1 < wg.nBands) do_band(sB, sA, band + 1);
     }
     if (multi)
         for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
@@ -176,11 +201,12 @@ template <typename T, int NS>
 static int launch_wave_fwd_ns(const snd_fwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
-    const int grid = wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
-    if (p.x != nullptr)
-        hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
-    else
-        hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false>), dim3(grid), dim3(64 * wg.nseg), 0, stream, p, wg);
+    const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
+    const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
+    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true, true>), grid, block, 0, stream, p, wg);
+    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
+    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false, true>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
