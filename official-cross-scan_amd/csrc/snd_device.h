@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "snd_scan.h"
 
 namespace snd {
@@ -386,25 +387,33 @@ __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, in
 // neighbours in the row come from wave_shr:1 / wave_shl:1; the state at a segment's last column goes to
 // the next wave through a few LDS words per row.
 struct WaveGeo {
-    int nseg;                      // row segments (waves per plane): ceil(W / 64)
+    int nseg;                      // row segments (waves per plane): ceil(W / (64 * cpl))
     int R;                         // rows per band: row-checkpoint spacing = rows the backward holds in registers
     int nBands;                    // ceil(H / R)
-    int Hp, Wp;                    // nBands * R, nseg * 64
+    int Hp, Wp;                    // nBands * R, nseg * 64 * cpl
+    int cpl;                       // columns per lane: 1, or 2 (a lane owns two neighbouring columns: the scan and every
+                                   // per-row overhead are paid once per two cells, and loads are twice as wide)
 };
 constexpr int kSeg = 64;
 constexpr int kMaxSeg = 8;
-__host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 && W <= kSeg * kMaxSeg; }
+// Two columns per lane for one state and rows of 514 to 1024 columns (an even number): eight waves then still
+// cover a row.  Narrower rows keep one column per lane - measured at 256 planes of 512 x 512: the same forward
+// time and a 1.5 x slower backward with two, whose doubled per-lane state leaves one wave per SIMD.  Decided by
+// the shape alone, because the saved state's segment boundaries follow from it.
+__host__ __device__ inline int wave_cpl(int W, int N) { return (N <= 1 && W > kSeg * kMaxSeg && W % 2 == 0) ? 2 : 1; }
+__host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 && W <= kSeg * kMaxSeg * wave_cpl(W, N); }
 __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     WaveGeo g;
-    g.nseg = (W + kSeg - 1) / kSeg;
+    g.cpl = wave_cpl(W, N);
+    g.nseg = (W + kSeg * g.cpl - 1) / (kSeg * g.cpl);
     g.R = N <= 1 ? 8 : 4;             // (the backward keeps a band's h, s, a and inputs of every state in registers)
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
-    g.Wp = g.nseg * kSeg;
+    g.Wp = g.nseg * kSeg * g.cpl;
     return g;
 }
-// Saved state of this family, per (batch, channel, state) plane, fp32:
-//   x    [segment w][2][Hp]   h, then a, at column 64w-1 of every row (what segment w needs from its left)
+// Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):
+//   x    [segment w][2][Hp]   h, then a, at column S*w-1 of every row (what segment w needs from its left)
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][2][Wp]        h, then a, on the last row of every band
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
@@ -424,19 +433,60 @@ __host__ inline int wave_grid(int nPairs, int rg) { return (nPairs >= 16 || (nPa
 // where they are used (a conversion at the load would put the wait for the load there).  They are loaded
 // without any lane condition: a load whose result is only needed under a lane condition is sunk into that
 // condition by the compiler - a branch with a full wait behind every load.
-__device__ __forceinline__ uint32_t ldraw_b(const float *base, uint32_t off) { uint32_t v = *(const uint32_t *)((const char *)base + off); return v; }
-__device__ __forceinline__ uint32_t ldraw_b(const bf16_t *base, uint32_t off) { uint32_t v = *(const uint16_t *)((const char *)base + off); return v; }
-__device__ __forceinline__ uint32_t ldraw_b(const f16_t *base, uint32_t off) { uint32_t v = *(const uint16_t *)((const char *)base + off); return v; }
-__device__ __forceinline__ uint32_t ldraw_dt(const void *base, uint32_t off, int dt) {
-    return dt == SND_F32 ? *(const uint32_t *)((const char *)base + off) : (uint32_t) * (const uint16_t *)((const char *)base + off);
+// A lane's CPL neighbouring elements come with one load when the tensor's alignment allows it (VEC: 4 bytes for
+// two 16-bit values, 8 for two floats), else with one load per element.  Element e is the e-th in memory order.
+template <typename T, int CPL, bool VEC> struct WaveRaw {
+    static constexpr bool PACKED = CPL == 2 && VEC && sizeof(T) == 2;          // two 16-bit values in one register
+    static constexpr int RW = PACKED ? 1 : CPL;
+    // 16-bit values stay 16-bit until they are converted: widening them at the load would be an instruction per
+    // value that has to wait for the load
+    typedef typename std::conditional<sizeof(T) == 4 || PACKED, uint32_t, uint16_t>::type word_t;
+    word_t w[RW];
+};
+template <typename T, int CPL, bool VEC>
+__device__ __forceinline__ void wave_ld(WaveRaw<T, CPL, VEC> &q, const T *base, uint32_t off) {
+    typedef WaveRaw<T, CPL, VEC> R;
+    const char *a = (const char *)base + off;
+    if (R::PACKED) {
+        q.w[0] = *(const typename R::word_t *)a;
+    } else if (CPL == 2 && VEC) {
+        const uint2 v = *(const uint2 *)a;
+        q.w[0] = v.x;
+        q.w[R::RW - 1] = v.y;
+    } else {
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) q.w[e] = *(const typename R::word_t *)(a + e * sizeof(T));
+    }
 }
-__device__ __forceinline__ float cvt_raw(const float *, uint32_t r) { return __builtin_bit_cast(float, r); }
-__device__ __forceinline__ float cvt_raw(const bf16_t *, uint32_t r) { return __builtin_bit_cast(float, r << 16); }
-__device__ __forceinline__ float cvt_raw(const f16_t *, uint32_t r) { return (float)__builtin_bit_cast(f16_t, (uint16_t)r); }
-__device__ __forceinline__ float cvt_raw_dt(uint32_t r, int dt) {
-    if (dt == SND_F32) return __builtin_bit_cast(float, r);
-    if (dt == SND_BF16) return __builtin_bit_cast(float, r << 16);
-    return (float)__builtin_bit_cast(f16_t, (uint16_t)r);
+__device__ __forceinline__ float cvt_bits(const float *, uint32_t r) { return __builtin_bit_cast(float, r); }
+__device__ __forceinline__ float cvt_bits(const bf16_t *, uint16_t r) { return __builtin_bit_cast(float, (uint32_t)r << 16); }
+__device__ __forceinline__ float cvt_bits(const f16_t *, uint16_t r) { return (float)__builtin_bit_cast(f16_t, r); }
+template <typename T, int CPL, bool VEC>
+__device__ __forceinline__ float wave_elem(const WaveRaw<T, CPL, VEC> &q, int e) {
+    typedef WaveRaw<T, CPL, VEC> R;
+    const T *const tp = nullptr;
+    if (R::PACKED) {
+        const uint32_t v = q.w[0];
+        if (std::is_same<T, bf16_t>::value) return __builtin_bit_cast(float, e == 0 ? v << 16 : v & 0xffff0000u);
+        return cvt_bits(tp, (uint16_t)(e == 0 ? v : v >> 16));
+    }
+    return cvt_bits(tp, q.w[e < R::RW ? e : 0]);
+}
+// CPL values to consecutive elements in memory order
+template <typename T, int CPL, bool VEC>
+__device__ __forceinline__ void wave_st(T *base, uint32_t off, const float (&v)[CPL]) {
+    char *a = (char *)base + off;
+    if (CPL == 2 && VEC && sizeof(T) == 4) {
+        *(float2 *)a = make_float2(v[0], v[CPL - 1]);
+    } else if (CPL == 2 && VEC) {
+        uint32_t lo, hi;
+        if (std::is_same<T, bf16_t>::value) { lo = f32_to_bf16(v[0]); hi = f32_to_bf16(v[CPL - 1]); }
+        else { lo = __builtin_bit_cast(uint16_t, (f16_t)v[0]); hi = __builtin_bit_cast(uint16_t, (f16_t)v[CPL - 1]); }
+        *(uint32_t *)a = lo | (hi << 16);
+    } else {
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) stg_b(base, off + e * (uint32_t)sizeof(T), v[e]);
+    }
 }
 // Block barrier for hand-overs through LDS only: waits for this wave's LDS traffic, not for its global loads
 // and stores (the prefetched rows and the row just written stay in flight across it; __syncthreads would
@@ -465,6 +515,36 @@ __device__ __forceinline__ void wave_scan3(float &y, float &s, float &a) {
             SND_SCAN3_LVL("row_shr:8", "0xf") SND_SCAN3_LVL("row_bcast:15", "0xa") SND_SCAN3_LVL("row_bcast:31", "0xc")
         : "+v"(y), "+v"(s), "+v"(a));
 }
+// One row of a segment: t_j = a_j*t_{j-1} + y_j and the same with s_j, over the CPL columns of each of the 64
+// lanes, lanes ascending in the direction of the recurrence, cy / cs entering the first column of lane 0.
+// The CPL maps of a lane are composed first, one scan runs over the lanes, and the lane's columns are filled
+// in from the value entering the lane.  Returns the solutions per column (the lane's last: oy[CPL-1]).
+template <int CPL>
+__device__ __forceinline__ void wave_row_solve(const float (&a)[CPL], const float (&y)[CPL], const float (&sv)[CPL], float cy,
+                                               float cs, float (&oy)[CPL], float (&os)[CPL]) {
+    float Y = y[0], S = sv[0], Ap = a[0];
+#pragma unroll
+    for (int k = 1; k < CPL; ++k) {
+        Y = fmaf(a[k], Y, y[k]);
+        S = fmaf(a[k], S, sv[k]);
+        Ap *= a[k];
+    }
+    wave_scan3(Y, S, Ap);
+    const float ey = fmaf(Ap, cy, Y), es = fmaf(Ap, cs, S);      // at the lane's last column
+    if (CPL > 1) {
+        float ty = from_prev_lane(ey, cy), ts = from_prev_lane(es, cs);   // entering the lane
+#pragma unroll
+        for (int k = 0; k < CPL - 1; ++k) {
+            ty = fmaf(a[k], ty, y[k]);
+            ts = fmaf(a[k], ts, sv[k]);
+            oy[k] = ty;
+            os[k] = ts;
+        }
+    }
+    oy[CPL - 1] = ey;
+    os[CPL - 1] = es;
+}
+
 // Sum over the 64 lanes; the total ends in lane 63.
 __device__ __forceinline__ float wave_sum_to_last(float v) {
     v += dpp_old<0x111, 0xF>(0.f, v);

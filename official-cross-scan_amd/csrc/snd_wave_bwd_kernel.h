@@ -13,9 +13,10 @@
 // states in registers.  Along a row the adjoint is first order towards the left,
 //     G_j = a_j*G_{j+1} + a_j*z_j,   z_j = dout*C + G[i+1,j] - 0.5*(a[i,j+1] + a[i+1,j])*G[i+1,j+1],
 // so a wave resolves a row with one DPP scan, exactly like the forward - provided its lanes run against
-// the columns.  Every load, store and the whole adjoint sweep therefore use the mirrored order (lane l =
-// column 64w + 63 - l); only the recomputation of h and s, which runs with the columns, sees its inputs and
-// leaves its results through a lane reversal (ds_bpermute: a register crossbar move, no LDS memory).
+// the columns.  Every load, store and the whole adjoint sweep therefore use the mirrored order (lane l owns
+// the columns that lane 63 - l owns in the forward, and walks them downwards); only the recomputation of h and
+// s, which runs with the columns, sees its inputs and leaves its results through a lane reversal (ds_bpermute:
+// a register crossbar move, no LDS memory).
 // A wave handles its segment band by band (R rows), bottom band first: recompute h, s of the band's rows
 // from the forward's checkpoints (row above the band from x_v, what entered the segment on every row from
 // x / x_sd: no wave waits for another here), then sweep the band's rows bottom-up.  The sweep needs G, Gs, a
@@ -23,6 +24,7 @@
 // LDS (one block barrier per band, no polling).  dB, dC leave as one global atomic per element and channel
 // (a wave-wide instruction covers 256 consecutive bytes), du / ddelta as whole row segments.
 #pragma once
+#include <initializer_list>
 #include <type_traits>
 #include "snd_device.h"
 
@@ -32,10 +34,11 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename T, int NS, bool DO32>
+template <typename T, int NS, int CPL, bool VEC, bool DO32>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
-    constexpr bool PF = NS <= 2;                     // load a band's inputs one band ahead (with four states the registers are needed elsewhere)
+    // load a band's inputs one band ahead (with four states, or two columns per lane, the registers are needed elsewhere)
+    constexpr bool PF = NS <= 2 && CPL == 1;
     // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and
     // state.  Wave w writes slot w and reads slot w+1; the slot after the last wave stays zero.
     __shared__ float4 sHO[2][kMaxSeg + 1][R][NS];
@@ -54,11 +57,13 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
-    const int jm = w * kSeg + 63 - lane;             // this lane's column (mirrored order)
-    const bool jin = jm < W;
-    const int jc = jin ? jm : W - 1;
-    const int mc = fh ? W - 1 - jc : jc;
-    const int jn = w * kSeg + lane;                  // natural order (row checkpoints, recomputation)
+    // Mirrored order: this lane owns scan columns jm0 .. jm0+CPL-1 and walks them downwards (its local index t is
+    // scan column jm0 + CPL-1-t); in natural order (row checkpoints, recomputation) lane l owns columns jn0 ...
+    const int jm0 = (w * kSeg + 63 - lane) * CPL;
+    const bool jin = jm0 < W;
+    const int jc = jin ? jm0 : W - CPL;
+    const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
+    const int jn0 = (w * kSeg + lane) * CPL;
     const int rev_addr = (63 - lane) * 4;
     auto mirror = [&](float v) {
         return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(rev_addr, __builtin_bit_cast(int, v)));
@@ -99,17 +104,17 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn;
+    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn0;
     const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
     const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
 
     // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
-    // last column (always in bounds) and only their dout is masked to zero where it is used, which makes every
+    // last columns (always in bounds) and only their dout is masked to zero where it is used, which makes every
     // adjoint there exactly zero.  h0, a0: the row above the band in natural order.  ch, cs, ca: what entered
     // the segment from the left on rows i0-1 .. i0+R-1, one row per lane.
-    struct In { uint32_t u[R], d[R], o[R], b[R][NS], c[R][NS]; float h0[NS], a0[NS], ch[NS], cs[NS], ca[NS]; };
-    const T *const tp = nullptr;                     // selects the conversions
-    const DoT *const dp = nullptr;
+    typedef WaveRaw<T, CPL, VEC> Raw;
+    typedef WaveRaw<DoT, CPL, VEC> RawO;
+    struct In { Raw u[R], d[R], b[R][NS], c[R][NS]; RawO o[R]; float h0[NS][CPL], a0[NS][CPL], ch[NS], cs[NS], ca[NS]; };
     // Every band issues the same loads on every path (the wait counters the compiler derives for the prefetch
     // need that): rows past the end of a ragged last band read the last row again and are never used.
     auto load_band = [&](In &q, int band) {
@@ -119,14 +124,14 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                  ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            q.u[r] = ldraw_b(ub, ou);
-            q.d[r] = ldraw_b(db, od);
-            q.o[r] = ldraw_b(dob, oo);
+            wave_ld(q.u[r], ub, ou);
+            wave_ld(q.d[r], db, od);
+            wave_ld(q.o[r], dob, oo);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 const int sn = (NS == 4 && n >= N) ? 0 : n;
-                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), ob);
-                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), oc);
+                wave_ld(q.b[r][n], (const T *)((const char *)Bb + sn * BsB), ob);
+                wave_ld(q.c[r][n], (const T *)((const char *)Cb + sn * CsB), oc);
             }
             const bool more = i0 + r + 1 < H;
             ou += more ? UhB : 0; od += more ? DhB : 0; oo += more ? DohB : 0; ob += more ? BhB : 0; oc += more ? ChB : 0;
@@ -134,12 +139,17 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         const int row = i0 - 1 + lane;
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
-            q.h0[n] = 0.f; q.a0[n] = 0.f; q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
+            q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
+#pragma unroll
+            for (int k = 0; k < CPL; ++k) { q.h0[n][k] = 0.f; q.a0[n][k] = 0.f; }
             if (NS != 4 || n < N) {
                 if (band > 0) {
                     const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
-                    q.h0[n] = __builtin_nontemporal_load(src);
-                    q.a0[n] = __builtin_nontemporal_load(src + wg.Wp);
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) {
+                        q.h0[n][k] = __builtin_nontemporal_load(src + k);
+                        q.a0[n][k] = __builtin_nontemporal_load(src + wg.Wp + k);
+                    }
                 }
                 if (w > 0 && lane <= R && row >= 0) {
                     const int64_t o = (int64_t)n * wave_x_plane(wg) + row;
@@ -150,123 +160,211 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
             }
         }
     };
+    // the lane's CPL values in its walking order t (element e of the raw bits is t = CPL-1-e, or t = e when fh)
+    auto unpack = [&](const auto &q, float (&v)[CPL]) {
+#pragma unroll
+        for (int k = 0; k < CPL; ++k) v[k] = wave_elem(q, k);
+        if (CPL == 2 && !fh) { const float t = v[0]; v[0] = v[CPL - 1]; v[CPL - 1] = t; }
+    };
 
-    float Gd[NS], ad[NS], GdEdge[NS];               // G, a of the row below at this column; G[i+1, 64(w+1)]
+    float Gd[NS][CPL], ad[NS][CPL], GdEdge[NS];     // G, a of the row below at this lane's columns; G[i+1, S*(w+1)]
     float dA_acc[NS];
     float dec_acc = 0.f, dD_acc = 0.f, dbias_acc = 0.f;
 #pragma unroll
-    for (int n = 0; n < NS; ++n) { Gd[n] = 0.f; ad[n] = 0.f; GdEdge[n] = 0.f; dA_acc[n] = 0.f; }
+    for (int n = 0; n < NS; ++n) {
+        GdEdge[n] = 0.f; dA_acc[n] = 0.f;
+#pragma unroll
+        for (int k = 0; k < CPL; ++k) { Gd[n][k] = 0.f; ad[n][k] = 0.f; }
+    }
     int step = nseg - 1 - w;                         // the waves on the right go first
     const bool hands_over = multi && w > 0;
 
     // one band from `cur`, with the loads of the band above issued into `nxt` first
     auto do_band = [&](In &cur, In &nxt, int band) {
-        if (PF) { if (band > 0) load_band(nxt, band - 1); }
+        if (PF) load_band(nxt, max(band - 1, 0));       // unconditionally (band 0 once more): a skipped load would leave two paths with
+                                                        // different numbers of loads in flight, and the waits follow the smaller
         else load_band(cur, band);
         const int i0 = band * R;
 
-        // ---- recompute h, s on the band's rows (with the columns); results back in mirrored order
-        float hT[R][NS], sT[R][NS], aT[R][NS], dl[R], dsp[R], hTop[NS];
+        // ---- recompute h, s on the band's rows (with the columns); results back in mirrored order.
+        // Index t of the mirrored order is natural column index CPL-1-t of the lane that holds the same columns.
+        float hT[R][NS][CPL], sT[R][NS][CPL], aT[R][NS][CPL], dl[R][CPL], dsp[R][CPL], uu[R][CPL], hTop[NS][CPL];
         {
-            float hp[NS], ap[NS], hdiag[NS];
+            float hp[NS][CPL], ap[NS][CPL], hdiag[NS];
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                hp[n] = cur.h0[n];
-                ap[n] = cur.a0[n];
                 hdiag[n] = bcast(cur.ch[n], 0);
-                hTop[n] = mirror(cur.h0[n]);
+#pragma unroll
+                for (int k = 0; k < CPL; ++k) {
+                    hp[n][k] = cur.h0[n][k];
+                    ap[n][k] = cur.a0[n][k];
+                    hTop[n][CPL - 1 - k] = mirror(cur.h0[n][k]);
+                }
+            }
+            // What the rows need that does not depend on the rows above them - softplus, delta' * u, and their
+            // copies in natural lane order - for the whole band at once: R independent chains of transcendentals and
+            // a train of lane reversals in flight, instead of one chain and three round trips in front of every row's scan.
+            float dln_[R][CPL], dlun_[R][CPL], bn_[R][NS][CPL];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                unpack(cur.u[r], uu[r]);
+                unpack(cur.d[r], dl[r]);
+#pragma unroll
+                for (int t = 0; t < CPL; ++t) {
+                    const float raw = dl[r][t] + bias;
+                    float sg = 1.f;
+                    dl[r][t] = softplus ? softplus20(raw, sg) : raw;
+                    dsp[r][t] = sg;
+                }
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                dl[r] = 0.f;
-                dsp[r] = 0.f;
+#pragma unroll
+                for (int t = 0; t < CPL; ++t) {
+                    dln_[r][CPL - 1 - t] = mirror(dl[r][t]);
+                    dlun_[r][CPL - 1 - t] = mirror(dl[r][t] * uu[r][t]);
+                }
+#pragma unroll
+                for (int n = 0; n < NS; ++n) {
+                    float bm[CPL];
+                    unpack(cur.b[r][n], bm);
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) bn_[r][n][CPL - 1 - t] = (NS == 4 && n >= N) ? 0.f : mirror(bm[t]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
                 if (i0 + r < H) {
-                    const float raw = cvt_raw(tp, cur.d[r]) + bias;
-                    float sg = 1.f;
-                    dl[r] = softplus ? softplus20(raw, sg) : raw;
-                    dsp[r] = sg;
-                    const float dl_n = mirror(dl[r]), dlu_n = mirror(dl[r] * cvt_raw(tp, cur.u[r]));
+                    const float (&dln)[CPL] = dln_[r], (&dlun)[CPL] = dlun_[r];
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
                         const float hin = bcast(cur.ch[n], r + 1), sin_ = bcast(cur.cs[n], r + 1), ain = bcast(cur.ca[n], r + 1);
-                        const float a = fast_exp2(fmaf(dl_n, A2[n], ld));
-                        const float bu = ((NS == 4 && n >= N) ? 0.f : mirror(cvt_raw(tp, cur.b[r][n]))) * dlu_n;
-                        const float a_l = from_prev_lane(a, ain);              // a[i, j-1]
-                        const float h_d = from_prev_lane(hp[n], hdiag[n]);     // h[i-1, j-1]
-                        const float X = fmaf(-0.5f * (ap[n] + a_l), h_d, hp[n]);
-                        float Y = fmaf(a, X, bu), S = bu, Ap = a;
-                        wave_scan3(Y, S, Ap);
-                        const float h = fmaf(Ap, hin, Y);
-                        const float s = fmaf(Ap, sin_, S);
-                        hT[r][n] = mirror(h);
-                        sT[r][n] = mirror(s);
-                        aT[r][n] = mirror(a);
-                        hp[n] = h;
-                        ap[n] = a;
+                        float a[CPL], bu[CPL], y[CPL], h[CPL], s[CPL];
+#pragma unroll
+                        for (int k = 0; k < CPL; ++k) {
+                            a[k] = fast_exp2(fmaf(dln[k], A2[n], ld));
+                            bu[k] = bn_[r][n][k] * dlun[k];
+                        }
+                        const float a_l = from_prev_lane(a[CPL - 1], ain);                 // a[i, j-1] of the lane's first column
+                        const float h_d = from_prev_lane(hp[n][CPL - 1], hdiag[n]);        // h[i-1, j-1]
+#pragma unroll
+                        for (int k = 0; k < CPL; ++k) {
+                            const float al = k == 0 ? a_l : a[k > 0 ? k - 1 : 0], hd = k == 0 ? h_d : hp[n][k > 0 ? k - 1 : 0];
+                            const float X = fmaf(-0.5f * (ap[n][k] + al), hd, hp[n][k]);
+                            y[k] = fmaf(a[k], X, bu[k]);
+                        }
+                        wave_row_solve<CPL>(a, y, bu, hin, sin_, h, s);
+#pragma unroll
+                        for (int k = 0; k < CPL; ++k) {
+                            hT[r][n][CPL - 1 - k] = mirror(h[k]);
+                            sT[r][n][CPL - 1 - k] = mirror(s[k]);
+                            aT[r][n][CPL - 1 - k] = mirror(a[k]);
+                            hp[n][k] = h[k];
+                            ap[n][k] = a[k];
+                        }
                         hdiag[n] = hin;
                     }
                 } else {
 #pragma unroll
-                    for (int n = 0; n < NS; ++n) { hT[r][n] = 0.f; sT[r][n] = 0.f; aT[r][n] = 0.f; }
+                    for (int n = 0; n < NS; ++n)
+#pragma unroll
+                        for (int t = 0; t < CPL; ++t) { hT[r][n][t] = 0.f; sT[r][n][t] = 0.f; aT[r][n][t] = 0.f; }
                 }
             }
         }
 
-        // ---- adjoint sweep over the band's rows, bottom-up (against the columns)
+        // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
         const int rows = min(R, H - i0);             // rows of this band inside the plane
         const int mlast = mad24(i0 + rows - 1, rs, r0m);
         uint32_t og = mad24(mlast, WB * rs, colB), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
 #pragma unroll
         for (int r = R - 1; r >= 0; --r) {
             if (i0 + r < H) {
-                const float dov = jin ? cvt_raw(dp, cur.o[r]) : 0.f, uv = cvt_raw(tp, cur.u[r]), dlv = dl[r];
-                const float dlu = dlv * uv;
-                float qsum = 0.f, psum = 0.f;
+                float dov[CPL], dlu[CPL], qsum[CPL], psum[CPL];
+                unpack(cur.o[r], dov);
+#pragma unroll
+                for (int t = 0; t < CPL; ++t) {
+                    dov[t] = jin ? dov[t] : 0.f;
+                    dlu[t] = dl[r][t] * uu[r][t];
+                    qsum[t] = 0.f;
+                    psum[t] = 0.f;
+                }
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
-                    // what the segment on the right left for this row: G, Gs, a at column 64(w+1)
+                    // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
                     const float4 in = sHO[(step + 1) & 1][w + 1][r][n];
-                    const float hin = bcast(cur.ch[n], r + 1);                 // h[i, 64w-1]
+                    const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
                     const bool live = NS != 4 || n < N;
-                    const float Bv = live ? cvt_raw(tp, cur.b[r][n]) : 0.f, Cv = live ? cvt_raw(tp, cur.c[r][n]) : 0.f;
-                    const float a = aT[r][n];
-                    const float bu = Bv * dlu;
-                    const float dyC = dov * Cv;
-                    const float a_r = from_prev_lane(a, in.z);                 // a[i, j+1]
-                    const float Gdiag = from_prev_lane(Gd[n], GdEdge[n]);      // G[i+1, j+1]
-                    const float z = fmaf(-0.5f * (a_r + ad[n]), Gdiag, dyC + Gd[n]);
-                    float Y = a * z, S = -a * dyC, Ap = a;
-                    wave_scan3(Y, S, Ap);
-                    const float Gt = fmaf(Ap, in.x, Y), Gst = fmaf(Ap, in.y, S);   // G[i,j], Gs[i,j]
-                    const float Gr = from_prev_lane(Gt, in.x), Gsr = from_prev_lane(Gst, in.y);
-                    const float g_ = Gr + z, gs = Gsr - dyC;
-                    const float dbu = fmaf(0.25f, dyC, g_ + gs);
-                    const float hv = hT[r][n], sv = sT[r][n];
-                    const float h_l = from_next_lane(hv, hin);                 // h[i, j-1]
-                    const float h_u = r > 0 ? hT[r > 0 ? r - 1 : 0][n] : hTop[n];
-                    const float hs = hv - sv, sb = sv - bu;
-                    const float cross = fmaf(Gd[n], h_l, Gr * h_u);
-                    const float da = fmaf(-0.5f * a, cross, fmaf(g_, hs, (g_ + gs) * sb));
-                    dA_acc[n] = fmaf(dlv, da, dA_acc[n]);
-                    if (want_decay) dec_acc += da;
-                    qsum = fmaf(dbu, Bv, qsum);
-                    psum = fmaf(Av[n], da, psum);
+                    float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
+                    unpack(cur.b[r][n], Bv);
+                    unpack(cur.c[r][n], Cv);
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        Bv[t] = live ? Bv[t] : 0.f;
+                        Cv[t] = live ? Cv[t] : 0.f;
+                        a[t] = aT[r][n][t];
+                        bu[t] = Bv[t] * dlu[t];
+                        dyC[t] = dov[t] * Cv[t];
+                    }
+                    const float a_r0 = from_prev_lane(a[CPL - 1], in.z);               // a[i, j+1] of the lane's first column
+                    const float Gdg0 = from_prev_lane(Gd[n][CPL - 1], GdEdge[n]);      // G[i+1, j+1]
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        const float ar = t == 0 ? a_r0 : a[t > 0 ? t - 1 : 0], gdg = t == 0 ? Gdg0 : Gd[n][t > 0 ? t - 1 : 0];
+                        z[t] = fmaf(-0.5f * (ar + ad[n][t]), gdg, dyC[t] + Gd[n][t]);
+                        ya[t] = a[t] * z[t];
+                        ys[t] = -a[t] * dyC[t];
+                    }
+                    wave_row_solve<CPL>(a, ya, ys, in.x, in.y, Gt, Gst);               // G[i,j], Gs[i,j]
+                    const float Gr0 = from_prev_lane(Gt[CPL - 1], in.x), Gsr0 = from_prev_lane(Gst[CPL - 1], in.y);
+                    const float hl_last = from_next_lane(hT[r][n][0], hin);            // h[i, j-1] of the lane's last column
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        const float Gr = t == 0 ? Gr0 : Gt[t > 0 ? t - 1 : 0], Gsr = t == 0 ? Gsr0 : Gst[t > 0 ? t - 1 : 0];
+                        const float g_ = Gr + z[t], gs = Gsr - dyC[t];
+                        const float dbu = fmaf(0.25f, dyC[t], g_ + gs);
+                        const float hv = hT[r][n][t], sv = sT[r][n][t];
+                        const float h_l = t == CPL - 1 ? hl_last : hT[r][n][t < CPL - 1 ? t + 1 : 0];
+                        const float h_u = r > 0 ? hT[r > 0 ? r - 1 : 0][n][t] : hTop[n][t];
+                        const float hs = hv - sv, sb = sv - bu[t];
+                        const float cross = fmaf(Gd[n][t], h_l, Gr * h_u);
+                        const float da = fmaf(-0.5f * a[t], cross, fmaf(g_, hs, (g_ + gs) * sb));
+                        dA_acc[n] = fmaf(dl[r][t], da, dA_acc[n]);
+                        if (want_decay) dec_acc += da;
+                        qsum[t] = fmaf(dbu, Bv[t], qsum[t]);
+                        psum[t] = fmaf(Av[n], da, psum[t]);
+                        ya[t] = dbu * dlu[t];                                          // dB, dC contributions (reusing the arrays)
+                        ys[t] = dov[t] * fmaf(0.25f, bu[t], hs);
+                    }
                     if (jin && live) {
-                        wave_glb_add((float *)((char *)dBg + n * HW4 + o4), dbu * dlu);
-                        wave_glb_add((float *)((char *)dCg + n * HW4 + o4), dov * fmaf(0.25f, bu, hs));
+#pragma unroll
+                        for (int e = 0; e < CPL; ++e) {                                // memory order
+                            const int t = fh ? e : CPL - 1 - e;
+                            const float vb = (CPL == 2 && t == 1) ? ya[CPL - 1] : ya[0], vc = (CPL == 2 && t == 1) ? ys[CPL - 1] : ys[0];
+                            wave_glb_add((float *)((char *)dBg + n * HW4 + o4) + e, vb);
+                            wave_glb_add((float *)((char *)dCg + n * HW4 + o4) + e, vc);
+                        }
                     }
                     GdEdge[n] = in.x;
-                    Gd[n] = Gt;
-                    ad[n] = a;
-                    if (hands_over && lane == 63) sHO[step & 1][w][r][n] = make_float4(Gt, Gst, a, 0.f);
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) { Gd[n][t] = Gt[t]; ad[n][t] = a[t]; }
+                    if (hands_over && lane == 63) sHO[step & 1][w][r][n] = make_float4(Gt[CPL - 1], Gst[CPL - 1], a[CPL - 1], 0.f);
                 }
-                const float duv = fmaf(Dv, dov, dlv * qsum);
-                const float ddl = fmaf(uv, qsum, psum) * dsp[r];
                 if (jin) {
-                    dD_acc = fmaf(dov, uv, dD_acc);
-                    dbias_acc += ddl;
-                    stg_b(dub, og, duv);
-                    stg_b(ddb, og, ddl);
+                    float duv[CPL], ddl[CPL];
+#pragma unroll
+                    for (int t = 0; t < CPL; ++t) {
+                        duv[t] = fmaf(Dv, dov[t], dl[r][t] * qsum[t]);
+                        ddl[t] = fmaf(uu[r][t], qsum[t], psum[t]) * dsp[r][t];
+                        dD_acc = fmaf(dov[t], uu[r][t], dD_acc);
+                        dbias_acc += ddl[t];
+                    }
+                    if (CPL == 2 && !fh) {                                             // to memory order
+                        float t_ = duv[0]; duv[0] = duv[CPL - 1]; duv[CPL - 1] = t_;
+                        t_ = ddl[0]; ddl[0] = ddl[CPL - 1]; ddl[CPL - 1] = t_;
+                    }
+                    wave_st<T, CPL, VEC>(dub, og, duv);
+                    wave_st<T, CPL, VEC>(ddb, og, ddl);
                 }
                 og -= WB;
                 o4 -= W4;
@@ -311,21 +409,40 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     }
 }
 
-template <typename T, int NS>
-static int launch_wave_bwd_ns(const snd_bwd_params &p, hipStream_t stream) {
+static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::initializer_list<int64_t> strides) {
+    if ((uintptr_t)ptr % bytes) return false;
+    for (int64_t st : strides)
+        if ((st * esz) % bytes) return false;
+    return true;
+}
+
+template <typename T, int NS, int CPL, bool VEC>
+static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
-    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
-    if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, true>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
+    if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
 template <typename T>
 int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
-    const int N = p.f.shape.dstate;
-    return N == 1 ? launch_wave_bwd_ns<T, 1>(p, stream) : N == 2 ? launch_wave_bwd_ns<T, 2>(p, stream)
-                                                                  : launch_wave_bwd_ns<T, 4>(p, stream);
+    const snd_fwd_params &f = p.f;
+    const snd_shape &sh = f.shape;
+    const int N = sh.dstate;
+    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    if (wg.cpl == 2) {                               // (N = 1 only)
+        const int e = (int)sizeof(T), oe = p.dout_dtype == SND_F32 ? 4 : e;
+        const bool vec = wave_aligned_b(f.u, e, 2 * e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&
+                         wave_aligned_b(f.delta, e, 2 * e, {f.delta_batch_stride, f.delta_d_stride, f.delta_h_stride}) &&
+                         wave_aligned_b(f.B, e, 2 * e, {f.B_batch_stride, f.B_group_stride, f.B_dstate_stride, f.B_h_stride}) &&
+                         wave_aligned_b(f.C, e, 2 * e, {f.C_batch_stride, f.C_group_stride, f.C_dstate_stride, f.C_h_stride}) &&
+                         wave_aligned_b(p.dout, oe, 2 * oe, {p.dout_batch_stride, p.dout_d_stride, p.dout_h_stride}) &&
+                         wave_aligned_b(p.du, e, 2 * e, {}) && wave_aligned_b(p.ddelta, e, 2 * e, {});
+        return vec ? launch_wave_bwd_v<T, 1, 2, true>(p, wg, stream) : launch_wave_bwd_v<T, 1, 2, false>(p, wg, stream);
+    }
+    return N == 1 ? launch_wave_bwd_v<T, 1, 1, true>(p, wg, stream) : N == 2 ? launch_wave_bwd_v<T, 2, 1, true>(p, wg, stream)
+                                                                              : launch_wave_bwd_v<T, 4, 1, true>(p, wg, stream);
 }
 
 }  // namespace snd

@@ -5,8 +5,9 @@
 //     delta' = softplus(delta + bias)          a = exp2(delta' * A * log2e) * A_decay          bu = B * delta' * u
 //     h[i,j] = a*(h[i,j-1] + h[i-1,j] - 0.5*(a[i-1,j] + a[i,j-1])*h[i-1,j-1]) + bu
 //     s[i,j] = a*s[i,j-1] + bu                 out = D*u + sum_n C*(h - s + 0.25*bu)
-// Mapping: a block owns one (batch, channel); wave w of the block owns columns 64w .. 64w+63 of the
-// plane (a row segment per row), lane = column, the channel's states are registers of the lane.
+// Mapping: a block owns one (batch, channel); wave w of the block owns columns S*w .. S*w+S-1 of the
+// plane (a row segment per row; S = 64, or 128 with two neighbouring columns per lane), the channel's states
+// are registers of the lane.
 // Along a row the recurrence is first order, h_j = a_j*h_{j-1} + y_j with
 //     y_j = a_j*(h[i-1,j] - 0.5*(a[i-1,j] + a[i,j-1])*h[i-1,j-1]) + bu_j
 // known from the row above, so a wave resolves its 64 cells of a row with one inclusive scan of the
@@ -21,6 +22,7 @@
 // entering every segment on every row (x, x_sd), so that the backward can recompute any band of any
 // segment on its own.
 #pragma once
+#include <initializer_list>
 #include <type_traits>
 #include "snd_device.h"
 
@@ -32,10 +34,13 @@
 
 namespace snd {
 
-template <typename T, int NS, bool SAVE, bool OUT32>
+template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band = rows per load group
-    constexpr int RD = 2;                            // rows per wavefront step
+#ifndef SND_WAVE_RD
+#define SND_WAVE_RD 4
+#endif
+    constexpr int RD = SND_WAVE_RD < R ? SND_WAVE_RD : R;   // rows per wavefront step
     static_assert(R % RD == 0, "a band is a whole number of steps");
     // what a wave leaves for the wave on its right: {h, s, a, -} at its last column, per step parity, row and
     // state.  Wave w writes slot w+1 and reads slot w; slot 0 stays zero (nothing enters the first segment).
@@ -52,13 +57,13 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     const bool multi = nseg > 1;
     if (threadIdx.x < 2 * RD * NS) (&sHO[0][0][0][0])[(threadIdx.x / (RD * NS)) * (kMaxSeg + 1) * RD * NS + threadIdx.x % (RD * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-    // scan origin of this group: memory row = r0m + rs*i, memory column = c0m + cs*j
+    // scan origin of this group: memory row = r0m + rs*i; with fh the columns run against the memory order
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
-    const int j = w * kSeg + lane;
-    const bool jin = j < W;
-    const int jc = jin ? j : W - 1;
-    const int mc = fh ? W - 1 - jc : jc;
+    const int j0 = (w * kSeg + lane) * CPL;          // this lane's first scan column
+    const bool jin = j0 < W;                         // (W is a multiple of CPL: a lane is inside or outside as a whole)
+    const int jc = jin ? j0 : W - CPL;
+    const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
 
     float A2[NS];
 #pragma unroll
@@ -84,14 +89,14 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j;
+    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j0;
     float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
     float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
 
-    // Raw bits of a band's rows.  Lanes beyond the last column read the last column (always in bounds): what they
+    // Raw bits of a band's rows.  Lanes beyond the last column read the last columns (always in bounds): what they
     // compute only feeds cells further right and is never stored.
-    struct Stage { uint32_t u[R], d[R], b[R][NS], c[R][NS]; };
-    const T *const tp = nullptr;                     // selects the conversion
+    typedef WaveRaw<T, CPL, VEC> Raw;
+    struct Stage { Raw u[R], d[R], b[R][NS], c[R][NS]; };
     // Byte offsets advance by one row step per load (one vector add each).  Every band issues the same loads on
     // every path - the wait counters the compiler derives for the prefetch need that - so rows past the end of a
     // ragged last band read the last row again (their step is zero) and are never used.
@@ -101,62 +106,112 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         uint32_t ou = mad24(m0, UhB * rs, colB), od = mad24(m0, DhB * rs, colB), ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            q.u[r] = ldraw_b(ub, ou);
-            q.d[r] = ldraw_b(db, od);
+            wave_ld(q.u[r], ub, ou);
+            wave_ld(q.d[r], db, od);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 const int sn = (NS == 4 && n >= N) ? 0 : n;
-                q.b[r][n] = ldraw_b((const T *)((const char *)Bb + sn * BsB), ob);
-                q.c[r][n] = ldraw_b((const T *)((const char *)Cb + sn * CsB), oc);
+                wave_ld(q.b[r][n], (const T *)((const char *)Bb + sn * BsB), ob);
+                wave_ld(q.c[r][n], (const T *)((const char *)Cb + sn * CsB), oc);
             }
             const bool more = i0 + r + 1 < H;
             ou += more ? UhB : 0; od += more ? DhB : 0; ob += more ? BhB : 0; oc += more ? ChB : 0;
         }
     };
-
-    float hprev[NS], aprev[NS], hdiag[NS];          // h, a of the row above at this column; h[i-1, 64w-1]
-    float ch[NS], cs[NS], ca[NS];                   // (SAVE) what entered this segment on row band*R + lane
+    // the lane's CPL values in scan order (element e of the raw bits is scan column CPL-1-e when fh)
+    auto unpack = [&](const Raw &q, float (&v)[CPL]) {
 #pragma unroll
-    for (int n = 0; n < NS; ++n) { hprev[n] = 0.f; aprev[n] = 0.f; hdiag[n] = 0.f; ch[n] = 0.f; cs[n] = 0.f; ca[n] = 0.f; }
+        for (int k = 0; k < CPL; ++k) v[k] = wave_elem(q, k);
+        if (CPL == 2 && fh) { const float t = v[0]; v[0] = v[CPL - 1]; v[CPL - 1] = t; }
+    };
+
+    float hprev[NS][CPL], aprev[NS][CPL], hdiag[NS];   // h, a of the row above at this lane's columns; h[i-1, S*w-1]
+    float ch[NS], cs[NS], ca[NS];                      // (SAVE) what entered this segment on row band*R + lane
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+        hdiag[n] = 0.f; ch[n] = 0.f; cs[n] = 0.f; ca[n] = 0.f;
+#pragma unroll
+        for (int k = 0; k < CPL; ++k) { hprev[n][k] = 0.f; aprev[n][k] = 0.f; }
+    }
 
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     const bool hands_over = multi && w + 1 < nseg;
 
     // one band of rows from `cur`, with the next band's loads issued into `nxt` first
     auto do_band = [&](Stage &cur, Stage &nxt, int band) {
-        if (band + 1 < wg.nBands) load_band(nxt, band + 1);
+        load_band(nxt, min(band + 1, wg.nBands - 1));   // unconditionally (the last band once more): a skipped load would leave two
+                                                        // paths with different numbers of loads in flight, and the waits follow the smaller
         const int i0 = band * R;
         uint32_t oo = mad24(mad24(i0, rs, r0m), OhB * rs, colO);
+        // What the rows need that does not depend on the rows above them - softplus, delta' * u - for the RD rows
+        // of a wavefront step at once: independent chains of transcendentals that fill each other's latencies,
+        // instead of one such chain in front of every row's scan.  (Per step, not per band: the waves of a block
+        // are at different rows of their bands in the same step, and a step lasts as long as its slowest wave.)
+        float ub_[R][CPL], dlb[R][CPL], dub_[R][CPL];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            if (r % RD == 0) {
+#pragma unroll
+                for (int q = r; q < r + RD; ++q) {
+                    unpack(cur.u[q], ub_[q]);
+                    unpack(cur.d[q], dlb[q]);
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) {
+                        const float raw = dlb[q][k] + bias;
+                        float dsp;
+                        dlb[q][k] = (softplus && !(SND_WAVE_ABLATE & 4)) ? softplus20(raw, dsp) : raw;
+                        dub_[q][k] = dlb[q][k] * ub_[q][k];
+                    }
+                }
+            }
             if (i0 + r < H) {
-                const float u = cvt_raw(tp, cur.u[r]);
-                const float raw = cvt_raw(tp, cur.d[r]) + bias;
-                float dsp;
-                const float dl = (softplus && !(SND_WAVE_ABLATE & 4)) ? softplus20(raw, dsp) : raw;
-                const float du = dl * u;
-                float acc = 0.f;
+                float acc[CPL];
+                const float (&u)[CPL] = ub_[r], (&dl)[CPL] = dlb[r], (&du)[CPL] = dub_[r];
+#pragma unroll
+                for (int k = 0; k < CPL; ++k) acc[k] = 0.f;
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
-                    // what the segment on the left left for this row: h, s, a at column 64w-1
+                    // what the segment on the left left for this row: h, s, a at column S*w-1
                     const float4 in = (SND_WAVE_ABLATE & 32) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][w][r % RD][n];
-                    const float a = fast_exp2(fmaf(dl, A2[n], ld));
-                    const float bu = ((NS == 4 && n >= N) ? 0.f : cvt_raw(tp, cur.b[r][n])) * du;
-                    const float a_l = from_prev_lane(a, in.z);                 // a[i, j-1]
-                    const float h_d = from_prev_lane(hprev[n], hdiag[n]);      // h[i-1, j-1]
-                    const float X = fmaf(-0.5f * (aprev[n] + a_l), h_d, hprev[n]);
-                    float Y = fmaf(a, X, bu), S = bu, Ap = a;
-                    if (!(SND_WAVE_ABLATE & 8)) wave_scan3(Y, S, Ap);
-                    const float h = fmaf(Ap, in.x, Y);
-                    const float s = fmaf(Ap, in.y, S);
-                    acc = fmaf(cvt_raw(tp, cur.c[r][n]), fmaf(0.25f, bu, h - s), acc);
+                    float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
+                    unpack(cur.b[r][n], bu);
+                    unpack(cur.c[r][n], cv);
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) {
+                        a[k] = fast_exp2(fmaf(dl[k], A2[n], ld));
+                        bu[k] = ((NS == 4 && n >= N) ? 0.f : bu[k]) * du[k];
+                    }
+                    const float a_l = from_prev_lane(a[CPL - 1], in.z);                // a[i, j-1] of the lane's first column
+                    const float h_d = from_prev_lane(hprev[n][CPL - 1], hdiag[n]);     // h[i-1, j-1]
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) {
+                        const float al = k == 0 ? a_l : a[k > 0 ? k - 1 : 0], hd = k == 0 ? h_d : hprev[n][k > 0 ? k - 1 : 0];
+                        const float X = fmaf(-0.5f * (aprev[n][k] + al), hd, hprev[n][k]);
+                        y[k] = fmaf(a[k], X, bu[k]);
+                    }
+                    if (SND_WAVE_ABLATE & 8) {
+#pragma unroll
+                        for (int k = 0; k < CPL; ++k) { h[k] = y[k]; s[k] = bu[k]; }
+                    } else {
+                        wave_row_solve<CPL>(a, y, bu, in.x, in.y, h, s);
+                    }
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) {
+                        acc[k] = fmaf(cv[k], fmaf(0.25f, bu[k], h[k] - s[k]), acc[k]);
+                        hprev[n][k] = h[k];
+                        aprev[n][k] = a[k];
+                    }
                     hdiag[n] = in.x;
-                    hprev[n] = h;
-                    aprev[n] = a;
-                    if (!(SND_WAVE_ABLATE & 32) && hands_over && lane == 63) sHO[step & 1][w + 1][r % RD][n] = make_float4(h, s, a, 0.f);
+                    if (!(SND_WAVE_ABLATE & 32) && hands_over && lane == 63) sHO[step & 1][w + 1][r % RD][n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
                     if (SAVE && lane == r) { ch[n] = in.x; cs[n] = in.y; ca[n] = in.z; }
                 }
-                if (jin && (!(SND_WAVE_ABLATE & 1) || acc == 1234.5f)) stg_b(outb, oo, fmaf(Dv, u, acc));
+                if (jin && (!(SND_WAVE_ABLATE & 1) || acc[0] == 1234.5f)) {
+                    float o[CPL];
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k) o[k] = fmaf(Dv, u[k], acc[k]);
+                    if (CPL == 2 && fh) { const float t = o[0]; o[0] = o[CPL - 1]; o[CPL - 1] = t; }
+                    wave_st<OutT, CPL, VEC>(outb, oo, o);
+                }
                 oo += OhB;
             }
             if (multi && r % RD == RD - 1) { if (!(SND_WAVE_ABLATE & 2)) lds_barrier(); ++step; }
@@ -166,8 +221,11 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         for (int n = 0; n < NS; ++n) {
             if ((NS != 4 || n < N) && !(SND_WAVE_ABLATE & 16)) {
                 float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
-                __builtin_nontemporal_store(hprev[n], dst);
-                __builtin_nontemporal_store(aprev[n], dst + wg.Wp);
+#pragma unroll
+                for (int k = 0; k < CPL; ++k) {
+                    __builtin_nontemporal_store(hprev[n][k], dst + k);
+                    __builtin_nontemporal_store(aprev[n][k], dst + wg.Wp + k);
+                }
             }
         }
         // column checkpoints: lanes 0..R-1 hold what entered the segment on the band's rows
@@ -197,24 +255,43 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
 }
 
-template <typename T, int NS>
-static int launch_wave_fwd_ns(const snd_fwd_params &p, hipStream_t stream) {
+// Whether every row of a tensor starts at a multiple of `bytes` (so that a lane's CPL elements come with one access)
+static inline bool wave_aligned(const void *ptr, int64_t esz, int bytes, std::initializer_list<int64_t> strides) {
+    if ((uintptr_t)ptr % bytes) return false;
+    for (int64_t st : strides)
+        if ((st * esz) % bytes) return false;
+    return true;
+}
+
+template <typename T, int NS, int CPL, bool VEC>
+static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.shape;
-    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, sh.dstate);
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
     const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
-    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true, true>), grid, block, 0, stream, p, wg);
-    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, true, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
-    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false, true>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, false, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
+    constexpr bool F = std::is_same<T, float>::value;
+    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true>), grid, block, 0, stream, p, wg);
+    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F>), grid, block, 0, stream, p, wg);
+    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
 template <typename T>
 int launch_wave_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
-    const int N = p.shape.dstate;
-    return N == 1 ? launch_wave_fwd_ns<T, 1>(p, stream) : N == 2 ? launch_wave_fwd_ns<T, 2>(p, stream)
-                                                                  : launch_wave_fwd_ns<T, 4>(p, stream);
+    const snd_shape &sh = p.shape;
+    const int N = sh.dstate;
+    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    if (wg.cpl == 2) {                               // (N = 1 only)
+        const int e = (int)sizeof(T), oe = p.out_dtype == SND_F32 ? 4 : e;
+        const bool vec = wave_aligned(p.u, e, 2 * e, {p.u_batch_stride, p.u_d_stride, p.u_h_stride}) &&
+                         wave_aligned(p.delta, e, 2 * e, {p.delta_batch_stride, p.delta_d_stride, p.delta_h_stride}) &&
+                         wave_aligned(p.B, e, 2 * e, {p.B_batch_stride, p.B_group_stride, p.B_dstate_stride, p.B_h_stride}) &&
+                         wave_aligned(p.C, e, 2 * e, {p.C_batch_stride, p.C_group_stride, p.C_dstate_stride, p.C_h_stride}) &&
+                         wave_aligned(p.out, oe, 2 * oe, {p.out_batch_stride, p.out_d_stride, p.out_h_stride});
+        return vec ? launch_wave_fwd_v<T, 1, 2, true>(p, wg, stream) : launch_wave_fwd_v<T, 1, 2, false>(p, wg, stream);
+    }
+    return N == 1 ? launch_wave_fwd_v<T, 1, 1, true>(p, wg, stream) : N == 2 ? launch_wave_fwd_v<T, 2, 1, true>(p, wg, stream)
+                                                                              : launch_wave_fwd_v<T, 4, 1, true>(p, wg, stream);
 }
 
 }  // namespace snd

@@ -27,6 +27,12 @@ SHAPES = [
     (3, 12, 14, 14, 4, 4, None, torch.bfloat16),
     (1, 4, 25, 90, 2, 2, None, torch.float16),
     (2, 48, 56, 56, 1, 4, None, torch.float32),      # stage-1 plane, d_state = 1
+    # one state and an even width above 64: two neighbouring columns per lane
+    (1, 4, 19, 66, 1, 2, None, torch.float32),       # 33 lanes of one wave
+    (1, 8, 17, 130, 1, 4, None, torch.float32),      # second segment holds one lane
+    (2, 8, 33, 256, 1, 4, 4, torch.bfloat16),        # two full segments, shared delta groups
+    (1, 4, 12, 1024, 1, 1, None, torch.float16),     # the widest plane: eight segments of 128 columns
+    (1, 8, 70, 200, 1, 4, None, torch.bfloat16),
 ]
 
 
@@ -140,8 +146,45 @@ def test_wavefront_shared_u_and_second_backward(gpu_device):
 
 
 def test_wavefront_refuses_what_it_does_not_cover(gpu_device):
-    d = O.make_inputs(1, 4, 8, 600, N=1, K=1, seed=1)
+    d = O.make_inputs(1, 4, 8, 601, N=1, K=1, seed=1)       # odd width above 512: one column per lane, nine segments
     t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
     f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], None, None, False, True, None, True, capi.SCHED_WAVEFRONT)
     assert f.plan.auto_schedule != capi.SCHED_WAVEFRONT
     assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -2
+
+
+@pytest.mark.parametrize("dtype,dirs", [(torch.float32, capi.DIR_TOPLEFT), (torch.bfloat16, capi.DIR_CORNERS), (torch.float32, capi.DIR_CORNERS)])
+def test_wavefront_two_columns_per_lane_unaligned_and_flipped(gpu_device, dtype, dirs):
+    """One state, even width: rows that do not start at a multiple of two elements (odd row pitch: every lane's
+    pair is loaded element by element) and column-reversed groups, against the tile kernels and the oracle."""
+    Bt, Dm, H, W, N, K = 1, 8, 21, 150, 1, 4
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=17)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+
+    def padded(x):                                    # same values, row pitch W + 1
+        buf = torch.zeros(*x.shape[:-1], W + 1, device=x.device, dtype=dtype)
+        buf[..., :W] = x.to(dtype)
+        return buf[..., :W]
+    res = {}
+    for name, mk in (("pitch", padded), ("dense", lambda x: x.to(dtype).contiguous())):
+        u, delta, B, C = (mk(t[k]) for k in ("u", "delta", "B", "C"))
+        dout = mk(t["dout"]).float() if name == "dense" else padded(t["dout"]).float()
+        args = (u, delta, t["A"], B, C, t["D"], t["delta_bias"])
+        for sched in (capi.SCHED_WAVEFRONT, capi.SCHED_PLANE):
+            f = capi.FwdCall(*args, True, True, None, True, sched, dirs)
+            f.launch()
+            b = capi.BwdCall(*args, dout, f.x, f.x_v, True, None, f.x_sd, sched, dirs)
+            b.launch()
+            torch.cuda.synchronize()
+            res[(name, sched)] = [f.out, b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias]
+    half = dtype != torch.float32
+    ref = res[("dense", capi.SCHED_PLANE)]
+    for key in (("pitch", capi.SCHED_WAVEFRONT), ("dense", capi.SCHED_WAVEFRONT), ("pitch", capi.SCHED_PLANE)):
+        for nm, a, w_ in zip(["out"] + NAMES, res[key], ref):
+            tol = 1e-2 if (half and nm in ("du", "ddelta")) else 1e-4
+            e = relerr(a.float().cpu().numpy(), w_.float().cpu().numpy())
+            assert e <= tol, (key, nm, e)
+    if dirs == capi.DIR_TOPLEFT:
+        r = {k: t[k].to(dtype).float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+        refo = OC.fwd(r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"], True, None, real="f64")
+        assert relerr(res[("pitch", capi.SCHED_WAVEFRONT)][0].cpu().numpy(), refo) <= 1e-4
