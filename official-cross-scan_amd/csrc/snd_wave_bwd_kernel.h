@@ -181,9 +181,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     // one band from `cur`, with the loads of the band above issued into `nxt` first
     auto do_band = [&](In &cur, In &nxt, int band) {
-        if (PF) load_band(nxt, max(band - 1, 0));       // unconditionally (band 0 once more): a skipped load would leave two paths with
-                                                        // different numbers of loads in flight, and the waits follow the smaller
-        else load_band(cur, band);
+        if (!PF) load_band(cur, band);
         const int i0 = band * R;
 
         // ---- recompute h, s on the band's rows (with the columns); results back in mirrored order.
@@ -272,6 +270,13 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                 }
             }
         }
+
+        // The loads of the band above are issued here, between the two phases, not at the top of the band: a wave
+        // can have 63 memory instructions in flight, and at the top of a band the 2 stores and 2N atomics per row of
+        // the sweep just finished still are (40 loads on top of them stalled the issue for a quarter of the kernel);
+        // here they have had the whole recomputation to complete.  Unconditionally (band 0 once more): a skipped
+        // load would leave two paths with different numbers of loads in flight, and the waits follow the smaller.
+        if (PF) load_band(nxt, max(band - 1, 0));
 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
         const int rows = min(R, H - i0);             // rows of this band inside the plane
