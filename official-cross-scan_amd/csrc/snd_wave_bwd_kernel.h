@@ -28,6 +28,11 @@
 #include <type_traits>
 #include "snd_device.h"
 
+// Timing studies only (-DSND_WAVE_ABLATE=<bits>, results wrong): 64 no dB / dC atomics, 128 no du / ddelta stores.
+#ifndef SND_WAVE_ABLATE
+#define SND_WAVE_ABLATE 0
+#endif
+
 namespace snd {
 
 __device__ __forceinline__ void wave_glb_add(float *p, float v) {
@@ -341,7 +346,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         ya[t] = dbu * dlu[t];                                          // dB, dC contributions (reusing the arrays)
                         ys[t] = dov[t] * fmaf(0.25f, bu[t], hs);
                     }
-                    if (jin && live) {
+                    if (jin && live && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
 #pragma unroll
                         for (int e = 0; e < CPL; ++e) {                                // memory order
                             const int t = fh ? e : CPL - 1 - e;
@@ -368,8 +373,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         float t_ = duv[0]; duv[0] = duv[CPL - 1]; duv[CPL - 1] = t_;
                         t_ = ddl[0]; ddl[0] = ddl[CPL - 1]; ddl[CPL - 1] = t_;
                     }
-                    wave_st<T, CPL, VEC>(dub, og, duv);
-                    wave_st<T, CPL, VEC>(ddb, og, ddl);
+                    if (!(SND_WAVE_ABLATE & 128) || duv[0] == 1234.5f) {
+                        wave_st<T, CPL, VEC>(dub, og, duv);
+                        wave_st<T, CPL, VEC>(ddb, og, ddl);
+                    }
                 }
                 og -= WB;
                 o4 -= W4;
