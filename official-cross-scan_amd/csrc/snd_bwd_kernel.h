@@ -69,6 +69,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;
+    // Pitches in floats, chosen for the 32 four-byte banks of LDS (a pitch of 64 would put every channel of a
+    // wave in the same bank).  PCH: pixel arrays that the sweep reads as one float4 per channel (all lanes of a
+    // channel the same address), so the channels of a wave must start 4 banks apart.  PCS: pixel arrays that
+    // only the staging and the per-pixel epilogue touch, lane n of a channel at element n, so a channel takes NP
+    // consecutive banks.  NSD: the dB/dC partial sums, which the 16-lane row q of a wave writes at element q of
+    // a state's tile row, so states must start 2 (16 states) or 4 banks apart.
+    constexpr int PCH = kTile + (NP == 16 ? 8 : 4);
+    constexpr int PCS = kTile + NP;
+    constexpr int NSD = NP == 16 ? kTile + 2 : kTile + 4;
     constexpr int NBC = 4;
     constexpr int NPX = kTile / NP;
     constexpr int HG = 10, DLP = HG * HG;           // delta' on the tile plus a one-cell halo
@@ -80,16 +89,16 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     extern __shared__ __align__(16) float smem[];
     float *sB = smem;                               // [NP][NSTR]
     float *sC = sB + NP * NSTR;
-    float *sdB = sC + NP * NSTR;                    // [NPART][NP][NSTR]
-    float *sdC = sdB + NPART * NP * NSTR;
-    float *sDl = sdC + NPART * NP * NSTR;           // [CB][DLP]
-    float *sDu = sDl + CB * DLP;                    // [CB][kTile] delta' * u
-    float *sU = sDu + CB * kTile;
-    float *sDo = sU + CB * kTile;                   // dout
-    float *sSg = sDo + CB * kTile;                  // d softplus / d raw
-    float *sQ = sSg + CB * kTile;                   // sum_n dbu*B
-    float *sP = sQ + CB * kTile;                    // sum_n A*da*a
-    float *sRed = sP + CB * kTile;                  // [WPB]
+    float *sdB = sC + NP * NSTR;                    // [NPART][NP][NSD]
+    float *sdC = sdB + NPART * NP * NSD;
+    float *sDl = sdC + NPART * NP * NSD;            // [CB][DLP]
+    float *sDu = sDl + CB * DLP;                    // [CB][PCH] delta' * u
+    float *sU = sDu + CB * PCH;                     // [CB][PCS]
+    float *sDo = sU + CB * PCS;                     // dout
+    float *sSg = sDo + CB * PCH;                    // [CB][PCS] d softplus / d raw
+    float *sQ = sSg + CB * PCS;                     // sum_n dbu*B
+    float *sP = sQ + CB * PCH + 4;                  // sum_n A*da*a (4 banks off sQ: a wave writes both in one instruction)
+    float *sRed = sP + CB * PCH;                    // [WPB]
 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
@@ -186,12 +195,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + (PIPE ? ((int64_t)cc * N + nn) * 2 : lane_off);
 
     const float *myDl = sDl + cl * DLP;
-    const float *myDu = sDu + cl * kTile;
-    const float *myDo = sDo + cl * kTile;
+    const float *myDu = sDu + cl * PCH;
+    const float *myDo = sDo + cl * PCH;
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
-    float *mydB = sdB + wave * NP * NSTR + n * NSTR;
-    float *mydC = sdC + wave * NP * NSTR + n * NSTR;
+    float *mydB = sdB + wave * NP * NSD + n * NSD;
+    float *mydC = sdC + wave * NP * NSD + n * NSD;
     const int qrow = (tid & 63) >> 4;               // 16-lane row of this lane inside its wave
 
     // ---- register staging of one tile's raw inputs (loaded at the start of the tile, then committed to LDS)
@@ -258,10 +267,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const float dl = softplus ? softplus20(raw, dsp) : raw;
             if (TE == 8 || ((pp >> 3) < TE && (pp & 7) < TE))     // slots beyond the tile belong to the halo ring
                 sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1] = dl;
-            sDu[cl * kTile + pp] = dl * qu[k];
-            sU[cl * kTile + pp] = qu[k];
-            sDo[cl * kTile + pp] = qdo[k];
-            sSg[cl * kTile + pp] = dsp;
+            sDu[cl * PCH + pp] = dl * qu[k];
+            sU[cl * PCS + pp] = qu[k];
+            sDo[cl * PCH + pp] = qdo[k];
+            sSg[cl * PCS + pp] = dsp;
         }
 #pragma unroll
         for (int k = 0; k < NHK; ++k) {
@@ -493,15 +502,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         // q[0..1], q[2..3], quads 2,3 with pp_[0..1], pp_[2..3]
                         group_scatter8(q[0], q[1], q[2], q[3], pp_[0], pp_[1], pp_[2], pp_[3]);
                         if ((n & 3) == 0) {
-                            float *dst = ((n & 8) ? sP : sQ) + cl * kTile + r * kCkX + C0 + ((n >> 1) & 2);
+                            float *dst = ((n & 8) ? sP : sQ) + cl * PCH + r * kCkX + C0 + ((n >> 1) & 2);
                             *(float2 *)dst = make_float2(q[0], q[1]);
                         }
                     } else {
                         group_sum4<NP>(q[0], q[1], q[2], q[3]);
                         group_sum4<NP>(pp_[0], pp_[1], pp_[2], pp_[3]);
                         if (n == 0) {
-                            *(float4 *)(sQ + cl * kTile + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
-                            *(float4 *)(sP + cl * kTile + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
+                            *(float4 *)(sQ + cl * PCH + r * kCkX + C0) = make_float4(q[0], q[1], q[2], q[3]);
+                            *(float4 *)(sP + cl * PCH + r * kCkX + C0) = make_float4(pp_[0], pp_[1], pp_[2], pp_[3]);
                         }
                     }
                     {
@@ -550,9 +559,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-                const float qv = sQ[cl * kTile + pp], pv = sP[cl * kTile + pp];
+                const float qv = sQ[cl * PCH + pp], pv = sP[cl * PCH + pp];
                 const float dl = sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1];
-                const float uv = sU[cl * kTile + pp], dov = sDo[cl * kTile + pp], sg = sSg[cl * kTile + pp];
+                const float uv = sU[cl * PCS + pp], dov = sDo[cl * PCH + pp], sg = sSg[cl * PCS + pp];
                 const float duv = fmaf(Dv, dov, dl * qv);
                 const float ddl = fmaf(uv, qv, pv) * sg;
                 if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W) {
@@ -576,8 +585,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     float tb = 0.f, tc = 0.f;
 #pragma unroll
                     for (int w = 0; w < NPART; ++w) {
-                        tb += sdB[w * NP * NSTR + sn * NSTR + px];
-                        tc += sdC[w * NP * NSTR + sn * NSTR + px];
+                        tb += sdB[w * NP * NSD + sn * NSD + px];
+                        tc += sdC[w * NP * NSD + sn * NSD + px];
                     }
                     if (in && sn < N) {
                         glb_add((float *)((char *)dBg + sn * HW4 + o), tb);
@@ -618,7 +627,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 
 // Dynamic LDS of one backward block (more than the 64 KB a kernel gets without asking).
 template <int NP> constexpr size_t bwd_lds_bytes() {
-    return sizeof(float) * ((2 + 2 * (NP / 4)) * NP * (kTile + 4) + 16 * 100 + 6 * 16 * kTile + NP / 4);
+    constexpr int PCH = kTile + (NP == 16 ? 8 : 4), PCS = kTile + NP, NSD = NP == 16 ? kTile + 2 : kTile + 4;
+    return sizeof(float) * (2 * NP * (kTile + 4) + 2 * (NP / 4) * NP * NSD + 16 * 100 + 16 * (4 * PCH + 2 * PCS) + 4 + NP / 4);
 }
 // Raise the dynamic LDS limit of every backward instantiation of one input dtype on the current device.
 // hipFuncSetAttribute is not stream-ordered and must not run under a stream capture, which is why it is

@@ -38,12 +38,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     constexpr int NBC = 4;                          // B/C elements per thread per tile
     constexpr int NPX = kTile / NP;                 // pixels per thread per tile
     constexpr int DLP = kTile + kCkX;               // delta' tile with one halo row above
+    // per-channel pitch of the pixel arrays: 8 mod 32 banks, so that the channels a wave reads at one tile offset
+    // sit in different banks (a pitch of 64 put them all in the same one)
+    constexpr int PCH = kTile + 8;
 
     __shared__ __align__(16) float sB[NP * NSTR];
     __shared__ __align__(16) float sC[NP * NSTR];
     __shared__ __align__(16) float sDl[CB * DLP];
-    __shared__ __align__(16) float sDu[CB * kTile];  // delta' * u
-    __shared__ __align__(16) float sY[CB * kTile];   // sum_n C*(h - s)
+    __shared__ __align__(16) float sDu[CB * PCH];    // delta' * u
+    __shared__ __align__(16) float sY[CB * PCH];     // sum_n C*(h - s)
     // The bu/4 term of the output, sum_n C*B*delta'*u/4, is delta'*u times a per-pixel sum that all
     // channels share: S/4 = sum_n B*C / 4 is built once per tile (per-wave partial sums at staging, added
     // up by one wave) instead of one multiply-add per state cell.
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     float *xs = SAVE ? p.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off : nullptr;
 
     const float *myDl = sDl + cl * DLP;
-    const float *myDu = sDu + cl * kTile;
+    const float *myDu = sDu + cl * PCH;
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
 
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             const float raw = q.qdl[k] + bias;
             const float dl = softplus ? softplus20(raw, dsp) : raw;
             sDl[cl * DLP + kCkX + pp] = dl;
-            sDu[cl * kTile + pp] = dl * q.qu[k];
+            sDu[cl * PCH + pp] = dl * q.qu[k];
             dukeep[k] = Dv * q.qu[k];
         }
 #pragma unroll
@@ -351,12 +354,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 if (NP == 16) {
                     // sum over the channel's 16 states; quad q of the lane group ends with columns 2q, 2q+1
                     group_scatter8(y[0], y[1], y[2], y[3], y[4], y[5], y[6], y[7]);
-                    if ((n & 3) == 0) *(float2 *)(sY + cl * kTile + r * kCkX + (n >> 1)) = make_float2(y[0], y[1]);
+                    if ((n & 3) == 0) *(float2 *)(sY + cl * PCH + r * kCkX + (n >> 1)) = make_float2(y[0], y[1]);
                 } else {
                     group_sum4<NP>(y[0], y[1], y[2], y[3]);
                     group_sum4<NP>(y[4], y[5], y[6], y[7]);
                     if (n == 0) {
-                        float4 *dst = (float4 *)(sY + cl * kTile + r * kCkX);
+                        float4 *dst = (float4 *)(sY + cl * PCH + r * kCkX);
                         dst[0] = make_float4(y[0], y[1], y[2], y[3]);
                         dst[1] = make_float4(y[4], y[5], y[6], y[7]);
                     }
@@ -402,7 +405,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                     const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                     if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
                         st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype,
-                                 fmaf(sDu[cl * kTile + pp], sS[pp], sY[cl * kTile + pp] + dukeep[k]));
+                                 fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]));
                 }
                 return;
             }
@@ -410,7 +413,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 if ((pp >> 3) < TE && (pp & 7) < TE)
-                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = fmaf(sDu[cl * kTile + pp], sS[pp], sY[cl * kTile + pp] + dukeep[k]);
+                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
