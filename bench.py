@@ -8,9 +8,13 @@ reference's fwd/bwd bindings would pay them) on synthetic inputs already residen
 Prints ONE JSON line.  `value` is the algorithmic HBM rate of the whole step:
     bytes = (2eP + 2eQ + 4P) + (4eP + 4eQ + 4P),  P = B*D*H*W, Q = B*K*N*H*W, e = input bytes
 (compulsory tensor I/O only) divided by the mean step time.  `roofline` is the same figure for the
-dominant kernel alone (the backward), from HIP events around its launches on the launch stream;
-`cpu_baseline` times the C restatement of the reference recurrence (oracle/) on the host cores on
-a bounded sample of the same workload.
+dominant kernel alone (the backward), from HIP events around its launches on the launch stream, with
+a second leg beside it: vector-ALU wave-instructions per second against 1024 SIMDs x clock / 4 cycles.
+The instruction count, the clock and the HBM traffic per launch are counter readings that a timed run
+cannot take; they come from the committed rocprofv3 summary of the same workload under profiles/
+(named in `roofline.counters_from`), while every duration is measured live.  `roofline.bound` names
+the leg with the higher fraction.  `cpu_baseline` times the C restatement of the reference recurrence
+(oracle/) on the host cores on a bounded sample of the same workload.
 """
 import argparse
 import json
@@ -101,16 +105,25 @@ def cpu_baseline(workload, budget_s=20.0):
             "ms_per_step_extrapolated": round(1e3 * t * (Bt * Dm) / (sb * sd), 1)}
 
 
-def measured_traffic(workload):
-    """HBM bytes per launch of the dominant kernel, and the fraction of cycles its SIMDs spend
-    issuing vector ALU instructions, from the committed rocprofv3 --pmc summary."""
-    path = os.path.join(ROOT, "profiles", "bwd_kernel_%s_pmc.txt" % workload)
+N_SIMD = 1024                   # 256 CUs x 4 SIMDs; a SIMD issues one wave-wide VALU instruction per 4 cycles
+
+
+def profile_counters(workload):
+    """Counter readings of the dominant kernel (the backward) from the committed rocprofv3 summary of
+    this workload: kernel name, HBM bytes per launch, VALU wave-instructions per launch, shader clock
+    under this load.  A timed run cannot read counters; durations are always measured live."""
+    rel = os.path.join("profiles", "bwd_kernel_%s_pmc.txt" % workload)
+    path = os.path.join(ROOT, rel)
     if not os.path.exists(path):
-        return None, None
+        return None
     text = open(path).read()
-    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", text)
-    v = re.search(r"backward [0-9.e]+ / \([0-9.e]+ / 2\) = ([0-9.]+)", text)
-    return (float(m.group(1)) if m else None), (float(v.group(1)) if v else None)
+    out = {"file": rel}
+    for key in ("dominant_kernel", "avg_ns", "traffic_bytes_per_launch", "valu_insts_per_launch", "clock_ghz"):
+        m = re.search(r"^%s:\s*(.+)$" % key, text, flags=re.M)
+        if not m:
+            return None
+        out[key] = m.group(1).strip() if key == "dominant_kernel" else float(m.group(1))
+    return out
 
 
 def main():
@@ -120,8 +133,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
-    ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands"],
-                    help="block mapping: chosen by shape (default), one block per plane chunk, or pipelined row strips")
+    ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
+                    help="kernel family and block mapping: chosen by shape (default), one block per plane chunk, "
+                         "pipelined row strips / bands, or the row-segment wavefront kernels (1-4 states)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -144,7 +158,7 @@ def main():
     import selective_nd_scan as snd
     from selective_nd_scan import capi
 
-    sched = {"auto": 0, "plane": 1, "strips": 2, "bands": 3}[args.schedule]
+    sched = {"auto": 0, "plane": 1, "strips": 2, "bands": 3, "wavefront": 4}[args.schedule]
     snd.set_schedule(sched)
     Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
     dtype = getattr(torch, dtn)
@@ -183,23 +197,39 @@ def main():
 
     value = (fb + bb) / (ms * 1e-3) / 1e9
     achieved = bb / (kb_ms * 1e-3) / 1e9
-    traffic, valu_frac = measured_traffic(args.workload)
+    st, plan = capi.make_plan(capi.make_shape(u, delta, A, B))
+    capi.check(st)
+    used = sched if sched else plan.auto_schedule
+    kernel = "snd::wave_bwd_kernel" if used == capi.SCHED_WAVEFRONT else "snd::bwd_kernel"
+    roof = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_launch": bb,
+            "kernel_ms": round(kb_ms, 4)}
+    pc = profile_counters(args.workload) if args.schedule == "auto" else None
+    if pc and pc["dominant_kernel"].startswith(kernel + "<"):
+        # counters from the committed profile of this workload; the rate uses the duration measured here
+        peak_valu = N_SIMD * pc["clock_ghz"] * 1e9 / 4.0
+        rate_valu = pc["valu_insts_per_launch"] / (kb_ms * 1e-3)
+        roof.update({"traffic": pc["traffic_bytes_per_launch"], "counters_from": pc["file"],
+                     "profile_kernel_ms": round(pc["avg_ns"] * 1e-6, 4),
+                     "valu": {"insts_per_launch": pc["valu_insts_per_launch"], "clock_ghz": pc["clock_ghz"],
+                              "achieved": round(rate_valu / 1e9, 2), "peak": round(peak_valu / 1e9, 2),
+                              "unit": "G wave-instructions/s"},
+                     "frac_valu": round(rate_valu / peak_valu, 4)})
+        if roof["frac_valu"] > roof["frac"]:
+            roof["bound"] = "valu"
     rec = {
         "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        # arithmetic type of the recurrence and of every accumulation, whatever the I/O dtype of the workload
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: selective_nd_scan fwd+bwd, B=%d D=%d H=%d W=%d N=%d K=%d, %s inputs, fp32 state"
                                % (args.workload, Bt, Dm, H, W, N, K, dtn),
-                   "schedule": args.schedule, "algorithmic_bytes": fb + bb, "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+                   "io_dtype": dtn, "schedule": args.schedule, "algorithmic_bytes": fb + bb, "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
                    "pixels_per_s": round(Bt * Dm * H * W / (ms * 1e-3), 1),
                    "state_cells_per_s": round(Bt * Dm * H * W * N / (ms * 1e-3), 1),
                    "kernel_ms": {"fwd": round(kf_ms, 4), "bwd": round(kb_ms, 4)},
                    "kernel_only_GBs": round((fb + bb) / ((kf_ms + kb_ms) * 1e-3) / 1e9, 2)},
-        "roofline": {"bound": "hbm", "kernel": "snd::bwd_kernel", "achieved": round(achieved, 2),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": traffic, "algorithmic_bytes_per_launch": bb,
-                     # the kernel is bound by vector-ALU issue, not by HBM: fraction of SIMD cycles issuing VALU
-                     "valu_issue_frac": valu_frac},
+        "roofline": roof,
     }
     if not args.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(args.workload)
