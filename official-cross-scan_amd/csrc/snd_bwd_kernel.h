@@ -206,7 +206,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // ---- register staging of one tile's raw inputs (loaded at the start of the tile, then committed to LDS)
     float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
     auto prefetch = [&](int I, int J) {
-        const int r0 = I * TE, j0 = J * TE;
+        const int r0 = (SND_TILE_ABLATE & 2) ? 0 : I * TE, j0 = (SND_TILE_ABLATE & 2) ? 0 : J * TE;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
             float Gd[kCkX];                                        // G of the row below
             if (I > 0) {
-                const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+                const float *src = xv + ((SND_TILE_ABLATE & 8) ? 1 : ((int64_t)(I - 1) * geo.nCX + J)) * DN8;
                 const float4 v0 = *(const float4 *)src, v1 = *(const float4 *)(src + DN4);
                 hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
                 hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
@@ -317,8 +317,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
             if (J > 0) {
-                const float *sh_ = xh + ((int64_t)(J - 1) * geo.nCY + I) * DN8;
-                const float *ss_ = xs + ((int64_t)(J - 1) * geo.nCY + I) * DN8;
+                const float *sh_ = xh + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8;
+                const float *ss_ = xs + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8;
                 const float4 h0 = *(const float4 *)sh_, h1 = *(const float4 *)(sh_ + DN4);
                 const float4 s0 = *(const float4 *)ss_, s1 = *(const float4 *)(ss_ + DN4);
                 hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
@@ -568,8 +568,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     dD_acc = fmaf(dov, uv, dD_acc);
                     dbias_acc += ddl;
                     const uint32_t o = cGb + mad24(mrow(row), WB, mcol(col) * ESZ);
-                    stg_b(dub, o, duv);
-                    stg_b(ddb, o, ddl);
+                    if (!(SND_TILE_ABLATE & 4)) {
+                        stg_b(dub, o, duv);
+                        stg_b(ddb, o, ddl);
+                    } else {
+                        dD_acc += duv;              // keeps the values live
+                    }
                 }
             }
             }
@@ -588,9 +592,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         tb += sdB[w * NP * NSD + sn * NSD + px];
                         tc += sdC[w * NP * NSD + sn * NSD + px];
                     }
-                    if (in && sn < N) {
+                    if (in && sn < N && !(SND_TILE_ABLATE & 1)) {
                         glb_add((float *)((char *)dBg + sn * HW4 + o), tb);
                         glb_add((float *)((char *)dCg + sn * HW4 + o), tc);
+                    } else if (SND_TILE_ABLATE & 1) {
+                        dbias_acc += tb + tc;       // keeps the values live
                     }
                 }
             }

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto load_tile = [&](Stage &q, int I, int J) {
-        const int r0 = I * TE, j0 = J * TE;
+        const int r0 = (SND_TILE_ABLATE & 2) ? 0 : I * TE, j0 = (SND_TILE_ABLATE & 2) ? 0 : J * TE;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     // schedule; every strip of a pipelined band but its first)
     auto prefetch_xv = [&](int I, int J) {
         if ((!PIPE || I > I_begin) && I > 0 && geo.nCX > 1) {   // with one column tile the row comes from registers
-            const float *src = xv + ((int64_t)(I - 1) * geo.nCX + J) * DN8;
+            const float *src = xv + ((SND_TILE_ABLATE & 8) ? 1 : ((int64_t)(I - 1) * geo.nCX + J)) * DN8;
             const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + DN4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
             qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
@@ -373,8 +373,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
-                st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
-                st4_stream(dst + DN4, hup[4], hup[5], hup[6], hup[7]);
+                if (!(SND_TILE_ABLATE & 4)) {
+                    st4_stream(dst, hup[0], hup[1], hup[2], hup[3]);
+                    st4_stream(dst + DN4, hup[4], hup[5], hup[6], hup[7]);
+                }
                 if (PIPE && I + 1 == I_end && I + 1 < geo.nCY) {   // and the hand-over copy for the block of the strip below
                     float *ho = hrow + (int64_t)J * DN8;
 #pragma unroll
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             }
             const bool hands_over = PIPE && I + 1 == I_end && I + 1 < geo.nCY;
             if (hands_over) strip_stores_done();
-            if (lvalid && SAVE && J + 1 < geo.nCX) {   // column checkpoints: only if a tile follows
+            if (lvalid && SAVE && J + 1 < geo.nCX && !(SND_TILE_ABLATE & 4)) {   // column checkpoints: only if a tile follows
                 float *dh = xh + ((int64_t)J * geo.nCY + I) * DN8;
                 float *ds = xs + ((int64_t)J * geo.nCY + I) * DN8;
                 st4_stream(dh, hl[0], hl[1], hl[2], hl[3]);
@@ -403,7 +405,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 for (int k = 0; k < NPX; ++k) {
                     const int pp = n + NP * k;
                     const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-                    if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W)
+                    if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W && !(SND_TILE_ABLATE & 1))
                         st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype,
                                  fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]));
                 }
@@ -426,7 +428,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 for (int idx = tid; idx < CB * PER_CH; idx += 16 * NP) {
                     const int ch = idx / PER_CH, rr = (idx / QC) & 7, c32 = idx & (QC - 1);
                     const int row = r0 + rr;
-                    if (rr < TE && row < H && c32 < ncols && cbase + ch < cend) {
+                    if (rr < TE && row < H && c32 < ncols && cbase + ch < cend && !(SND_TILE_ABLATE & 1)) {
                         const uint32_t o = (uint32_t)(cbase + ch) * (uint32_t)p.out_d_stride * esz_out;
                         st_f32_b(outb, o + mad24(mrow(row), OhB, mcol(c0 + c32) << sh_out), p.out_dtype, sOut[ch * OCH + rr * OROW + c32]);
                     }
