@@ -139,7 +139,18 @@ typedef struct snd_fwd_params {
                                       the same channels (channel g*(dim/n_groups) + i reads u channel i):
                                       the CrossScan of one feature map without its n_groups copies.
                                       out, du and every other tensor keep their dim-wide layouts. */
-    int32_t reserved_;             /* set to 0 */
+    int32_t merge;                 /* 0: out is [batch, dim, nrows, ncols] (the reference's layout).
+                                      1: CrossMerge fused into the output stores: out is fp32
+                                      [batch, dim / n_groups, nrows, ncols], zero-filled by the caller, and
+                                      channel g*(dim/n_groups) + i adds merge_weights[that channel] * (its result)
+                                      to out channel i with a float atomic, so out ends as the weighted sum of
+                                      the n_groups results per feature (the summation order, hence the last
+                                      bits, vary from run to run).  out_dtype must be SND_F32; out strides
+                                      describe the merged tensor.  In snd_bwd_params.f it says that dout has
+                                      the merged shape (see there).  No counterpart in the reference kernel:
+                                      it is the fusion "with trainable weights" of README.md:45. */
+    const float *merge_weights;    /* [dim] fp32, one weight per (group, feature) in channel order, or null
+                                      (all ones: the plain CrossMerge sum).  Read only when merge = 1. */
 } snd_fwd_params;
 
 /* Replaces SSMParamsBwd (selective_scan_oflex.h:53-86). Gradient buffers are dense (contiguous):
@@ -152,10 +163,13 @@ typedef struct snd_fwd_params {
  *                                                 zero-fills, then casts to the input dtype
  *                                                 (host.cpp:398-399,432)
  *     dD [dim], ddelta_bias [dim] (per channel, host.cpp:403), dA_decay [1]: fp32, optional,
- *                                                 accumulated with atomics: caller zero-fills */
+ *                                                 accumulated with atomics: caller zero-fills
+ * With f.merge = 1 (fused CrossMerge) dout is the gradient of the merged output,
+ * [batch, dim / n_groups, nrows, ncols] with the dout strides describing that tensor; channel
+ * g*(dim/n_groups) + i reads dout channel i scaled by merge_weights[g*(dim/n_groups) + i]. */
 typedef struct snd_bwd_params {
     snd_fwd_params f;              /* inputs and saved state; f.out / f.out_dtype are ignored */
-    const void *dout;              /* [batch, dim, nrows, ncols], last dim contiguous */
+    const void *dout;              /* [batch, dim, nrows, ncols] (merged shape if f.merge), last dim contiguous */
     int32_t dout_dtype;            /* SND_F32 or shape.in_dtype (host.cpp:303) */
     int64_t dout_batch_stride, dout_d_stride, dout_h_stride;
     void *du, *ddelta;
@@ -163,6 +177,14 @@ typedef struct snd_bwd_params {
     float *dD, *ddelta_bias, *dA_decay;
     void *workspace;               /* plan.bwd_workspace_bytes bytes, 16-byte aligned */
     int64_t workspace_bytes;
+    float *dmerge;                 /* [dim] fp32, optional, accumulated with atomics: caller zero-fills.
+                                      With f.merge = 1 channel c receives
+                                          merge_weights[c] * d loss / d merge_weights[c]
+                                        = sum over batch and pixels of  merge_weights[c] * dout * (result of channel c)
+                                      (every gradient of the op is linear in the weighted dout, so the kernel
+                                      carries the weight through; the caller divides by merge_weights[c], and
+                                      handles a weight of exactly 0 on the unfused path).  Ignored when
+                                      f.merge = 0. */
 } snd_bwd_params;
 
 /* Library / ABI version (major*100 + minor). */

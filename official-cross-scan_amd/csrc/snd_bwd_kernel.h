@@ -31,10 +31,6 @@
 
 namespace snd {
 
-__device__ __forceinline__ void glb_add(float *p, float v) {
-    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Sum two sets of four values over the four 16-lane rows of a wave (its four channels when a row
 // holds the 16 states of one channel): a reduce-scatter, row q of the wave ends with the totals of
 // b[q] (in b0) and c[q] (in c0).  v_permlane32_swap exchanges the upper 32 lanes of its first
@@ -172,7 +168,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // row pitches / state strides in bytes
     constexpr int ESZ = (int)sizeof(T);
     const uint32_t cUb = (uint32_t)(f.u_shared ? cc - g * rg : cc) * (uint32_t)f.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)f.delta_d_stride * ESZ;
-    const uint32_t cDob = ((uint32_t)cc * (uint32_t)p.dout_d_stride) << sh_do;
+    // fused CrossMerge: dout is the gradient of the merged output (one channel per feature, shared by the groups);
+    // the channel's weight is applied where dout is staged, and every gradient, being linear in dout, follows
+    const bool merge = f.merge != 0;
+    const float wm = merge && f.merge_weights ? f.merge_weights[cc] : 1.f;
+    const uint32_t cDob = ((uint32_t)(merge ? cc - g * rg : cc) * (uint32_t)p.dout_d_stride) << sh_do;
     const uint32_t cGb = (uint32_t)cc * (uint32_t)(H * W) * ESZ;      // du, ddelta
     const int BhB = (int)f.B_h_stride * ESZ, ChB = (int)f.C_h_stride * ESZ, UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ;
     const int DohB = (int)p.dout_h_stride << sh_do, WB = W * ESZ, W4 = W * 4;
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1] = dl;
             sDu[cl * PCH + pp] = dl * qu[k];
             sU[cl * PCS + pp] = qu[k];
-            sDo[cl * PCH + pp] = qdo[k];
+            sDo[cl * PCH + pp] = wm * qdo[k];
             sSg[cl * PCS + pp] = dsp;
         }
 #pragma unroll
@@ -291,6 +291,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float dA_acc = 0.f, dec_acc = 0.f;              // per lane: sum delta'*da*a, sum da*a
     const bool want_decay = p.dA_decay != nullptr;  // the second sum is skipped when nobody reads it
     float dD_acc = 0.f, dbias_acc = 0.f;            // per thread, for its channel's staged pixels
+    // Fused CrossMerge: weight * d(weight) = <weighted dout, result of the channel>.  The result is linear in u
+    // (D*u plus a recurrence that is linear in B*delta'*u), so this inner product equals <du, u>: summed per pixel
+    // beside dD, at no cost in the sweep.
+    float dw_acc = 0.f;
 
     for (int I = I_hi; I >= I_lo; --I) {
         const int r0 = I * TE;
@@ -566,6 +570,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 const float ddl = fmaf(uv, qv, pv) * sg;
                 if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W) {
                     dD_acc = fmaf(dov, uv, dD_acc);
+                    dw_acc = fmaf(duv, uv, dw_acc);
                     dbias_acc += ddl;
                     const uint32_t o = cGb + mad24(mrow(row), WB, mcol(col) * ESZ);
                     if (!(SND_TILE_ABLATE & 4)) {
@@ -615,6 +620,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     if (n == 0 && cvalid) {
         if (p.dD) glb_add(p.dD + c, dD_acc);
         if (p.ddelta_bias) glb_add(p.ddelta_bias + c, dbias_acc);
+    }
+    if (merge && p.dmerge) {
+        dw_acc = group_sum<NP>(dw_acc);
+        if (n == 0 && cvalid) glb_add(p.dmerge + c, dw_acc);
     }
     if (p.dA_decay) {
         float v = lvalid ? dec_acc : 0.f;

@@ -134,7 +134,7 @@ int check_fwd(const snd_fwd_params &p, bool need_state) {
 
 extern "C" {
 
-int snd_version(void) { return 200; }
+int snd_version(void) { return 210; }
 
 const char *snd_status_string(int status) {
     switch (status) {
@@ -197,8 +197,10 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (!params->out) return SND_ERR_NULL;
     if (params->out_dtype != SND_F32 && params->out_dtype != params->shape.in_dtype) return SND_ERR_DTYPE;
-    if (!fits32(params->shape.dim, params->out_d_stride, params->shape.nrows, params->out_h_stride, params->shape.ncols,
-                esize(params->out_dtype)))
+    if (params->merge != 0 && params->merge != 1) return SND_ERR_SHAPE;
+    if (params->merge && params->out_dtype != SND_F32) return SND_ERR_DTYPE;   // accumulated with float atomics
+    if (!fits32(params->merge ? params->shape.dim / params->shape.n_groups : params->shape.dim, params->out_d_stride,
+                params->shape.nrows, params->out_h_stride, params->shape.ncols, esize(params->out_dtype)))
         return SND_ERR_STRIDE;
     if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_WAVEFRONT) return SND_ERR_SHAPE;
     if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
@@ -241,8 +243,9 @@ static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
     if (st != SND_OK) return st;
     if (params->f.schedule < SND_SCHED_AUTO || params->f.schedule > SND_SCHED_WAVEFRONT) return SND_ERR_SHAPE;
     if (params->f.directions != SND_DIR_TOPLEFT && params->f.directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
-    if (!fits32(params->f.shape.dim, params->dout_d_stride, params->f.shape.nrows, params->dout_h_stride,
-                params->f.shape.ncols, esize(params->dout_dtype)))
+    if (params->f.merge != 0 && params->f.merge != 1) return SND_ERR_SHAPE;
+    if (!fits32(params->f.merge ? params->f.shape.dim / params->f.shape.n_groups : params->f.shape.dim, params->dout_d_stride,
+                params->f.shape.nrows, params->dout_h_stride, params->f.shape.ncols, esize(params->dout_dtype)))
         return SND_ERR_STRIDE;
     const int wave = use_wavefront(params->f.shape, params->f.schedule);
     if (wave < 0) return SND_ERR_SHAPE;

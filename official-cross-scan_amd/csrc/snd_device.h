@@ -81,6 +81,10 @@ __device__ __forceinline__ void st_f32_b(void *base, uint32_t off, int dt, float
     else if (dt == SND_BF16) *(uint16_t *)q = f32_to_bf16(v);
     else *(f16_t *)q = (f16_t)v;
 }
+// float add to global memory, no value returned (one L2 atomic)
+__device__ __forceinline__ void glb_add(float *p, float v) {
+    __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 // a*b + c with 24-bit a, b (full-rate multiply-add; 32-bit integer multiplies are quarter rate)
 __device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }
 

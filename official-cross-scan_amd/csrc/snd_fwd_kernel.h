@@ -110,6 +110,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     const float Dv = p.D ? p.D[cc] : 0.f;
     const float bias = p.delta_bias ? p.delta_bias[cc / rd] : 0.f;
     const bool softplus = p.delta_softplus != 0;
+    // fused CrossMerge: the channel's result is scaled by its weight and added to the merged feature channel
+    const bool merge = p.merge != 0;
+    const float wm = merge && p.merge_weights ? p.merge_weights[cc] : 1.f;
+    const int mshift = merge ? g * rg : 0;          // out channel of channel c is c - mshift
 
     // per-batch-image base pointers (uniform) and 32-bit offsets inside the image
     const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
@@ -400,14 +404,17 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             SND_THREAD_MAPS(NP);
             const int jq = J % QT;
             if (geo.nCX <= 2) {                     // narrow planes: nothing to gather, write directly
-                const uint32_t cOb = (uint32_t)cc * (uint32_t)p.out_d_stride * esz_out;
+                const uint32_t cOb = (uint32_t)(cc - mshift) * (uint32_t)p.out_d_stride * esz_out;
 #pragma unroll
                 for (int k = 0; k < NPX; ++k) {
                     const int pp = n + NP * k;
                     const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-                    if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W && !(SND_TILE_ABLATE & 1))
-                        st_f32_b(outb, cOb + mad24(mrow(row), OhB, mcol(col) << sh_out), p.out_dtype,
-                                 fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]));
+                    if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W && !(SND_TILE_ABLATE & 1)) {
+                        const float v = fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
+                        const uint32_t o = cOb + mad24(mrow(row), OhB, mcol(col) << sh_out);
+                        if (merge) glb_add((float *)((char *)outb + o), wm * v);
+                        else st_f32_b(outb, o, p.out_dtype, v);
+                    }
                 }
                 return;
             }
@@ -415,7 +422,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 if ((pp >> 3) < TE && (pp & 7) < TE)
-                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
+                    sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = wm * fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
@@ -429,8 +436,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                     const int ch = idx / PER_CH, rr = (idx / QC) & 7, c32 = idx & (QC - 1);
                     const int row = r0 + rr;
                     if (rr < TE && row < H && c32 < ncols && cbase + ch < cend && !(SND_TILE_ABLATE & 1)) {
-                        const uint32_t o = (uint32_t)(cbase + ch) * (uint32_t)p.out_d_stride * esz_out;
-                        st_f32_b(outb, o + mad24(mrow(row), OhB, mcol(c0 + c32) << sh_out), p.out_dtype, sOut[ch * OCH + rr * OROW + c32]);
+                        const uint32_t o = (uint32_t)(cbase + ch - mshift) * (uint32_t)p.out_d_stride * esz_out +
+                                           mad24(mrow(row), OhB, mcol(c0 + c32) << sh_out);
+                        if (merge) glb_add((float *)((char *)outb + o), sOut[ch * OCH + rr * OROW + c32]);
+                        else st_f32_b(outb, o, p.out_dtype, sOut[ch * OCH + rr * OROW + c32]);
                     }
                 }
                 // the next write of sOut is behind the next tile's barriers

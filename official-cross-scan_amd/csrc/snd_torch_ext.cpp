@@ -150,18 +150,37 @@ void fill_fwd(snd_fwd_params &p, const Checked &c, const at::Tensor &u, const at
     p.C_batch_stride = C.stride(0); p.C_group_stride = C.stride(1); p.C_dstate_stride = C.stride(2); p.C_h_stride = C.stride(3);
 }
 
+// Fused CrossMerge arguments: weights are one float32 per channel, contiguous, on the inputs' device.
+void check_merge(const Checked &c, bool merge, const c10::optional<at::Tensor> &w, const at::Tensor &u) {
+    if (!merge) {
+        TORCH_CHECK(!w.has_value(), "merge_weights given without merge=True");
+        return;
+    }
+    if (w.has_value()) {
+        const at::Tensor &t = w.value();
+        TORCH_CHECK(t.scalar_type() == at::ScalarType::Float && t.is_cuda() && t.is_contiguous() && t.numel() == c.dim &&
+                        t.device() == u.device(),
+                    "merge_weights must be a contiguous float32 GPU tensor with dim = ", c.dim, " elements");
+    }
+}
+
 std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor &delta, const at::Tensor &A,
                                            const at::Tensor &B, const at::Tensor &C,
                                            const c10::optional<at::Tensor> &D_,
                                            const c10::optional<at::Tensor> &delta_bias_, bool delta_softplus,
                                            bool out_float, const c10::optional<at::Tensor> &A_decay_,
-                                           int64_t directions, int64_t schedule) {
+                                           int64_t directions, int64_t schedule, bool merge,
+                                           const c10::optional<at::Tensor> &merge_weights_) {
     TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
+    check_merge(c, merge, merge_weights_, u);
+    TORCH_CHECK(!merge || out_float, "the fused merge accumulates in float32: out_float must be true");
     at::hip::HIPGuardMasqueradingAsCUDA device_guard{u.device()};
     const auto f32 = u.options().dtype(at::ScalarType::Float);
-    at::Tensor out = torch::empty({c.batch, c.dim, c.nrows, c.ncols},
-                                  u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
+    // merged: one fp32 channel per feature, zero-filled, to which every group adds its weighted result
+    at::Tensor out = merge ? torch::zeros({c.batch, c.dim / c.n_groups, c.nrows, c.ncols}, f32)
+                           : torch::empty({c.batch, c.dim, c.nrows, c.ncols},
+                                          u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
     at::Tensor x = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
     at::Tensor x_v = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_y, c.plan.xv_inner}, f32);
     at::Tensor x_sd = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
@@ -183,6 +202,8 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
         p.workspace_bytes = c.plan.fwd_workspace_bytes;
     }
     p.directions = (int32_t)directions;
+    p.merge = merge ? 1 : 0;
+    p.merge_weights = merge && merge_weights_.has_value() ? merge_weights_.value().data_ptr<float>() : nullptr;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_fwd(&p, (snd_stream_t)stream), "fwd");
     check_pipeline(ws, stream, "fwd");
@@ -195,15 +216,17 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
                                            const c10::optional<at::Tensor> &delta_bias_, const at::Tensor &dout,
                                            const c10::optional<at::Tensor> &x_, const c10::optional<at::Tensor> &x_v_,
                                            bool delta_softplus, const c10::optional<at::Tensor> &A_decay_,
-                                           const c10::optional<at::Tensor> &x_sd_, int64_t directions, int64_t schedule) {
+                                           const c10::optional<at::Tensor> &x_sd_, int64_t directions, int64_t schedule,
+                                           bool merge, const c10::optional<at::Tensor> &merge_weights_) {
     TORCH_CHECK(directions == SND_DIR_TOPLEFT || directions == SND_DIR_CORNERS, "directions must be 0 (top-left) or 1 (four corners)");
     const Checked c = check_inputs(u, delta, A, B, C, D_, delta_bias_, A_decay_);
+    check_merge(c, merge, merge_weights_, u);
     const int batch_size = c.batch, dim = c.dim, nrows = c.nrows, ncols = c.ncols, dstate = c.dstate;
     TORCH_CHECK(dout.scalar_type() == u.scalar_type() || dout.scalar_type() == at::ScalarType::Float,
                 "dout must be float32 or the input dtype");
     TORCH_CHECK(dout.is_cuda());
     TORCH_CHECK(dout.stride(-1) == 1 || dout.size(-1) == 1, "dout must be contiguous in its last dimension");
-    CHECK_SHAPE(dout, batch_size, dim, nrows, ncols);
+    CHECK_SHAPE(dout, batch_size, merge ? dim / c.n_groups : dim, nrows, ncols);   // merged: the gradient of the merged output
     // the saved state is required: gradients computed without it would belong to another function
     TORCH_CHECK(x_.has_value() && x_v_.has_value() && x_sd_.has_value(),
                 "bwd needs the x, x_v and x_sd tensors returned by fwd");
@@ -230,13 +253,15 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     at::Tensor accBC = torch::zeros({2 * round64(nBC)}, f32);
     at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
     at::Tensor dC = accBC.narrow(0, round64(nBC), nBC).view(C.sizes());
-    const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim);
-    at::Tensor accP = torch::zeros({oDec + 64}, f32);
+    const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim), oMerge = oDec + 64;
+    at::Tensor accP = torch::zeros({oMerge + (merge ? round64(dim) : 0)}, f32);
     at::Tensor dA = accP.narrow(0, 0, nA).view({dim, dstate});
     at::Tensor dD, ddelta_bias, dA_decay;
     if (D_.has_value()) dD = accP.narrow(0, oD, dim);
     if (delta_bias_.has_value()) ddelta_bias = accP.narrow(0, oBias, dim);
     if (A_decay_.has_value()) dA_decay = accP.narrow(0, oDec, 1);
+    at::Tensor dmerge;                              // weight * d(weight) per channel (the caller divides)
+    if (merge) dmerge = accP.narrow(0, oMerge, dim);
     const int sched = resolve_schedule(schedule);
     at::Tensor ws;                                  // the wavefront kernels need none
     if (!wavefront(sched, c.plan)) ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
@@ -257,6 +282,9 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     p.workspace_bytes = ws.defined() ? c.plan.bwd_workspace_bytes : 0;
     p.f.schedule = sched;
     p.f.directions = (int32_t)directions;
+    p.f.merge = merge ? 1 : 0;
+    p.f.merge_weights = merge && merge_weights_.has_value() ? merge_weights_.value().data_ptr<float>() : nullptr;
+    p.dmerge = dmerge.defined() ? dmerge.data_ptr<float>() : nullptr;
     auto stream = at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     check_status(snd_bwd(&p, (snd_stream_t)stream), "bwd");
     if (sched == SND_SCHED_STRIPS || sched == SND_SCHED_BANDS || (sched == SND_SCHED_AUTO && c.plan.auto_bwd_jobs != 0))
@@ -271,22 +299,27 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     }
     if (c.u_shared)   // one feature map scanned by every group: its gradient is the sum over the groups
         result[0] = du.view({batch_size, c.n_groups, dim / c.n_groups, nrows, ncols}).sum(1);
+    if (merge) result.push_back(dmerge);
     return result;
 }
 
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
-    // the reference's positional lists (selective_scan_oflex.cpp:179-187,286-297) plus two trailing
-    // optional arguments: the per-group scan origin the reference leaves as a TODO (fwd.cuh:140) and the
-    // block mapping of this call (-1: the module default)
+    // the reference's positional lists (selective_scan_oflex.cpp:179-187,286-297) plus trailing optional
+    // arguments: the per-group scan origin the reference leaves as a TODO (fwd.cuh:140), the block mapping
+    // of this call (-1: the module default), and the fused CrossMerge (out / dout have dim / n_groups
+    // channels, merge_weights [dim] float32 or None for the plain sum; bwd then returns a ninth tensor,
+    // merge_weights * d merge_weights per channel)
     namespace py = pybind11;
     m.def("fwd", &selective_scan_fwd, "Selective nd scan forward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("delta_softplus"), py::arg("out_float"),
-          py::arg("A_decay"), py::arg("directions") = 0, py::arg("schedule") = -1);
+          py::arg("A_decay"), py::arg("directions") = 0, py::arg("schedule") = -1, py::arg("merge") = false,
+          py::arg("merge_weights") = py::none());
     m.def("bwd", &selective_scan_bwd, "Selective nd scan backward (gfx950)", py::arg("u"), py::arg("delta"), py::arg("A"),
           py::arg("B"), py::arg("C"), py::arg("D"), py::arg("delta_bias"), py::arg("dout"), py::arg("x"), py::arg("x_v"),
-          py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0, py::arg("schedule") = -1);
+          py::arg("delta_softplus"), py::arg("A_decay"), py::arg("x_sd"), py::arg("directions") = 0, py::arg("schedule") = -1,
+          py::arg("merge") = false, py::arg("merge_weights") = py::none());
     m.def("set_schedule", [](int mode) {
         TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_WAVEFRONT, "schedule must be 0 (auto), 1 (plane), 2 (strips), 3 (bands) or 4 (row-segment wavefront)");
         g_schedule.store(mode);

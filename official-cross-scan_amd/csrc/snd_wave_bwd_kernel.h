@@ -96,7 +96,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
     const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chunk : c) * f.u_d_stride;
     const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(c / rd) * f.delta_d_stride;
-    const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)c * p.dout_d_stride;
+    // fused CrossMerge: dout is the gradient of the merged output, shared by the groups and scaled by the channel's weight
+    const bool merge = f.merge != 0;
+    const float wm = merge && f.merge_weights ? f.merge_weights[c] : 1.f;
+    const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)(merge ? chunk : c) * p.dout_d_stride;
     T *dub = (T *)p.du + ((int64_t)b * Dm + c) * H * W;                 // du, ddelta: dense [b, c, H, W]
     T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + c) * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;               // dense [b, g, N, H, W]
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     float Gd[NS][CPL], ad[NS][CPL], GdEdge[NS];     // G, a of the row below at this lane's columns; G[i+1, S*(w+1)]
     float dA_acc[NS];
-    float dec_acc = 0.f, dD_acc = 0.f, dbias_acc = 0.f;
+    float dec_acc = 0.f, dD_acc = 0.f, dbias_acc = 0.f, dw_acc = 0.f;
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
         GdEdge[n] = 0.f; dA_acc[n] = 0.f;
@@ -294,7 +297,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                 unpack(cur.o[r], dov);
 #pragma unroll
                 for (int t = 0; t < CPL; ++t) {
-                    dov[t] = jin ? dov[t] : 0.f;
+                    dov[t] = jin ? wm * dov[t] : 0.f;
                     dlu[t] = dl[r][t] * uu[r][t];
                     qsum[t] = 0.f;
                     psum[t] = 0.f;
@@ -367,6 +370,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         duv[t] = fmaf(Dv, dov[t], dl[r][t] * qsum[t]);
                         ddl[t] = fmaf(uu[r][t], qsum[t], psum[t]) * dsp[r][t];
                         dD_acc = fmaf(dov[t], uu[r][t], dD_acc);
+                        dw_acc = fmaf(duv[t], uu[r][t], dw_acc);
                         dbias_acc += ddl[t];
                     }
                     if (CPL == 2 && !fh) {                                             // to memory order
@@ -413,6 +417,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         if (lane == 63) {
             if (p.dD) wave_glb_add(p.dD + c, td);
             if (p.ddelta_bias) wave_glb_add(p.ddelta_bias + c, tb);
+        }
+        // Fused CrossMerge: weight * d(weight) = <weighted dout, result of the channel>, and since the result is
+        // linear in u (D*u plus a recurrence linear in B*delta'*u) that inner product equals <du, u>.
+        if (merge && p.dmerge) {
+            const float tw = wave_sum_to_last(dw_acc);
+            if (lane == 63) wave_glb_add(p.dmerge + c, tw);
         }
     }
     if (want_decay) {

@@ -80,7 +80,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
     const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chunk : c) * p.u_d_stride;
     const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(c / rd) * p.delta_d_stride;
-    OutT *outb = (OutT *)p.out + (int64_t)b * p.out_batch_stride + (int64_t)c * p.out_d_stride;
+    // fused CrossMerge (fp32 out only): the channel adds weight * result to the feature channel it belongs to
+    const bool merge = p.merge != 0;
+    const float wm = merge && p.merge_weights ? p.merge_weights[c] : 1.f;
+    OutT *outb = (OutT *)p.out + (int64_t)b * p.out_batch_stride + (int64_t)(merge ? chunk : c) * p.out_d_stride;
     // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
     const int UhB = (int)p.u_h_stride * ESZ * rs, DhB = (int)p.delta_h_stride * ESZ * rs, BhB = (int)p.B_h_stride * ESZ * rs,
               ChB = (int)p.C_h_stride * ESZ * rs, OhB = (int)p.out_h_stride * OSZ * rs;
@@ -210,7 +213,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) o[k] = fmaf(Dv, u[k], acc[k]);
                     if (CPL == 2 && fh) { const float t = o[0]; o[0] = o[CPL - 1]; o[CPL - 1] = t; }
-                    wave_st<OutT, CPL, VEC>(outb, oo, o);
+                    if (OUT32 && merge) {
+#pragma unroll
+                        for (int k = 0; k < CPL; ++k) glb_add((float *)((char *)outb + oo) + k, wm * o[k]);
+                    } else {
+                        wave_st<OutT, CPL, VEC>(outb, oo, o);
+                    }
                 }
                 oo += OhB;
             }

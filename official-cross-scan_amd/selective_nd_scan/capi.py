@@ -38,14 +38,14 @@ class FwdParams(C.Structure):
                                     "B_batch_stride", "B_group_stride", "B_dstate_stride", "B_h_stride",
                                     "C_batch_stride", "C_group_stride", "C_dstate_stride", "C_h_stride",
                                     "out_batch_stride", "out_d_stride", "out_h_stride")] +
-                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("directions", i32), ("u_shared", i32), ("reserved_", i32)])
+                [("workspace", vp), ("workspace_bytes", i64), ("schedule", i32), ("directions", i32), ("u_shared", i32), ("merge", i32), ("merge_weights", vp)])
 
 
 class BwdParams(C.Structure):
     _fields_ = ([("f", FwdParams), ("dout", vp), ("dout_dtype", i32)] +
                 [(n, i64) for n in ("dout_batch_stride", "dout_d_stride", "dout_h_stride")] +
                 [(n, vp) for n in ("du", "ddelta", "dA", "dB", "dC", "dD", "ddelta_bias", "dA_decay", "workspace")] +
-                [("workspace_bytes", i64)])
+                [("workspace_bytes", i64), ("dmerge", vp)])
 
 
 def declared_symbols():
@@ -133,26 +133,32 @@ class FwdCall:
     """Outputs, saved state and the filled snd_fwd_params of one forward; launch() only enqueues."""
 
     def __init__(self, u, delta, A, B, Cc, D=None, delta_bias=None, delta_softplus=False, out_float=True,
-                 A_decay=None, save=True, schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
+                 A_decay=None, save=True, schedule=SCHED_AUTO, directions=DIR_TOPLEFT, merge=False, merge_weights=None):
         import torch
-        self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay)
+        self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, merge_weights)
         shape = make_shape(u, delta, A, B)
         st, plan = make_plan(shape)
         check(st)
         self.plan = plan
         Bt, Dm, N = u.shape[0], A.shape[0], A.shape[1]
         f32 = dict(device=u.device, dtype=torch.float32)
-        self.out = torch.empty((Bt, Dm, u.shape[2], u.shape[3]), device=u.device, dtype=torch.float32 if out_float else u.dtype)
+        if merge:                                # fused CrossMerge: one zero-filled fp32 channel per feature
+            self.out = torch.zeros((Bt, Dm // B.shape[1], u.shape[2], u.shape[3]), **f32)
+        else:
+            self.out = torch.empty((Bt, Dm, u.shape[2], u.shape[3]), device=u.device, dtype=torch.float32 if out_float else u.dtype)
         self.x_v = torch.empty((Bt, Dm, N, plan.n_chunks_y, plan.xv_inner), **f32)
         self.x = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.params = FwdParams()
         _fill_fwd(self.params, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, self.out,
                   self.x, self.x_v, self.x_sd, schedule, directions)
+        self.params.merge, self.params.merge_weights = int(merge), _ptr(merge_weights)
         self.ws = torch.empty(plan.fwd_workspace_bytes // 4 + 4, **f32)
         self.params.workspace, self.params.workspace_bytes = self.ws.data_ptr(), plan.fwd_workspace_bytes
 
     def launch(self, stream=None):
+        if self.params.merge:
+            self.out.zero_()
         check(lib().snd_fwd(C.byref(self.params), _stream(stream)))
 
 
@@ -162,9 +168,9 @@ class BwdCall:
     enqueues the kernel; launch_kernel_only() skips the zero-fill (timing)."""
 
     def __init__(self, u, delta, A, B, Cc, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd,
-                 schedule=SCHED_AUTO, directions=DIR_TOPLEFT):
+                 schedule=SCHED_AUTO, directions=DIR_TOPLEFT, merge=False, merge_weights=None):
         import torch
-        self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, dout, x, x_v, x_sd)
+        self.keep = (u, delta, A, B, Cc, D, delta_bias, A_decay, dout, x, x_v, x_sd, merge_weights)
         shape = make_shape(u, delta, A, B)
         st, plan = make_plan(shape)
         check(st)
@@ -177,6 +183,7 @@ class BwdCall:
         self.dD = torch.zeros_like(D) if D is not None else None
         self.dbias = torch.zeros(Dm, **f32) if delta_bias is not None else None
         self.ddec = torch.zeros_like(A_decay) if A_decay is not None else None
+        self.dmerge = torch.zeros(Dm, **f32) if merge else None    # merge_weights * d merge_weights per channel
         self.ws = torch.empty(plan.bwd_workspace_bytes // 4 + 4, **f32)
         bp = self.params = BwdParams()
         _fill_fwd(bp.f, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, None, x, x_v, x_sd,
@@ -187,9 +194,10 @@ class BwdCall:
         bp.dA, bp.dB, bp.dC = self.dA.data_ptr(), self.dB.data_ptr(), self.dC.data_ptr()
         bp.dD, bp.ddelta_bias, bp.dA_decay = _ptr(self.dD), _ptr(self.dbias), _ptr(self.ddec)
         bp.workspace, bp.workspace_bytes = self.ws.data_ptr(), plan.bwd_workspace_bytes
+        bp.f.merge, bp.f.merge_weights, bp.dmerge = int(merge), _ptr(merge_weights), _ptr(self.dmerge)
 
     def zero(self):
-        for t in (self.dA, self.dB, self.dC, self.dD, self.dbias, self.ddec):
+        for t in (self.dA, self.dB, self.dC, self.dD, self.dbias, self.ddec, self.dmerge):
             if t is not None:
                 t.zero_()
 

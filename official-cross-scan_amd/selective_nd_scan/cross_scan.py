@@ -15,7 +15,7 @@ of B and C belongs to corner k (G = 4, or a multiple of 4 with group g -> corner
 """
 import torch
 
-from .interface import selective_nd_scan
+from .interface import selective_nd_scan, selective_nd_scan_merged
 
 # corner k = (rows reversed, columns reversed): 0 top-left, 1 top-right, 2 bottom-left, 3 bottom-right
 CORNER_FLIPS = ((False, False), (False, True), (True, False), (True, True))
@@ -76,7 +76,17 @@ def cross_scan_2d(x, delta, A, B, C, D=None, delta_bias=None, delta_softplus=Tru
                   A_decay=None):
     """The block's scan stage: x [B, C, H, W] is scanned from the four corners (delta [B, 4*C, H, W],
     A [4*C, N], B, C [B, 4, N, H, W], D, delta_bias [4*C] are per direction) and the four results are
-    fused into [B, C, H, W] (fp32).  x is passed as it is: the kernels let every direction group read
-    the same C channels (u with dim / n_groups channels), so not even cross_scan's copies are made."""
+    fused into [B, C, H, W] (fp32).  One kernel call each way: x is passed as it is (the kernels let every
+    direction group read the same C channels, so not even cross_scan's copies are made), and the four
+    results of a feature are added, with their weights, straight into the merged output (no [B, 4*C, H, W]
+    tensor is written or read back; the backward reads the merged gradient the same way).
+    merge_weights: None, [4] or [4, C]."""
+    return selective_nd_scan_merged(x, delta, A, B, C, D, delta_bias, delta_softplus, A_decay, 1, merge_weights)
+
+
+def cross_scan_2d_unfused(x, delta, A, B, C, D=None, delta_bias=None, delta_softplus=True, merge_weights=None,
+                          A_decay=None):
+    """cross_scan_2d as two steps (the scan writes [B, 4*C, H, W], cross_merge reduces it): the check of the
+    fused path."""
     y = four_corner_scan(x, delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay)
     return cross_merge(y, merge_weights)

@@ -25,17 +25,22 @@ from ._ext import ext
 
 
 def fwd(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True, A_decay=None,
-        directions=0, schedule=-1):
+        directions=0, schedule=-1, merge=False, merge_weights=None):
     """Reference binding `fwd` -> [out, x, x_v, x_sd] (selective_scan_oflex.cpp:179-187,282).
-    schedule: block mapping of this call (-1 = the module default, see set_schedule)."""
-    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions, schedule)
+    schedule: block mapping of this call (-1 = the module default, see set_schedule).
+    merge: the CrossMerge fused into the output stores: out is [B, D/G, H, W] fp32, the sum over the G
+    groups of merge_weights[channel] * (result of the channel) (merge_weights [D] fp32, None = ones)."""
+    return ext().fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions, schedule,
+                     merge, merge_weights)
 
 
-def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions=0, schedule=-1):
+def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions=0, schedule=-1,
+        merge=False, merge_weights=None):
     """Reference binding `bwd` -> [du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay]
-    (selective_scan_oflex.cpp:286-297,432-438)."""
+    (selective_scan_oflex.cpp:286-297,432-438).  With merge, dout is the gradient of the merged output
+    [B, D/G, H, W] and a ninth tensor follows: merge_weights * d merge_weights, per channel [D]."""
     return ext().bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay, x_sd, directions,
-                     schedule)
+                     schedule, merge, merge_weights)
 
 
 def set_schedule(mode):
@@ -91,3 +96,73 @@ def selective_nd_scan(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus
     """Differentiable 2D-CrossScan selective scan (forward and backward run on the HIP kernels).
     directions=1: group g of B/C (and its dim/G channels) is scanned from corner g % 4."""
     return SelectiveNdScanFn.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)
+
+
+# Magnitude below which a merge weight enters the backward as +-1e-20 instead of itself.  The kernels return
+# weight * d(weight) (every gradient of the op is linear in the weighted dout, so the weight is applied once,
+# where dout is staged); dividing by a weight of exactly 0 would lose d(weight), which is <dout, result> and does
+# not vanish with the weight.  With the floor, the other gradients of such a channel come out scaled by 1e-20
+# instead of 0: far below one ulp of anything they are added to.
+_MERGE_WEIGHT_FLOOR = 1e-20
+
+
+class SelectiveNdScanMergedFn(torch.autograd.Function):
+    """The scan with the CrossMerge fused into its output stores: out [B, D/G, H, W] fp32 is the sum over the
+    G groups of merge_weights[g, i] * (result of channel g*(D/G) + i)."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, u, delta, A, B, C, D, delta_bias, delta_softplus, A_decay, directions, merge_weights):
+        u, delta, B, C = map(_last_dim_contiguous, (u, delta, B, C))
+        w = None
+        if merge_weights is not None:
+            G = B.shape[1]
+            w = merge_weights.detach().to(torch.float32).reshape(G, -1).expand(G, A.shape[0] // G).contiguous().view(-1)
+        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay, directions, -1, True, w)
+        ctx.delta_softplus = delta_softplus
+        ctx.directions = directions
+        ctx.has = (D is not None, delta_bias is not None, A_decay is not None)
+        ctx.w_shape = None if merge_weights is None else tuple(merge_weights.shape)
+        ctx.w_dtype = None if merge_weights is None else merge_weights.dtype
+        ctx.save_for_backward(u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd, w)
+        return out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dout):
+        u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd, w = ctx.saved_tensors
+        dout = _last_dim_contiguous(dout)
+        wb = None
+        if w is not None:
+            floor = torch.full_like(w, _MERGE_WEIGHT_FLOOR)
+            wb = torch.where(w.abs() < _MERGE_WEIGHT_FLOOR, floor, w)
+        du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay, wdw = bwd(
+            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions, -1,
+            True, wb)
+        dw = None
+        if w is not None and ctx.needs_input_grad[10]:
+            G = B.shape[1]
+            dw = (wdw / wb).view(G, -1)
+            if ctx.w_shape != tuple(dw.shape):       # weights were given per group ([G] or [G, 1]): sum the features
+                dw = dw.sum(1).view(ctx.w_shape)
+            dw = dw.to(ctx.w_dtype)
+        has_D, has_bias, has_decay = ctx.has
+        return (du, ddelta, dA, dB, dC, dD if has_D else None, ddelta_bias if has_bias else None,
+                None, dA_decay if has_decay else None, None, dw)
+
+
+def selective_nd_scan_merged(u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, A_decay=None,
+                             directions=1, merge_weights=None):
+    """selective_nd_scan followed by the merge of the G group results of every feature, in one kernel call:
+    returns [B, D/G, H, W] fp32 = sum_g merge_weights[g, i] * out[:, g*(D/G) + i].  merge_weights: None (plain
+    sum), [G], [G, 1] or [G, D/G]; differentiable.  The sum is accumulated with float atomics, so its last bits
+    depend on the order the groups arrive in."""
+    if merge_weights is not None:
+        G = B.shape[1]
+        if merge_weights.dim() == 1:
+            if merge_weights.numel() != G:
+                raise ValueError("merge_weights must have shape [G], [G, 1] or [G, D/G]")
+        elif tuple(merge_weights.shape) not in ((G, 1), (G, A.shape[0] // G)):
+            raise ValueError("merge_weights must have shape [G], [G, 1] or [G, D/G]")
+    return SelectiveNdScanMergedFn.apply(u, delta, A, B, C, D, delta_bias, delta_softplus, A_decay, directions,
+                                         merge_weights)

@@ -17,23 +17,23 @@ def test_library_exports_every_declared_symbol():
     lib = capi.lib()
     for n in names:
         assert getattr(lib, n) is not None, n
-    assert lib.snd_version() >= 200
+    assert lib.snd_version() >= 210
 
 
 def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
     assert C.sizeof(capi.Plan) == 64
-    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4
-    assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8
+    assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4 + 8
+    assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8 + 8
 
 
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
     probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs"]),
-              ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared"]),
-              ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes"])]
+              ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared", "merge", "merge_weights"]),
+              ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes", "dmerge"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
     for cname, _, fields in probes:
         src.append('printf("%%zu\\n", sizeof(%s));' % cname)
