@@ -119,6 +119,9 @@ def test_address_range_limits_are_status_codes():
     assert lib.snd_fwd(C.byref(params(u_d_stride=1 << 28)), None) == -4          # image >= 2^32 bytes
     assert lib.snd_fwd(C.byref(params(out_d_stride=-1)), None) == -4             # negative stride
     assert lib.snd_fwd(C.byref(params(H=1 << 15, W=1 << 15, dim=8)), None) == -4  # dense gradients >= 2^32 bytes
+    assert lib.snd_fwd(C.byref(params(H=1, W=1 << 21, dim=4)), None) == -4         # 2^21 columns: beyond the 24-bit column math
+    assert lib.snd_fwd(C.byref(params(merge=2)), None) == -2                      # fused merge is a flag
+    assert lib.snd_fwd(C.byref(params(merge=1, out_dtype=capi.SND_BF16)), None) == -3   # merged output is accumulated in fp32
     assert b"2^32" in lib.snd_status_string(-4)
 
 
