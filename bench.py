@@ -9,11 +9,13 @@ Prints ONE JSON line.  `value` is the algorithmic HBM rate of the whole step:
     bytes = (2eP + 2eQ + 4P) + (4eP + 4eQ + 4P),  P = B*D*H*W, Q = B*K*N*H*W, e = input bytes
 (compulsory tensor I/O only) divided by the mean step time.  `roofline` is the same figure for the
 dominant kernel alone (the backward), from HIP events around its launches on the launch stream, with
-a second leg beside it: vector-ALU wave-instructions per second against 1024 SIMDs x clock / 4 cycles.
-The instruction count, the clock and the HBM traffic per launch are counter readings that a timed run
-cannot take; they come from the committed rocprofv3 summary of the same workload under profiles/
-(named in `roofline.counters_from`), while every duration is measured live.  `roofline.bound` names
-the leg with the higher fraction.  `cpu_baseline` times the C restatement of the reference recurrence
+a second leg beside it: vector-ALU wave-instructions per second against the published FP32 vector peak
+(157.3 TFLOP/s = 1228.9 G wave-wide multiply-adds per second: a SIMD retires one 64-lane FP32 instruction
+per two cycles), with the rate `--issue-probe` measures for a pure multiply-add stream on all CUs beside
+it (`valu.probe_peak`, from profiles/issue_probe_mi355x.txt).  The instruction count, the clock and the
+HBM traffic per launch are counter readings that a timed run cannot take; they come from the committed
+rocprofv3 summary of the same workload under profiles/ (named in `roofline.counters_from`), while every
+duration is measured live.  `roofline.bound` names the leg with the higher fraction.  `cpu_baseline` times the C restatement of the reference recurrence
 (oracle/) on the host cores on a bounded sample of the same workload.
 """
 import argparse
@@ -105,7 +107,17 @@ def cpu_baseline(workload, budget_s=20.0):
             "ms_per_step_extrapolated": round(1e3 * t * (Bt * Dm) / (sb * sd), 1)}
 
 
-N_SIMD = 1024                   # 256 CUs x 4 SIMDs; a SIMD issues one wave-wide VALU instruction per 4 cycles
+VALU_PEAK = 157.3e12 / 128.0    # published FP32 vector peak in wave-wide multiply-adds per second (64 lanes x 2 flop)
+
+
+def probe_peak():
+    """Wave-instructions per second of a pure v_fma_f32 stream on all CUs, as `bench.py --issue-probe` measured it
+    (committed summary), or None."""
+    path = os.path.join(ROOT, "profiles", "issue_probe_mi355x.txt")
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"^fma_stream_ginst_per_s:\s*([0-9.]+)", open(path).read(), flags=re.M)
+    return float(m.group(1)) * 1e9 if m else None
 
 
 def profile_counters(workload):
@@ -136,6 +148,9 @@ def main():
     ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
                     help="kernel family and block mapping: chosen by shape (default), one block per plane chunk, "
                          "pipelined row strips / bands, or the row-segment wavefront kernels (1-4 states)")
+    ap.add_argument("--issue-probe", action="store_true",
+                    help="only time register-only instruction streams (library hook snd_debug_issue_probe) at 1-4 "
+                         "waves per SIMD on every CU and exit: the vector-ALU rate the roofline's second leg uses")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -154,6 +169,29 @@ def main():
             y.copy_(x)
         torch.cuda.synchronize()
         print(json.dumps({"copy_probe_bytes_each_way": x.numel() * 4}))
+        return
+    if args.issue_probe:
+        from selective_nd_scan import capi
+        lib = capi.lib()
+        sink = torch.empty(256 * 1024, device=dev)
+        stream = torch.cuda.current_stream()
+        iters = 4000
+        kinds = ["v_fma_f32", "v_fma_f32 + s_nop 0", "v_exp_f32", "v_add_f32 (DPP operand)", "v_permlane32_swap_b32"]
+        res = {}
+        for kind, name in enumerate(kinds):
+            row = []
+            for wps in (1, 2, 3, 4):
+                capi.check(lib.snd_debug_issue_probe(kind, wps, 200, sink.data_ptr(), stream.cuda_stream))
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                capi.check(lib.snd_debug_issue_probe(kind, wps, iters, sink.data_ptr(), stream.cuda_stream))
+                e1.record(stream)
+                torch.cuda.synchronize()
+                # a SIMD hosts wps waves, each issuing iters x 64 probe instructions
+                row.append(round(e0.elapsed_time(e1) * 1e6 / (iters * 64.0 * wps), 3))
+            res[name] = row
+        print(json.dumps({"issue_probe_ns_per_instruction_per_simd": res, "waves_per_simd": [1, 2, 3, 4],
+                          "note": "256 blocks (one per CU); kind 1 counts only its v_fma_f32"}))
         return
     import selective_nd_scan as snd
     from selective_nd_scan import capi
@@ -207,13 +245,14 @@ def main():
     pc = profile_counters(args.workload) if args.schedule == "auto" else None
     if pc and pc["dominant_kernel"].startswith(kernel + "<"):
         # counters from the committed profile of this workload; the rate uses the duration measured here
-        peak_valu = N_SIMD * pc["clock_ghz"] * 1e9 / 4.0
+        peak_valu = VALU_PEAK
         rate_valu = pc["valu_insts_per_launch"] / (kb_ms * 1e-3)
+        pp = probe_peak()
         roof.update({"traffic": pc["traffic_bytes_per_launch"], "counters_from": pc["file"],
                      "profile_kernel_ms": round(pc["avg_ns"] * 1e-6, 4),
                      "valu": {"insts_per_launch": pc["valu_insts_per_launch"], "clock_ghz": pc["clock_ghz"],
                               "achieved": round(rate_valu / 1e9, 2), "peak": round(peak_valu / 1e9, 2),
-                              "unit": "G wave-instructions/s"},
+                              "probe_peak": round(pp / 1e9, 2) if pp else None, "unit": "G wave-instructions/s"},
                      "frac_valu": round(rate_valu / peak_valu, 4)})
         if roof["frac_valu"] > roof["frac"]:
             roof["bound"] = "valu"

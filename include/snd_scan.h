@@ -229,6 +229,14 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream);
  * kernel still runs to completion. */
 void snd_debug_set_spin_limit(int polls);
 
+/* Measurement hook (bench.py --issue-probe): launches, on every CU, blocks of `waves_per_simd` x 4 waves that
+ * each issue `iters` x 64 register-only instructions of one kind on eight independent accumulators:
+ * kind 0 v_fma_f32, 1 v_fma_f32 alternating with s_nop 0, 2 v_exp_f32, 3 v_add_f32 with a DPP operand,
+ * 4 v_permlane32_swap_b32.  `sink` (>= 4 bytes per launched thread: 256 x waves_per_simd x 256 floats) takes
+ * the accumulators.  The caller times the launch; the time per instruction and SIMD is what the vector-ALU
+ * leg of the roofline is priced with.  No counterpart in the reference. */
+int snd_debug_issue_probe(int kind, int waves_per_simd, int iters, float *sink, snd_stream_t stream);
+
 /* snd_bwd for callers that cannot allocate device memory (code under HIP-graph capture, serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference, which allocates its scratch with
  * torch::empty / torch::zeros inside every call (selective_scan_oflex.cpp:393-403).  Identical to
