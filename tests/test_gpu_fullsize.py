@@ -58,8 +58,11 @@ def test_full_size_configuration(gpu_device, name, Bt, Dm, H, W, N, K, dtype, fw
     for i in range(3):
         if same_kernels:
             assert torch.equal(auto[i], plane[i]), NAMES[i]
+    # sums over pixels / channels arrive through fp32 atomics whose order differs between the schedules (and from
+    # run to run): observed up to 1.0e-5 of the largest element for dA of a 512 x 512 plane; both results are held
+    # to the float64 oracle at 1e-4 below
     for i in range(3, 8):
-        assert relerr(auto[i].cpu().numpy(), plane[i].cpu().numpy()) <= (1e-5 if same_kernels else 1e-4), NAMES[i]
+        assert relerr(auto[i].cpu().numpy(), plane[i].cpu().numpy()) <= (3e-5 if same_kernels else 1e-4), NAMES[i]
 
     # the float64 oracle over the WHOLE problem, on the values the kernels saw
     f32 = lambda t_: t_.float().cpu().numpy()
