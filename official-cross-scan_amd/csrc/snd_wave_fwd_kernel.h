@@ -151,8 +151,19 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         // instead of one such chain in front of every row's scan.  (Per step, not per band: the waves of a block
         // are at different rows of their bands in the same step, and a step lasts as long as its slowest wave.)
         float ub_[R][CPL], dlb[R][CPL], dub_[R][CPL];
+        // what the segment on the left left for the rows of a step, fetched together right after the step's barrier
+        // (one LDS round trip per step instead of one in front of every row's chain); with four states the
+        // registers are needed elsewhere and the rows fetch their own
+        constexpr bool HOIST_IN = NS <= 2;
+        float4 inb[HOIST_IN ? RD : 1][NS];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            if (r % RD == 0 && HOIST_IN && !(SND_WAVE_ABLATE & 32)) {
+#pragma unroll
+                for (int q = 0; q < RD; ++q)
+#pragma unroll
+                    for (int n = 0; n < NS; ++n) inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
+            }
             if (r % RD == 0) {
 #pragma unroll
                 for (int q = r; q < r + RD; ++q) {
@@ -175,7 +186,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column S*w-1
-                    const float4 in = (SND_WAVE_ABLATE & 32) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][w][r % RD][n];
+                    const float4 in = (SND_WAVE_ABLATE & 32) ? make_float4(0.f, 0.f, 0.f, 0.f)
+                                      : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
                     float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
                     unpack(cur.b[r][n], bu);
                     unpack(cur.c[r][n], cv);
