@@ -45,6 +45,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     // what a wave leaves for the wave on its right: {h, s, a, -} at its last column, per step parity, row and
     // state.  Wave w writes slot w+1 and reads slot w; slot 0 stays zero (nothing enters the first segment).
     __shared__ float4 sHO[2][kMaxSeg + 1][RD][NS];
+    // Only lane 63 of a wave has something to hand over.  Instead of masking the other lanes off (a compare, two
+    // exec writes and a branch around every hand-over store), every lane stores: lane 63 to the slot, the others to
+    // a word of their own that nobody reads.  One wave instruction costs the wave the same issue time either way.
+    __shared__ float4 sDump[64 * kMaxSeg];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -139,6 +143,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     const bool hands_over = multi && w + 1 < nseg;
+    const bool writer = hands_over && lane == 63;
+    float4 *const dump = &sDump[threadIdx.x];
 
     // one band of rows from `cur`, with the next band's loads issued into `nxt` first
     auto do_band = [&](Stage &cur, Stage &nxt, int band) {
@@ -173,7 +179,11 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                     for (int k = 0; k < CPL; ++k) {
                         const float raw = dlb[q][k] + bias;
                         float dsp;
-                        dlb[q][k] = (softplus && !(SND_WAVE_ABLATE & 4)) ? softplus20(raw, dsp) : raw;
+                        // always evaluated, then selected: a branch around it (the flag is uniform) costs a wave more
+                        // issue time than the select, and every model in practice asks for the softplus
+                        float sp = (SND_WAVE_ABLATE & 4) ? raw : softplus20(raw, dsp);
+                        asm volatile("" : "+v"(sp));
+                        dlb[q][k] = softplus ? sp : raw;
                         dub_[q][k] = dlb[q][k] * ub_[q][k];
                     }
                 }
@@ -217,8 +227,16 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                         aprev[n][k] = a[k];
                     }
                     hdiag[n] = in.x;
-                    if (!(SND_WAVE_ABLATE & 32) && hands_over && lane == 63) sHO[step & 1][w + 1][r % RD][n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
-                    if (SAVE && lane == r) { ch[n] = in.x; cs[n] = in.y; ca[n] = in.z; }
+                    if (!(SND_WAVE_ABLATE & 32)) {
+                        float4 *dst = writer ? &sHO[step & 1][w + 1][r % RD][n] : dump;
+                        *dst = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
+                    }
+                    if (SAVE) {                     // lane r keeps what entered the segment on row r (selects, no branch)
+                        const bool mine = lane == r;
+                        ch[n] = mine ? in.x : ch[n];
+                        cs[n] = mine ? in.y : cs[n];
+                        ca[n] = mine ? in.z : ca[n];
+                    }
                 }
                 if (jin && (!(SND_WAVE_ABLATE & 1) || acc[0] == 1234.5f)) {
                     float o[CPL];
