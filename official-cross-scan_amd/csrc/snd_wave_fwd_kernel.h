@@ -48,7 +48,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     // Only lane 63 of a wave has something to hand over.  Instead of masking the other lanes off (a compare, two
     // exec writes and a branch around every hand-over store), every lane stores: lane 63 to the slot, the others to
     // a word of their own that nobody reads.  One wave instruction costs the wave the same issue time either way.
-    __shared__ float4 sDump[64 * kMaxSeg];
+    __shared__ float4 sDump[64 * kMaxSeg + RD * NS];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -147,7 +147,9 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     float4 *const dump = &sDump[threadIdx.x];
 
     // one band of rows from `cur`, with the next band's loads issued into `nxt` first
-    auto do_band = [&](Stage &cur, Stage &nxt, int band) {
+    // (MERGE_: whether out is accumulated with atomics - decided once around the band loop, not at every row's store)
+    auto do_band = [&](auto MERGE_, Stage &cur, Stage &nxt, int band) {
+        constexpr bool MERGE = decltype(MERGE_)::value;
         load_band(nxt, min(band + 1, wg.nBands - 1));   // unconditionally (the last band once more): a skipped load would leave two
                                                         // paths with different numbers of loads in flight, and the waits follow the smaller
         const int i0 = band * R;
@@ -162,6 +164,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         // registers are needed elsewhere and the rows fetch their own
         constexpr bool HOIST_IN = NS <= 2;
         float4 inb[HOIST_IN ? RD : 1][NS];
+        float4 *wr = dump;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (r % RD == 0 && HOIST_IN && !(SND_WAVE_ABLATE & 32)) {
@@ -170,6 +173,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
                     for (int n = 0; n < NS; ++n) inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
             }
+            if (r % RD == 0) wr = writer ? &sHO[step & 1][w + 1][0][0] : dump;   // this step's slot (or the lane's own word)
             if (r % RD == 0) {
 #pragma unroll
                 for (int q = r; q < r + RD; ++q) {
@@ -228,8 +232,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                     }
                     hdiag[n] = in.x;
                     if (!(SND_WAVE_ABLATE & 32)) {
-                        float4 *dst = writer ? &sHO[step & 1][w + 1][r % RD][n] : dump;
-                        *dst = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
+                        wr[(r % RD) * NS + n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
                     }
                     if (SAVE) {                     // lane r keeps what entered the segment on row r (selects, no branch)
                         const bool mine = lane == r;
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) o[k] = fmaf(Dv, u[k], acc[k]);
                     if (CPL == 2 && fh) { const float t = o[0]; o[0] = o[CPL - 1]; o[CPL - 1] = t; }
-                    if (OUT32 && merge) {
+                    if (OUT32 && MERGE) {
 #pragma unroll
                         for (int k = 0; k < CPL; ++k) glb_add((float *)((char *)outb + oo) + k, wm * o[k]);
                     } else {
@@ -285,9 +288,16 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     lds_barrier();                                   // the zeroed slot
     if (multi)
         for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
-    for (int band = 0; band < wg.nBands; band += 2) {
-        do_band(sA, sB, band);
-        if (band + 1 < wg.nBands) do_band(sB, sA, band + 1);
+    if (OUT32 && merge) {
+        for (int band = 0; band < wg.nBands; band += 2) {
+            do_band(std::true_type{}, sA, sB, band);
+            if (band + 1 < wg.nBands) do_band(std::true_type{}, sB, sA, band + 1);
+        }
+    } else {
+        for (int band = 0; band < wg.nBands; band += 2) {
+            do_band(std::false_type{}, sA, sB, band);
+            if (band + 1 < wg.nBands) do_band(std::false_type{}, sB, sA, band + 1);
+        }
     }
     if (multi)
         for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
