@@ -291,7 +291,14 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
         check_pipeline(ws, stream, "bwd");
 
     // host.cpp:432-438: cast dB/dC to the input dtype, fold channel groups that share a delta
-    std::vector<at::Tensor> result = {du, ddelta, dA, dB.to(B.dtype()), dC.to(C.dtype()), dD, ddelta_bias, dA_decay};
+    // (16-bit inputs: one cast kernel for the two tensors, which share a buffer)
+    at::Tensor dBo = dB, dCo = dC;
+    if (B.scalar_type() != at::ScalarType::Float) {
+        const at::Tensor cast = accBC.to(B.dtype());
+        dBo = cast.narrow(0, 0, nBC).view(B.sizes());
+        dCo = cast.narrow(0, round64(nBC), nBC).view(C.sizes());
+    }
+    std::vector<at::Tensor> result = {du, ddelta, dA, dBo, dCo, dD, ddelta_bias, dA_decay};
     if (dim != c.delta_dim) {
         const int rep = dim / c.delta_dim;
         result[1] = ddelta.view({batch_size, c.delta_dim, rep, nrows, ncols}).sum(2);
