@@ -119,13 +119,40 @@ int check_shape(const snd_shape &s) {
 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Which kernel family a call runs: the row-segment wavefront when asked for, or under AUTO whenever the
-// shape qualifies (1-4 states, at most 512 columns); the tile kernels otherwise.  -1: WAVEFRONT asked for a
-// shape it does not cover.
+// Which of the two kernel families is the faster one for a shape with 1-4 states, from a model of the backward
+// (the longer kernel) fitted to measurements on one MI355X (32 x D x HxW planes, D*H*W constant, H = W = 7 .. 112,
+// N = 1, 2, 4, bf16):
+//   * row-segment wavefront: a plane is a block of nseg waves, 2048 waves fit the chip at once, a wave takes a
+//     row of its segment in about 1.3 us (one state), 2.4 (two), 4.5 (three or four), whatever the row's width:
+//     a 14-column row leaves 50 of its 64 lanes idle.
+//   * tile kernels with four lanes per channel: a block is one wave of 16 channels, 1024 fit at once, and a block
+//     takes one 8x8 (7x7) tile in about 18.5 us - or, with few blocks and many strips, the strip pipeline takes
+//     (column tiles + strips - 1) steps of about 25 us per round of its jobs.
+// Small planes of many channels (7x7 .. 21x21 at any state count, up to 40x40 with four states) go to the tile
+// kernels (7x7, one state: 0.11 ms instead of 0.46; 14x14, four states: 0.21 instead of 0.73), large or few planes
+// to the wavefront (512x512 x 256 channels, one state: 0.7 ms instead of 3.2).
+bool wave_family_pays(const snd_shape &s) {
+    const snd::Geo g = snd::make_geo(s.nrows, s.ncols);
+    const snd::WaveGeo wg = snd::make_wave_geo(s.nrows, s.ncols, s.dstate);
+    const double t_row = s.dstate <= 1 ? 1.3 : s.dstate == 2 ? 2.4 : 4.5;
+    const int64_t waves = (int64_t)s.batch * s.dim * wg.nseg;
+    const double t_wave = (double)((waves + 2047) / 2048) * (wg.Hp + (wg.nseg - 1) * wg.R) * t_row;
+    const int64_t blocks = plane_chunks(s);
+    const double t_plane = (double)((blocks + 1023) / 1024) * g.nCX * g.nCY * 18.5;
+    const int64_t rounds = (blocks * g.nCY + 1023) / 1024;
+    const double steps = (double)rounds * g.nCX > g.nCX + g.nCY - 1 ? (double)rounds * g.nCX : g.nCX + g.nCY - 1;
+    // (the tile kernels pipeline the strips of a plane only where use_strip_pipeline() says so)
+    const bool pipelined = snd::use_strip_pipeline(snd::kSchedAuto, blocks, g.nCY, &s);
+    return t_wave <= (pipelined ? steps * 25.0 : t_plane);
+}
+
+// Which kernel family a call runs: the row-segment wavefront when asked for, or under AUTO when the shape
+// qualifies (1-4 states, at most 512 columns) and the model above prefers it; the tile kernels otherwise.
+// -1: WAVEFRONT asked for a shape it does not cover.
 int use_wavefront(const snd_shape &s, int schedule) {
     const bool fits = snd::wave_family_fits(s.ncols, s.dstate);
     if (schedule == SND_SCHED_WAVEFRONT) return fits ? 1 : -1;
-    return schedule == SND_SCHED_AUTO && fits ? 1 : 0;
+    return schedule == SND_SCHED_AUTO && fits && wave_family_pays(s) ? 1 : 0;
 }
 
 // The kernels address inside one batch image with unsigned 32-bit BYTE offsets from a scalar base
@@ -215,7 +242,7 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
     plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
                                               (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
-    if (wave) {
+    if (wave && wave_family_pays(*shape)) {
         plan->auto_schedule = SND_SCHED_WAVEFRONT;
         plan->auto_bwd_jobs = 0;
     }

@@ -62,7 +62,6 @@ def run(dev, Bt, Dm, H, W, N, K, Dd, dtype, sched, dirs=capi.DIR_TOPLEFT, softpl
 def test_wavefront_matches_oracle_and_tiles(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype):
     print("wavefront", Bt, Dm, H, W, N, K, Dd, dtype, flush=True)
     d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_WAVEFRONT)
-    assert f.plan.auto_schedule == capi.SCHED_WAVEFRONT and f.plan.auto_bwd_jobs == 0
     r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
     o = (r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"])
     ref = OC.fwd(*o, True, None, real="f64")

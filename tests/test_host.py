@@ -197,6 +197,28 @@ def test_forward_job_split():
     assert sched(70, 192, 8, 56) == capi.SCHED_PLANE      # one strip
 
 
+def test_kernel_family_choice():
+    """1-4 states: large or few planes go to the row-segment wavefront, small planes of many channels to the tile
+    kernels (a 14-column row fills 14 of a wave's 64 lanes); 5-16 states always to the tile kernels."""
+    def family(Bt, Dm, H, W, N, K=4):
+        st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, N, K, Dm, capi.SND_BF16))
+        assert st == 0
+        assert plan.auto_bwd_jobs == 0 or plan.auto_schedule != capi.SCHED_WAVEFRONT
+        return "wave" if plan.auto_schedule == capi.SCHED_WAVEFRONT else "tile"
+    assert family(1, 256, 512, 512, 1) == "wave"          # 256 planes: nothing else fills the chip
+    assert family(64, 192, 56, 56, 1) == "wave"
+    assert family(64, 384, 28, 28, 1) == "wave"
+    assert family(64, 768, 14, 14, 1) == "tile"
+    assert family(64, 1536, 7, 7, 1) == "tile"
+    assert family(64, 768, 14, 14, 4) == "tile"
+    assert family(32, 256, 40, 40, 4) == "tile"
+    assert family(64, 192, 56, 56, 4) == "tile"           # 768 one-wave blocks fill the chip in one round
+    assert family(16, 192, 56, 56, 4) == "wave"           # 192 blocks do not
+    assert family(64, 192, 56, 56, 2) == "wave"
+    assert family(64, 192, 56, 56, 16) == "tile"
+    assert family(1, 8, 9, 1500, 4, K=2) == "tile"         # wider than the wavefront kernels cover
+
+
 def test_tile_extent_choice():
     """7x7 tiles where they leave clearly fewer padded cells (the 14 / 28 / 7 stage sizes), else 8x8."""
     def tiles(H, W):
