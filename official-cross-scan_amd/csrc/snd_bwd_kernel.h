@@ -666,7 +666,7 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
     constexpr size_t lds = bwd_lds_bytes<NP>();
-    const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate);   // 0: one block per plane chunk
+    const int bands = bwd_band_count(p.f.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate, geo.nCX);   // 0: one block per plane chunk
     const bool pipe = bands > 0;
     // the dynamic LDS limit of these kernels is raised by snd_init() / on the first launch on a device
     if (int st = ensure_device_ready(); st != SND_OK) return st;

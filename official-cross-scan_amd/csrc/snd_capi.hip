@@ -142,7 +142,7 @@ bool wave_family_pays(const snd_shape &s) {
     const int64_t rounds = (blocks * g.nCY + 1023) / 1024;
     const double steps = (double)rounds * g.nCX > g.nCX + g.nCY - 1 ? (double)rounds * g.nCX : g.nCX + g.nCY - 1;
     // (the tile kernels pipeline the strips of a plane only where use_strip_pipeline() says so)
-    const bool pipelined = snd::use_strip_pipeline(snd::kSchedAuto, blocks, g.nCY, &s);
+    const bool pipelined = snd::use_strip_pipeline(snd::kSchedAuto, blocks, g.nCY, &s, g.nCX, snd::bwd_slots(s.dstate));
     return t_wave <= (pipelined ? steps * 25.0 : t_plane);
 }
 
@@ -238,10 +238,10 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
     const int fwd_jobs = snd::fwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
-                                             (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
+                                             (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate, g.nCX);
     plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
     plan->auto_bwd_jobs = snd::bwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
-                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate);
+                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate, g.nCX);
     if (wave && wave_family_pays(*shape)) {
         plan->auto_schedule = SND_SCHED_WAVEFRONT;
         plan->auto_bwd_jobs = 0;

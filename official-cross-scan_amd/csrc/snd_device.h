@@ -344,13 +344,21 @@ int ensure_device_ready();
 // How a launch is scheduled (snd_fwd_params::schedule): one block per plane chunk walking all its
 // strips, or one block per strip with the strips of a plane pipelined.
 enum { kSchedAuto = 0, kSchedPlane = 1, kSchedStrips = 2, kSchedBands = 3 };
-// Strip pipelining pays when there are fewer whole-plane blocks than CUs (256): a strip waits for
-// the strip above at every tile, which costs more than it gains once the planes alone fill the chip
-// (measured at 768 plane blocks of 7x7 tiles: 2.2x slower forward, 1.3x slower backward).
-__host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int nStrips, const void *sync) {
+// Strip pipelining pays while whole-plane blocks leave the chip short of waves: always below 128 plane blocks, and
+// up to 0.8 x the backward's block slots (410 of 512 for the 16-state kernels) when the strips of a plane give at
+// least two blocks' worth of work side by side - a plane of nStrips x nTilesX tiles keeps
+// nStrips*nTilesX / (nStrips + nTilesX - 1) of its strips busy on average (7x7 tiles: 3.8, 4x4: 2.3, 2x2: 1.3).
+// Measured (16 states, fp32, 192 channels of 56x56, fwd + bwd ms, whole planes / strips): 192 plane blocks
+// 0.93 / 0.61, 288: 1.19 / 0.83, 384: 1.24 / 1.08, 480: 1.31 / 1.35, 768: strips 1.07x slower; 384 blocks of 28x28:
+// 0.36 / 0.31; 384 blocks of 14x14 (two strips): 0.097 / 0.116.  A strip waits for the strip above at every tile,
+// which costs more than it gains once the planes alone fill the chip.
+__host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int nStrips, const void *sync, int nTilesX = 0,
+                                        int64_t bwdSlots = 512) {
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return false;
     if (schedule == kSchedStrips) return true;
-    return planeBlocks < 128 || (planeBlocks < 256 && nStrips >= 16);
+    if (planeBlocks < 128 || (planeBlocks < 256 && nStrips >= 16)) return true;
+    const bool wide = nTilesX > 0 && (int64_t)nStrips * nTilesX >= 2 * ((int64_t)nStrips + nTilesX - 1);
+    return wide && planeBlocks * 5 <= bwdSlots * 4;
 }
 
 // Jobs per plane chunk: 0 = one block walks the whole plane, nStrips = one strip per job, 2-4 = bands of
@@ -359,11 +367,12 @@ __host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int n
 // whole-plane blocks leaves slots idle (backward, 768 chunks: two rounds, the second half empty);
 // cutting every plane into a few bands of strips, handed over like strips but only at band ends, lets
 // the ticket order pack them (768 x 2 bands: three rounds of half the length).
-__host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int64_t slots) {
+__host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int64_t slots,
+                               int nTilesX = 0, int64_t bwdSlots = 512) {
     const int64_t planeBlocks = nPairs * nChunks;
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return 0;
     if (schedule == kSchedStrips) return nStrips;
-    if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync)) return nStrips;
+    if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync, nTilesX, bwdSlots)) return nStrips;
     // whole planes: every (batch, group) pair is pinned to one XCD (an eighth of the slots), so the rounds
     // are those of the fullest XCD (backward, 340 pairs x 3 chunks: 129 blocks there, three rounds)
     int best = 1;
@@ -380,11 +389,12 @@ __host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nS
 }
 // Blocks per CU by the state-lane count of the kernels (16, 8 or 4 lanes per channel): the backward is held
 // to 2, 3, 4 by its LDS, the forward to 3, 6, 6.
-__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate) {
-    return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 512 : dstate > 4 ? 768 : 1024);
+__host__ inline int64_t bwd_slots(int dstate) { return dstate > 8 ? 512 : dstate > 4 ? 768 : 1024; }
+__host__ inline int bwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate, int nTilesX = 0) {
+    return band_count(schedule, nPairs, nChunks, nStrips, sync, bwd_slots(dstate), nTilesX, bwd_slots(dstate));
 }
-__host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate) {
-    return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 768 : 1536);
+__host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int dstate, int nTilesX = 0) {
+    return band_count(schedule, nPairs, nChunks, nStrips, sync, dstate > 8 ? 768 : 1536, nTilesX, bwd_slots(dstate));
 }
 
 

@@ -466,7 +466,7 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
     const int rg = sh.dim / sh.n_groups;
     const int nChunks = (rg + 15) / 16;
     const int64_t nPC = (int64_t)sh.batch * sh.n_groups * nChunks;
-    const int bands = fwd_band_count(p.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate);
+    const int bands = fwd_band_count(p.schedule, (int64_t)sh.batch * sh.n_groups, nChunks, geo.nCY, p.workspace, sh.dstate, geo.nCX);
     if (bands > 0) {
         if (nPC * geo.nCY >= (int64_t)1 << 31) return SND_ERR_SHAPE;
         if (zero_words((int *)p.workspace, sync_words(nPC, geo.nCY), stream) != SND_OK) return SND_ERR_LAUNCH;

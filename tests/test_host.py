@@ -178,7 +178,9 @@ def test_backward_job_split():
     assert jobs(1, 256, 512, 512) == (64, 64)
     assert jobs(43, 192, 56, 56) == (3, 7)        # 516 chunks: 4 rounds of a third instead of 2 whole ones
     assert jobs(64, 192, 8, 56) == (0, 1)         # a single strip cannot be split
-    assert jobs(32, 192, 56, 56) == (0, 7)        # 384 chunks are all resident at once: a plane's bands are a chain
+    assert jobs(32, 192, 56, 56) == (7, 7)        # 384 chunks leave the chip short of waves: one job per strip
+    assert jobs(40, 192, 56, 56) == (0, 7)        # 480 chunks are all resident at once: a plane's bands are a chain
+    assert jobs(8, 768, 14, 14) == (0, 2)         # 384 chunks of two strips: nothing to run side by side
     assert jobs(85, 192, 56, 56) == (2, 7)        # 1020 chunks, but 129 of them pinned to each of four XCDs: 3 rounds
     assert jobs(128, 192, 56, 56) == (0, 7)       # 1536 chunks: three full rounds
 
@@ -194,6 +196,8 @@ def test_forward_job_split():
     assert sched(128, 192, 56, 56) == capi.SCHED_PLANE    # 1536: two full rounds
     assert sched(70, 192, 56, 56, N=8) == capi.SCHED_PLANE   # 840 of 1536 slots
     assert sched(2, 192, 200, 336) == capi.SCHED_STRIPS
+    assert sched(24, 192, 56, 56) == capi.SCHED_STRIPS    # 288 plane chunks: strips fill the chip better
+    assert sched(40, 192, 56, 56) == capi.SCHED_PLANE
     assert sched(70, 192, 8, 56) == capi.SCHED_PLANE      # one strip
 
 
@@ -213,7 +217,7 @@ def test_kernel_family_choice():
     assert family(64, 768, 14, 14, 4) == "tile"
     assert family(32, 256, 40, 40, 4) == "tile"
     assert family(64, 192, 56, 56, 4) == "tile"           # 768 one-wave blocks fill the chip in one round
-    assert family(16, 192, 56, 56, 4) == "wave"           # 192 blocks do not
+    assert family(4, 192, 56, 56, 4) == "wave"            # 48 blocks: the strip pipeline's ramp costs more than the rows
     assert family(64, 192, 56, 56, 2) == "wave"
     assert family(64, 192, 56, 56, 16) == "tile"
     assert family(1, 8, 9, 1500, 4, K=2) == "tile"         # wider than the wavefront kernels cover
