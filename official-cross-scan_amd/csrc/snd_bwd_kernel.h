@@ -296,6 +296,33 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // beside dD, at no cost in the sweep.
     float dw_acc = 0.f;
 
+    // dB, dC of a tile leave the block (summed over its channels) one tile late, from the partial sums that stay
+    // in LDS until the next sweep: after the next tile's inputs have arrived, so that the wait for those inputs
+    // does not also cover the acknowledgement of these atomics, which then complete under the sweep
+    // (4 % of the backward at B=2, D=192, 200x336 under the strip pipeline; nothing at B=64, 56x56).
+    int pI = -1, pJ = 0;                            // the tile whose partial sums are still in LDS
+    auto flush_bc = [&](int I_, int J_) __attribute__((always_inline)) {
+        SND_THREAD_MAPS(NP);
+        const int row = I_ * TE + pr, col = J_ * TE + pj;
+        const bool in = pr < TE && pj < TE && row < H && col < W;
+        const uint32_t o = mad24(mrow(row), W4, mcol(col) * 4);
+#pragma unroll
+        for (int k = 0; k < NBC; ++k) {
+            const int sn = wave_u + WPB * k;                        // scalar: folded into the base
+            float tb = 0.f, tc = 0.f;
+#pragma unroll
+            for (int w = 0; w < NPART; ++w) {
+                tb += sdB[w * NP * NSD + sn * NSD + px];
+                tc += sdC[w * NP * NSD + sn * NSD + px];
+            }
+            if (in && sn < N && !(SND_TILE_ABLATE & 1)) {
+                glb_add((float *)((char *)dBg + sn * HW4 + o), tb);
+                glb_add((float *)((char *)dCg + sn * HW4 + o), tc);
+            } else if (SND_TILE_ABLATE & 1) {
+                dbias_acc += tb + tc;               // keeps the values live
+            }
+        }
+    };
     for (int I = I_hi; I >= I_lo; --I) {
         const int r0 = I * TE;
         float GR[kRows], GsR[kRows];                // G, Gs at the column right of the tile
@@ -356,6 +383,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             }
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
             commit();
+            if (pI >= 0) flush_bc(pI, pJ);          // the previous tile's dB, dC
+            pI = I; pJ = J;
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
             if (handed && wave == 0) {
@@ -582,31 +611,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
             }
             }
-            // ---- dB, dC of this tile leave the block (summed over its channels)
-            {
-                SND_THREAD_MAPS(NP);
-                const int row = r0 + pr, col = j0 + pj;
-                const bool in = pr < TE && pj < TE && row < H && col < W;
-                const uint32_t o = mad24(mrow(row), W4, mcol(col) * 4);
-#pragma unroll
-                for (int k = 0; k < NBC; ++k) {
-                    const int sn = wave_u + WPB * k;                        // scalar: folded into the base
-                    float tb = 0.f, tc = 0.f;
-#pragma unroll
-                    for (int w = 0; w < NPART; ++w) {
-                        tb += sdB[w * NP * NSD + sn * NSD + px];
-                        tc += sdC[w * NP * NSD + sn * NSD + px];
-                    }
-                    if (in && sn < N && !(SND_TILE_ABLATE & 1)) {
-                        glb_add((float *)((char *)dBg + sn * HW4 + o), tb);
-                        glb_add((float *)((char *)dCg + sn * HW4 + o), tc);
-                    } else if (SND_TILE_ABLATE & 1) {
-                        dbias_acc += tb + tc;       // keeps the values live
-                    }
-                }
-            }
         }
     }
+    if (pI >= 0) flush_bc(pI, pJ);
 #undef DL
 #undef AEXP
 

@@ -66,6 +66,14 @@ __device__ __forceinline__ void stg(f16_t *base, int i, float v) { base[i] = (f1
 __device__ __forceinline__ float ldg_b(const float *base, uint32_t off) { return *(const float *)((const char *)base + off); }
 __device__ __forceinline__ float ldg_b(const bf16_t *base, uint32_t off) { return bf16_to_f32(((const bf16_t *)((const char *)base + off))->v); }
 __device__ __forceinline__ float ldg_b(const f16_t *base, uint32_t off) { return (float)*(const f16_t *)((const char *)base + off); }
+// The same load without the conversion, and the conversion: a value that is converted (or masked) where it is loaded
+// is waited for there; kept raw, it is waited for where it is first needed.
+__device__ __forceinline__ uint32_t ldraw_b(const float *base, uint32_t off) { return *(const uint32_t *)((const char *)base + off); }
+__device__ __forceinline__ uint32_t ldraw_b(const bf16_t *base, uint32_t off) { return *(const uint16_t *)((const char *)base + off); }
+__device__ __forceinline__ uint32_t ldraw_b(const f16_t *base, uint32_t off) { return *(const uint16_t *)((const char *)base + off); }
+__device__ __forceinline__ float raw_to_f32(const float *, uint32_t r) { return __builtin_bit_cast(float, r); }
+__device__ __forceinline__ float raw_to_f32(const bf16_t *, uint32_t r) { return __builtin_bit_cast(float, r << 16); }
+__device__ __forceinline__ float raw_to_f32(const f16_t *, uint32_t r) { return (float)__builtin_bit_cast(f16_t, (uint16_t)r); }
 __device__ __forceinline__ void stg_b(float *base, uint32_t off, float v) { *(float *)((char *)base + off) = v; }
 __device__ __forceinline__ void stg_b(bf16_t *base, uint32_t off, float v) { ((bf16_t *)((char *)base + off))->v = f32_to_bf16(v); }
 __device__ __forceinline__ void stg_b(f16_t *base, uint32_t off, float v) { *(f16_t *)((char *)base + off) = (f16_t)v; }

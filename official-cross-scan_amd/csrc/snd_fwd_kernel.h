@@ -146,14 +146,15 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     const float *myB = sB + n * NSTR;
     const float *myC = sC + n * NSTR;
 
-    // Raw values of a tile, held in registers between their global load and their LDS commit.
+    // Raw values of a tile, held in registers between their global load and their LDS commit: as loaded, neither
+    // converted nor masked, so that nothing touches them (and waits for them) before the commit.
     // Tiles are loaded in aligned pairs (columns 16m..16m+15, both tiles' loads issued together),
     // so that the two 32-byte halves of each 64-byte run are requested while the memory line is in
     // flight: a line is fetched from HBM twice per strip instead of four times.
     // (Only where it pays and fits: the 16-state whole-plane kernels, which are bandwidth-bound.)
     constexpr bool PAIR = NP == 16;
     constexpr int NHL = (kCkX + NP - 1) / NP;       // halo-row elements per thread (1; 2 with four lanes per channel)
-    struct Stage { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; };
+    struct Stage { uint32_t qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; };   // raw: masked and converted at commit
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto load_tile = [&](Stage &q, int I, int J) {
@@ -161,40 +162,30 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
-        // loads are always in bounds (clamped coordinates); values outside the plane become zero
+        // loads are always in bounds (clamped coordinates); commit() zeroes what lies outside the plane
         {
             const int row = r0 + pr, col = j0 + pj;
-            const bool in = pr < TE && pj < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
             const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
                 const int sn = wave_u + WPB * k, sc = min(sn, N - 1);       // scalar: folded into the base
-                const float vb = ldg_b((const T *)((const char *)Bb + sc * BsB), ob);
-                const float vc = ldg_b((const T *)((const char *)Cb + sc * CsB), oc);
-                q.qb[k] = (in && sn < N) ? vb : 0.f;
-                q.qc[k] = (in && sn < N) ? vc : 0.f;
+                q.qb[k] = ldraw_b((const T *)((const char *)Bb + sc * BsB), ob);
+                q.qc[k] = ldraw_b((const T *)((const char *)Cb + sc * CsB), oc);
             }
         }
 #pragma unroll
         for (int k = 0; k < NPX; ++k) {
             const int pp = n + NP * k;
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-            const bool ok = cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
-            const float vd = ldg_b(db, cDb + mad24(mr, DhB, mcB)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mcB));
-            q.qdl[k] = ok ? vd : 0.f;
-            q.qu[k] = ok ? vu : 0.f;
+            q.qdl[k] = ldraw_b(db, cDb + mad24(mr, DhB, mcB));
+            q.qu[k] = ldraw_b(ub, cUb + mad24(mr, UhB, mcB));
         }
 #pragma unroll
         for (int k = 0; k < NHL; ++k) {     // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
-            const int hj = n + NP * k;
-            q.qhalo[k] = 0.f;
-            if (hj < TE) {
-                const int row = r0 - 1, col = j0 + hj;
-                const float vd = ldg_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
-                q.qhalo[k] = (cvalid && row >= 0 && col < W) ? vd : 0.f;
-            }
+            const int row = r0 - 1, col = j0 + min(n + NP * k, TE - 1);
+            q.qhalo[k] = ldraw_b(db, cDb + mad24(mrow(max(row, 0)), DhB, mcol(min(col, W - 1)) * ESZ));
         }
     };
     // the pair of tiles that starts at (I, J), J even (or the single tile when not pairing)
@@ -210,7 +201,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             const float4 v0 = ld4_stream(src), v1 = ld4_stream(src + DN4);
             qxv[0] = v0.x; qxv[1] = v0.y; qxv[2] = v0.z; qxv[3] = v0.w;
             qxv[4] = v1.x; qxv[5] = v1.y; qxv[6] = v1.z; qxv[7] = v1.w;
-            qcorner = J > 0 ? src[((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8] : 0.f;   // last column of the tile on the left
+            qcorner = src[J > 0 ? ((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8 : 0];   // last column of the tile on the left (if any: masked at its use)
         }
     };
     // Strip pipeline: h of the row above tile (I, J), written by the block of strip I-1.  Fetched
@@ -231,8 +222,31 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
         for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, row[k], row[k + 1]);
     };
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
-    auto commit = [&](const Stage &q) {
+    auto commit = [&](const Stage &qr, int I, int J) {
         SND_THREAD_MAPS(NP);
+        struct { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; } q;
+        {   // to fp32; zero outside the plane, the tile (7 x 7 tiles) and the state / channel ranges
+            const int r0 = I * TE, j0 = J * TE;
+            const bool in = pr < TE && pj < TE && r0 + pr < H && j0 + pj < W;
+#pragma unroll
+            for (int k = 0; k < NBC; ++k) {
+                const bool ok = in && wave_u + WPB * k < N;
+                q.qb[k] = ok ? raw_to_f32((const T *)nullptr, qr.qb[k]) : 0.f;
+                q.qc[k] = ok ? raw_to_f32((const T *)nullptr, qr.qc[k]) : 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < NPX; ++k) {
+                const int pp = n + NP * k;
+                const bool ok = cvalid && (pp >> 3) < TE && (pp & 7) < TE && r0 + (pp >> 3) < H && j0 + (pp & 7) < W;
+                q.qdl[k] = ok ? raw_to_f32((const T *)nullptr, qr.qdl[k]) : 0.f;
+                q.qu[k] = ok ? raw_to_f32((const T *)nullptr, qr.qu[k]) : 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < NHL; ++k) {
+                const int hj = n + NP * k;
+                q.qhalo[k] = (hj < TE && cvalid && r0 > 0 && j0 + hj < W) ? raw_to_f32((const T *)nullptr, qr.qhalo[k]) : 0.f;
+            }
+        }
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
             const int sn = wave + WPB * k;
@@ -277,7 +291,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
         // free once it is committed, so the next pair's loads can be issued under its compute
         auto do_tile = [&](const int J, const Stage &mine, const bool last_of_pair) {
             const int j0 = J * TE;
-            commit(mine);
+            commit(mine, I, J);
             // first strip of a pipelined band: the row above comes from another block
             const bool handed = PIPE && I == I_begin && I > 0;
             if (handed && wave == 0) {
@@ -302,7 +316,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                     for (int j = 0; j < kCkX; ++j) hup[j] = __builtin_nanf("");
                 }
             } else {
-                corner = (I > 0) ? qcorner : 0.f;
+                corner = (I > 0 && J > 0) ? qcorner : 0.f;
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hup[j] = (I > 0) ? qxv[j] : 0.f;
             }
@@ -374,6 +388,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];
                 qcorner = 0.f;
             }
+            // The loads issued at the top of this tile have had the whole tile to arrive.  Waiting for them here, before
+            // this tile's stores are issued, keeps every later wait for a loaded value from also covering the
+            // acknowledgement of those stores (one counter counts both, and it is not decremented in order across
+            // loads and stores).
+            __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
             if (lvalid) {
                 // row checkpoint / carry to the next strip: h at the strip's last row
                 float *dst = xv + ((int64_t)I * geo.nCX + J) * DN8;
