@@ -39,7 +39,12 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename T, int NS, int CPL, bool VEC, bool DO32>
+// EVEN: the plane is a whole number of bands high and of 64-lane segments wide.  No row of a band and no lane is then
+// skipped, so no branch surrounds the stores and atomics of a row: every band issues the same memory instructions on
+// every path, and the waits the compiler derives for the prefetched loads count the instructions issued after them
+// instead of also waiting for the acknowledgement of the band's last stores and atomics (the counter is decremented
+// in order, and with a store on only some paths the wait has to assume it was not issued).
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
     // load a band's inputs one band ahead (with four states, or two columns per lane, the registers are needed elsewhere)
@@ -65,7 +70,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     // Mirrored order: this lane owns scan columns jm0 .. jm0+CPL-1 and walks them downwards (its local index t is
     // scan column jm0 + CPL-1-t); in natural order (row checkpoints, recomputation) lane l owns columns jn0 ...
     const int jm0 = (w * kSeg + 63 - lane) * CPL;
-    const bool jin = jm0 < W;
+    const bool jin = EVEN || jm0 < W;
     const int jc = jin ? jm0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
     const int jn0 = (w * kSeg + lane) * CPL;
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                if (i0 + r < H) {
+                if (EVEN || i0 + r < H) {
                     const float (&dln)[CPL] = dln_[r], (&dlun)[CPL] = dlun_[r];
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
@@ -287,12 +292,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         if (PF) load_band(nxt, max(band - 1, 0));
 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
-        const int rows = min(R, H - i0);             // rows of this band inside the plane
+        const int rows = EVEN ? R : min(R, H - i0);  // rows of this band inside the plane
         const int mlast = mad24(i0 + rows - 1, rs, r0m);
         uint32_t og = mad24(mlast, WB * rs, colB), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
 #pragma unroll
         for (int r = R - 1; r >= 0; --r) {
-            if (i0 + r < H) {
+            if (EVEN || i0 + r < H) {
                 float dov[CPL], dlu[CPL], qsum[CPL], psum[CPL];
                 unpack(cur.o[r], dov);
 #pragma unroll
@@ -391,6 +396,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 
     In sA;
     if (PF) load_band(sA, wg.nBands - 1);
+    // (nothing in flight on the way into the band loop: its first waits then follow the loop's own path as well)
+    if (PF && EVEN) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     lds_barrier();                                   // the zeroed slot
     if (multi)
         for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
@@ -442,8 +449,18 @@ template <typename T, int NS, int CPL, bool VEC>
 static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
-    if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, std::is_same<T, float>::value>), grid, block, 0, stream, p, wg);
+    constexpr bool F32 = std::is_same<T, float>::value;
+    constexpr int R = NS <= 1 ? 8 : 4;
+    // (the even-plane variant only where the loads are prefetched: it is their waits that it makes exact)
+    const bool even = NS <= 2 && CPL == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
+    if (even) {
+        constexpr bool E = NS <= 2 && CPL == 1;
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E>), grid, block, 0, stream, p, wg);
+    } else {
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false>), grid, block, 0, stream, p, wg);
+    }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
