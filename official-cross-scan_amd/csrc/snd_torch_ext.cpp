@@ -181,9 +181,13 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     at::Tensor out = merge ? torch::zeros({c.batch, c.dim / c.n_groups, c.nrows, c.ncols}, f32)
                            : torch::empty({c.batch, c.dim, c.nrows, c.ncols},
                                           u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
-    at::Tensor x = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
+    // x and x_sd are written (and later read) at equal offsets at the same time: one allocation, the second a few KiB
+    // past the 4 KiB-rounded end of the first, so that the pair never sits a multiple of 2 MiB apart (snd_plan.saved_skew_bytes)
+    const int64_t nX = c.plan.x_elems, oXsd = ((nX * 4 + 4095) / 4096 * 4096 + c.plan.saved_skew_bytes) / 4;
+    at::Tensor xbuf = torch::empty({oXsd + nX}, f32);
+    at::Tensor x = xbuf.narrow(0, 0, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
+    at::Tensor x_sd = xbuf.narrow(0, oXsd, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
     at::Tensor x_v = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_y, c.plan.xv_inner}, f32);
-    at::Tensor x_sd = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
 
     snd_fwd_params p;
     fill_fwd(p, c, u, delta, A, B, C, D_, delta_bias_, A_decay_, delta_softplus);
@@ -250,9 +254,12 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // so that a parameter gradient kept by the optimizer never pins the large buffer.
     const int64_t nA = (int64_t)dim * dstate, nBC = B.numel();
     auto round64 = [](int64_t v) { return (v + 63) / 64 * 64; };
-    at::Tensor accBC = torch::zeros({2 * round64(nBC)}, f32);
+    // (dC a chosen distance past the 4 KiB-rounded end of dB, snd_plan.dC_skew_bytes: the two are accumulated at equal
+    // offsets at the same time and must not sit a multiple of 2 MiB apart)
+    const int64_t oC = ((nBC * 4 + 4095) / 4096 * 4096 + c.plan.dC_skew_bytes) / 4;
+    at::Tensor accBC = torch::zeros({oC + round64(nBC)}, f32);
     at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
-    at::Tensor dC = accBC.narrow(0, round64(nBC), nBC).view(C.sizes());
+    at::Tensor dC = accBC.narrow(0, oC, nBC).view(C.sizes());
     const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim), oMerge = oDec + 64;
     at::Tensor accP = torch::zeros({oMerge + (merge ? round64(dim) : 0)}, f32);
     at::Tensor dA = accP.narrow(0, 0, nA).view({dim, dstate});
@@ -296,7 +303,7 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     if (B.scalar_type() != at::ScalarType::Float) {
         const at::Tensor cast = accBC.to(B.dtype());
         dBo = cast.narrow(0, 0, nBC).view(B.sizes());
-        dCo = cast.narrow(0, round64(nBC), nBC).view(C.sizes());
+        dCo = cast.narrow(0, oC, nBC).view(C.sizes());
     }
     std::vector<at::Tensor> result = {du, ddelta, dA, dBo, dCo, dD, ddelta_bias, dA_decay};
     if (dim != c.delta_dim) {

@@ -26,7 +26,8 @@ class Shape(C.Structure):
 class Plan(C.Structure):
     _fields_ = [("n_chunks_x", i32), ("n_chunks_y", i32), ("x_inner", i32), ("xv_inner", i32),
                 ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64),
-                ("fwd_workspace_bytes", i64), ("auto_schedule", i32), ("auto_bwd_jobs", i32)]
+                ("fwd_workspace_bytes", i64), ("auto_schedule", i32), ("auto_bwd_jobs", i32),
+                ("saved_skew_bytes", i64), ("dC_skew_bytes", i64)]
 
 
 class FwdParams(C.Structure):
@@ -130,6 +131,18 @@ def _stream(stream):
     return torch.cuda.current_stream().cuda_stream if stream is None else stream
 
 
+def carve_pair(shape_a, shape_b, skew_bytes, device, zero=False):
+    """Two fp32 tensors from one allocation, the second `skew_bytes` past the 4 KiB-rounded end of the first
+    (snd_plan.saved_skew_bytes / dC_skew_bytes: buffers the kernels stream at equal offsets at the same time must
+    not sit a multiple of 2 MiB apart, which is where separate large allocations land)."""
+    import math
+    import torch
+    na, nb = math.prod(shape_a), math.prod(shape_b)
+    off = ((na * 4 + 4095) // 4096 * 4096 + int(skew_bytes)) // 4
+    buf = (torch.zeros if zero else torch.empty)(off + nb, device=device, dtype=torch.float32)
+    return buf[:na].view(shape_a), buf[off:off + nb].view(shape_b)
+
+
 class FwdCall:
     """Outputs, saved state and the filled snd_fwd_params of one forward; launch() only enqueues."""
 
@@ -148,8 +161,10 @@ class FwdCall:
         else:
             self.out = torch.empty((Bt, Dm, u.shape[2], u.shape[3]), device=u.device, dtype=torch.float32 if out_float else u.dtype)
         self.x_v = torch.empty((Bt, Dm, N, plan.n_chunks_y, plan.xv_inner), **f32)
-        self.x = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
-        self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
+        self.x = self.x_sd = None
+        if save:
+            xs = (Bt, Dm, N, plan.n_chunks_x, plan.x_inner)
+            self.x, self.x_sd = carve_pair(xs, xs, plan.saved_skew_bytes, u.device)
         self.params = FwdParams()
         _fill_fwd(self.params, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, self.out,
                   self.x, self.x_v, self.x_sd, schedule, directions)
@@ -180,7 +195,7 @@ class BwdCall:
         self.du = torch.empty((u.shape[0], Dm, u.shape[2], u.shape[3]), device=u.device, dtype=u.dtype)
         self.ddelta = torch.empty_like(self.du)
         self.dA = torch.zeros_like(A)
-        self.dB, self.dC = torch.zeros(B.shape, **f32), torch.zeros(Cc.shape, **f32)
+        self.dB, self.dC = carve_pair(tuple(B.shape), tuple(Cc.shape), plan.dC_skew_bytes, u.device, zero=True)
         self.dD = torch.zeros_like(D) if D is not None else None
         self.dbias = torch.zeros(Dm, **f32) if delta_bias is not None else None
         self.ddec = torch.zeros_like(A_decay) if A_decay is not None else None
