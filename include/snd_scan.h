@@ -86,8 +86,8 @@ typedef struct snd_plan {
      * time.  Separate large allocations start 2 MiB apart or a multiple of it, which on an MI355X puts those
      * pairs of accesses in the same memory bank (measured: forward at B=64, D=192, 56x56, N=16 0.56 instead of
      * 0.51 ms; row-segment backward at 256 planes of 512x512, N=1 0.55 instead of 0.46 ms).  Carve each pair
-     * from one allocation instead: x_sd at x + round_up(bytes of x, 4096) + saved_skew_bytes (x_v anywhere),
-     * dC at dB + round_up(bytes of dB, 4096) + dC_skew_bytes.  Both are multiples of 256.  Results do not
+     * from one allocation instead: x_sd at x + round_up(bytes of x, 2 MiB) + saved_skew_bytes (x_v anywhere),
+     * dC at dB + round_up(bytes of dB, 2 MiB) + dC_skew_bytes (the distances the advice was measured at).  Both are multiples of 256.  Results do not
      * depend on placement. */
     int64_t saved_skew_bytes;
     int64_t dC_skew_bytes;

@@ -24,6 +24,9 @@ namespace {
 #define CHECK_SHAPE(x, ...) \
     TORCH_CHECK(x.sizes() == torch::IntArrayRef({__VA_ARGS__}), #x " must have shape (" #__VA_ARGS__ ")")
 
+// bytes rounded up to the 2 MiB grid that large allocations start on (the grid snd_plan's placement advice refers to)
+int64_t round_2mib(int64_t bytes) { return (bytes + (2 << 20) - 1) / (2 << 20) * (2 << 20); }
+
 int dtype_code(at::ScalarType t) {
     switch (t) {
         case at::ScalarType::Float: return SND_F32;
@@ -182,8 +185,8 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
                            : torch::empty({c.batch, c.dim, c.nrows, c.ncols},
                                           u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
     // x and x_sd are written (and later read) at equal offsets at the same time: one allocation, the second a few KiB
-    // past the 4 KiB-rounded end of the first, so that the pair never sits a multiple of 2 MiB apart (snd_plan.saved_skew_bytes)
-    const int64_t nX = c.plan.x_elems, oXsd = ((nX * 4 + 4095) / 4096 * 4096 + c.plan.saved_skew_bytes) / 4;
+    // past the 2 MiB-rounded end of the first, so that the pair never sits a multiple of 2 MiB apart (snd_plan.saved_skew_bytes)
+    const int64_t nX = c.plan.x_elems, oXsd = (round_2mib(nX * 4) + c.plan.saved_skew_bytes) / 4;
     at::Tensor xbuf = torch::empty({oXsd + nX}, f32);
     at::Tensor x = xbuf.narrow(0, 0, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
     at::Tensor x_sd = xbuf.narrow(0, oXsd, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
@@ -254,9 +257,9 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // so that a parameter gradient kept by the optimizer never pins the large buffer.
     const int64_t nA = (int64_t)dim * dstate, nBC = B.numel();
     auto round64 = [](int64_t v) { return (v + 63) / 64 * 64; };
-    // (dC a chosen distance past the 4 KiB-rounded end of dB, snd_plan.dC_skew_bytes: the two are accumulated at equal
+    // (dC a chosen distance past the 2 MiB-rounded end of dB, snd_plan.dC_skew_bytes: the two are accumulated at equal
     // offsets at the same time and must not sit a multiple of 2 MiB apart)
-    const int64_t oC = ((nBC * 4 + 4095) / 4096 * 4096 + c.plan.dC_skew_bytes) / 4;
+    const int64_t oC = (round_2mib(nBC * 4) + c.plan.dC_skew_bytes) / 4;
     at::Tensor accBC = torch::zeros({oC + round64(nBC)}, f32);
     at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
     at::Tensor dC = accBC.narrow(0, oC, nBC).view(C.sizes());

@@ -132,13 +132,13 @@ def _stream(stream):
 
 
 def carve_pair(shape_a, shape_b, skew_bytes, device, zero=False):
-    """Two fp32 tensors from one allocation, the second `skew_bytes` past the 4 KiB-rounded end of the first
+    """Two fp32 tensors from one allocation, the second `skew_bytes` past the 2 MiB-rounded end of the first
     (snd_plan.saved_skew_bytes / dC_skew_bytes: buffers the kernels stream at equal offsets at the same time must
     not sit a multiple of 2 MiB apart, which is where separate large allocations land)."""
     import math
     import torch
     na, nb = math.prod(shape_a), math.prod(shape_b)
-    off = ((na * 4 + 4095) // 4096 * 4096 + int(skew_bytes)) // 4
+    off = ((na * 4 + (2 << 20) - 1) // (2 << 20) * (2 << 20) + int(skew_bytes)) // 4
     buf = (torch.zeros if zero else torch.empty)(off + nb, device=device, dtype=torch.float32)
     return buf[:na].view(shape_a), buf[off:off + nb].view(shape_b)
 
