@@ -375,22 +375,44 @@ __host__ inline bool use_strip_pipeline(int schedule, int64_t planeBlocks, int n
 // whole-plane blocks leaves slots idle (backward, 768 chunks: two rounds, the second half empty);
 // cutting every plane into a few bands of strips, handed over like strips but only at band ends, lets
 // the ticket order pack them (768 x 2 bands: three rounds of half the length).
+// Cost of q = jobs / slots rounds of equal jobs, in job lengths: full rounds cost one each; a last, partly filled
+// round runs faster, because a block shares its CU with fewer others (k of the L blocks a CU holds: a share
+// `serial` of a block's time does not depend on k - 0.6 in the issue-bound backward, where one block per CU takes
+// 0.83 of the time it takes beside a second one, 0.15 in the bandwidth-bound forward); a round after the first
+// costs a tenth more (tail of the round before).  Measured, 192 channels of 56x56, 16 states, whole planes, in
+// units of a full round: backward 1.72 / 1.74 / 1.75 / 2.09 / 2.13 / 2.74 / 3.16 / 3.25 at 576 / 672 / 768 / 864 /
+// 960 / 1152 / 1344 / 1536 plane chunks on 512 slots; forward 0.71 / 0.95 / 0.99 / 1.00 / 1.34 / 1.36 / 1.62 / 1.89 /
+// 1.97 at 480 .. 1536 on 768 slots.
+__host__ inline double rounds_cost(double q, int perCU, double serial) {
+    const double full = (double)(int64_t)q, frac = q - full;
+    if (frac < 1e-9) return full;
+    int k = (int)(frac * perCU + 0.999999);
+    if (k > perCU) k = perCU;
+    return full + serial + (1.0 - serial) * k / perCU + (full >= 1.0 ? 0.1 : 0.0);
+}
 __host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nStrips, const void *sync, int64_t slots,
                                int nTilesX = 0, int64_t bwdSlots = 512) {
     const int64_t planeBlocks = nPairs * nChunks;
     if (schedule == kSchedPlane || sync == nullptr || nStrips < 2) return 0;
     if (schedule == kSchedStrips) return nStrips;
     if (schedule != kSchedBands && use_strip_pipeline(kSchedAuto, planeBlocks, nStrips, sync, nTilesX, bwdSlots)) return nStrips;
+    const bool forward = slots > bwdSlots;
+    const int perCU = (int)(slots / 256);
+    const double serial = forward ? 0.15 : 0.6;
+    // the forward holds more blocks than the backward: between the backward's slots and 0.8 x its own, whole planes
+    // put a third block on some CUs while the strips of a wide plane spread evenly (576 plane chunks: 0.48 -> 0.44 ms)
+    const bool wide = nTilesX > 0 && (int64_t)nStrips * nTilesX >= 2 * ((int64_t)nStrips + nTilesX - 1);
+    if (schedule != kSchedBands && forward && wide && planeBlocks > bwdSlots && planeBlocks * 5 <= slots * 4) return nStrips;
     // whole planes: every (batch, group) pair is pinned to one XCD (an eighth of the slots), so the rounds
     // are those of the fullest XCD (backward, 340 pairs x 3 chunks: 129 blocks there, three rounds)
     int best = 1;
-    double best_cost = (double)(((nPairs + 7) / 8 * nChunks + slots / 8 - 1) / (slots / 8));
+    double best_cost = rounds_cost((double)((nPairs + 7) / 8 * nChunks) / (double)(slots / 8), perCU, serial);
     for (int nb = 2; nb <= 4 && nb <= nStrips; ++nb) {
         // rounds of jobs of length 1/nb (drawn from queues that balance the XCDs), never less than the
         // chain of one plane's bands, and a few percent per extra band for the hand-over
-        double cost = (double)((planeBlocks * nb + slots - 1) / slots) / nb;
+        double cost = rounds_cost((double)(planeBlocks * nb) / (double)slots, perCU, serial) / nb;
         cost = (cost < 1.0 ? 1.0 : cost) * (1.0 + 0.03 * (nb - 1));
-        if (cost < best_cost * 0.95) { best = nb; best_cost = cost; }
+        if (cost < best_cost * 0.96) { best = nb; best_cost = cost; }
     }
     if (schedule == kSchedBands) return best > 1 ? best : 2;
     return best > 1 ? best : 0;

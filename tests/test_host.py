@@ -196,6 +196,8 @@ def test_backward_job_split():
     assert jobs(8, 768, 14, 14) == (0, 2)         # 384 chunks of two strips: nothing to run side by side
     assert jobs(85, 192, 56, 56) == (2, 7)        # 1020 chunks, but 129 of them pinned to each of four XCDs: 3 rounds
     assert jobs(128, 192, 56, 56) == (0, 7)       # 1536 chunks: three full rounds
+    assert jobs(72, 192, 56, 56) == (2, 7)        # 864: the second round of whole planes would be 0.69 full and run at full-round pace
+    assert jobs(80, 192, 56, 56) == (0, 7)        # 960: nearly two full rounds either way
 
 
 def test_forward_job_split():
@@ -207,7 +209,11 @@ def test_forward_job_split():
     assert sched(64, 192, 56, 56) == capi.SCHED_PLANE     # 768 plane chunks on 768 slots
     assert sched(70, 192, 56, 56) == capi.SCHED_BANDS     # 840: a second round for 72 blocks otherwise
     assert sched(128, 192, 56, 56) == capi.SCHED_PLANE    # 1536: two full rounds
-    assert sched(70, 192, 56, 56, N=8) == capi.SCHED_PLANE   # 840 of 1536 slots
+    assert sched(70, 192, 56, 56, N=8) == capi.SCHED_STRIPS  # 840 chunks, between the backward's 768 slots and 0.8 x 1536 (measured 0.45 against 0.51 ms)
+    assert sched(64, 192, 56, 56, N=8) == capi.SCHED_PLANE   # 768 of 1536 slots
+    assert sched(48, 192, 56, 56) == capi.SCHED_STRIPS    # 576 chunks: whole planes would put a third block on a quarter of the CUs
+    assert sched(56, 192, 56, 56) == capi.SCHED_PLANE     # 672: beyond 0.8 x 768
+    assert sched(112, 192, 56, 56) == capi.SCHED_BANDS    # 1344: 1.75 rounds
     assert sched(2, 192, 200, 336) == capi.SCHED_STRIPS
     assert sched(24, 192, 56, 56) == capi.SCHED_STRIPS    # 288 plane chunks: strips fill the chip better
     assert sched(40, 192, 56, 56) == capi.SCHED_PLANE
