@@ -403,6 +403,10 @@ __host__ inline int band_count(int schedule, int64_t nPairs, int nChunks, int nS
     // put a third block on some CUs while the strips of a wide plane spread evenly (576 plane chunks: 0.48 -> 0.44 ms)
     const bool wide = nTilesX > 0 && (int64_t)nStrips * nTilesX >= 2 * ((int64_t)nStrips + nTilesX - 1);
     if (schedule != kSchedBands && forward && wide && planeBlocks > bwdSlots && planeBlocks * 5 <= slots * 4) return nStrips;
+    // the 8-state forward (six 128-thread blocks per CU) prefers strips up to one full round of wide planes: 192 channels
+    // of 56x56, bf16, whole planes / strips 0.407 / 0.380 ms at 768 plane chunks, 0.825 / 0.704 at 1536 (fp32 0.415 /
+    // 0.414, 0.883 / 0.783); 28x28 at 1536: 0.232 / 0.222; beyond a round whole planes or bands are as good or better
+    if (schedule != kSchedBands && forward && perCU >= 6 && wide && planeBlocks <= slots) return nStrips;
     // whole planes: every (batch, group) pair is pinned to one XCD (an eighth of the slots), so the rounds
     // are those of the fullest XCD (backward, 340 pairs x 3 chunks: 129 blocks there, three rounds)
     int best = 1;

@@ -210,7 +210,10 @@ def test_forward_job_split():
     assert sched(70, 192, 56, 56) == capi.SCHED_BANDS     # 840: a second round for 72 blocks otherwise
     assert sched(128, 192, 56, 56) == capi.SCHED_PLANE    # 1536: two full rounds
     assert sched(70, 192, 56, 56, N=8) == capi.SCHED_STRIPS  # 840 chunks, between the backward's 768 slots and 0.8 x 1536 (measured 0.45 against 0.51 ms)
-    assert sched(64, 192, 56, 56, N=8) == capi.SCHED_PLANE   # 768 of 1536 slots
+    assert sched(64, 192, 56, 56, N=8) == capi.SCHED_STRIPS  # the 8-state forward prefers strips up to one full round of wide planes
+    assert sched(128, 192, 56, 56, N=8) == capi.SCHED_STRIPS # 1536 of 1536 slots (measured 0.70 against 0.83 ms)
+    assert sched(256, 192, 56, 56, N=8) == capi.SCHED_PLANE  # two full rounds
+    assert sched(64, 768, 14, 14, N=8) == capi.SCHED_PLANE   # 2 x 2 tiles: nothing to run side by side
     assert sched(48, 192, 56, 56) == capi.SCHED_STRIPS    # 576 chunks: whole planes would put a third block on a quarter of the CUs
     assert sched(56, 192, 56, 56) == capi.SCHED_PLANE     # 672: beyond 0.8 x 768
     assert sched(112, 192, 56, 56) == capi.SCHED_BANDS    # 1344: 1.75 rounds
