@@ -82,14 +82,13 @@ typedef struct snd_plan {
                                                   the backward runs WAVEFRONT too and needs no workspace),
                                                   n_chunks_y = one per strip, 2-4 = bands */
     /* Placement advice for callers that allocate the buffers (no counterpart in the reference, which leaves
-     * placement to torch::empty).  The kernels stream x and x_sd, and dB and dC, at equal offsets at the same
-     * time.  Separate large allocations start 2 MiB apart or a multiple of it, which on an MI355X puts those
-     * pairs of accesses in the same memory bank (measured: forward at B=64, D=192, 56x56, N=16 0.56 instead of
-     * 0.51 ms; row-segment backward at 256 planes of 512x512, N=1 0.55 instead of 0.46 ms).  Carve each pair
-     * from one allocation instead: x_sd at x + round_up(bytes of x, 2 MiB) + saved_skew_bytes (x_v anywhere),
-     * dC at dB + round_up(bytes of dB, 2 MiB) + dC_skew_bytes (the distances the advice was measured at).  Both are multiples of 256.  Results do not
-     * depend on placement. */
-    int64_t saved_skew_bytes;
+     * placement to torch::empty).  The backward accumulates dB and dC at equal offsets at the same time.
+     * Separate large allocations start 2 MiB apart or a multiple of it, which on an MI355X puts the two
+     * atomics of a pixel in the same memory bank: the row-segment backward at 256 planes of 512x512, N=1 takes
+     * 0.55-0.63 ms that way and 0.46-0.50 ms with dC half an fp32 row further on.  Put both in one allocation,
+     * dC at dB + round_up(bytes of dB, 2 MiB) + dC_skew_bytes (a multiple of 256; the distance the advice was
+     * measured at).  Results do not depend on placement, and no other pair of buffers shows the effect
+     * (`python bench.py --placement-probe`). */
     int64_t dC_skew_bytes;
 } snd_plan;
 

@@ -249,8 +249,7 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     // Placement advice (see the header).  Measured on dC - dB modulo the fp32 row of dB/dC: the row-segment
     // backward is fastest half a row apart when a row is 2 KiB or more (512 x 512: 0.46 ms at 1 KiB + k * 2 KiB,
     // 0.55 at k * 2 KiB), and with narrower rows at 16 KiB (0 .. 9 KiB cost some shapes 10 % and gain others as much);
-    // the tile kernels and the saved state are indifferent beyond 1 KiB.
-    plan->saved_skew_bytes = 5 * 1024;
+    // the tile kernels are indifferent.
     const int64_t row = (int64_t)shape->ncols * 4;
     plan->dC_skew_bytes = plan->auto_schedule != SND_SCHED_WAVEFRONT ? 5 * 1024 : row >= 2048 ? (row / 2 + 255) / 256 * 256 : 16 * 1024;
     return SND_OK;

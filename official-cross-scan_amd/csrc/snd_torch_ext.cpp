@@ -184,13 +184,9 @@ std::vector<at::Tensor> selective_scan_fwd(const at::Tensor &u, const at::Tensor
     at::Tensor out = merge ? torch::zeros({c.batch, c.dim / c.n_groups, c.nrows, c.ncols}, f32)
                            : torch::empty({c.batch, c.dim, c.nrows, c.ncols},
                                           u.options().dtype(out_float ? at::ScalarType::Float : u.scalar_type()));
-    // x and x_sd are written (and later read) at equal offsets at the same time: one allocation, the second a few KiB
-    // past the 2 MiB-rounded end of the first, so that the pair never sits a multiple of 2 MiB apart (snd_plan.saved_skew_bytes)
-    const int64_t nX = c.plan.x_elems, oXsd = (round_2mib(nX * 4) + c.plan.saved_skew_bytes) / 4;
-    at::Tensor xbuf = torch::empty({oXsd + nX}, f32);
-    at::Tensor x = xbuf.narrow(0, 0, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
-    at::Tensor x_sd = xbuf.narrow(0, oXsd, nX).view({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner});
+    at::Tensor x = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
     at::Tensor x_v = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_y, c.plan.xv_inner}, f32);
+    at::Tensor x_sd = torch::empty({c.batch, c.dim, c.dstate, c.plan.n_chunks_x, c.plan.x_inner}, f32);
 
     snd_fwd_params p;
     fill_fwd(p, c, u, delta, A, B, C, D_, delta_bias_, A_decay_, delta_softplus);

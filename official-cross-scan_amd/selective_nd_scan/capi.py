@@ -27,7 +27,7 @@ class Plan(C.Structure):
     _fields_ = [("n_chunks_x", i32), ("n_chunks_y", i32), ("x_inner", i32), ("xv_inner", i32),
                 ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64),
                 ("fwd_workspace_bytes", i64), ("auto_schedule", i32), ("auto_bwd_jobs", i32),
-                ("saved_skew_bytes", i64), ("dC_skew_bytes", i64)]
+                ("dC_skew_bytes", i64)]
 
 
 class FwdParams(C.Structure):
@@ -133,8 +133,8 @@ def _stream(stream):
 
 def carve_pair(shape_a, shape_b, skew_bytes, device, zero=False):
     """Two fp32 tensors from one allocation, the second `skew_bytes` past the 2 MiB-rounded end of the first
-    (snd_plan.saved_skew_bytes / dC_skew_bytes: buffers the kernels stream at equal offsets at the same time must
-    not sit a multiple of 2 MiB apart, which is where separate large allocations land)."""
+    (snd_plan.dC_skew_bytes: dB and dC, accumulated at equal offsets at the same time, must not sit a multiple of
+    2 MiB apart, which is where separate large allocations land)."""
     import math
     import torch
     na, nb = math.prod(shape_a), math.prod(shape_b)
@@ -161,10 +161,8 @@ class FwdCall:
         else:
             self.out = torch.empty((Bt, Dm, u.shape[2], u.shape[3]), device=u.device, dtype=torch.float32 if out_float else u.dtype)
         self.x_v = torch.empty((Bt, Dm, N, plan.n_chunks_y, plan.xv_inner), **f32)
-        self.x = self.x_sd = None
-        if save:
-            xs = (Bt, Dm, N, plan.n_chunks_x, plan.x_inner)
-            self.x, self.x_sd = carve_pair(xs, xs, plan.saved_skew_bytes, u.device)
+        self.x = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
+        self.x_sd = torch.empty((Bt, Dm, N, plan.n_chunks_x, plan.x_inner), **f32) if save else None
         self.params = FwdParams()
         _fill_fwd(self.params, shape, u, delta, A, B, Cc, D, delta_bias, delta_softplus, A_decay, self.out,
                   self.x, self.x_v, self.x_sd, schedule, directions)

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
-    assert C.sizeof(capi.Plan) == 80
+    assert C.sizeof(capi.Plan) == 72
     assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4 + 8
     assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8 + 8
 
@@ -31,7 +31,7 @@ def test_struct_layouts_match_header_sizes():
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
-    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs", "saved_skew_bytes", "dC_skew_bytes"]),
+    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs", "dC_skew_bytes"]),
               ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared", "merge", "merge_weights"]),
               ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes", "dmerge"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
@@ -52,16 +52,15 @@ def test_struct_layouts_match_the_c_compiler(tmp_path):
 
 
 def test_placement_advice():
-    """x_sd and dC are to be carved a few KiB past the 4 KiB-rounded end of x and dB: multiples of 256 bytes, never
-    a multiple of 2 MiB; half an fp32 row for the row-segment kernels on rows of 2 KiB or more."""
+    """dC is to be carved past the 2 MiB-rounded end of dB by a multiple of 256 bytes that is no multiple of 2 MiB: half
+    an fp32 row for the row-segment kernels on rows of 2 KiB or more."""
     for shp, want in (((64, 192, 56, 56, 16, 4, 192, capi.SND_F32), 5120), ((1, 256, 512, 512, 1, 4, 256, capi.SND_BF16), 1024),
                       ((1, 64, 1024, 1024, 1, 4, 64, capi.SND_BF16), 2048), ((8, 192, 64, 64, 1, 4, 192, capi.SND_BF16), 16384),
                       ((64, 768, 14, 14, 1, 4, 768, capi.SND_BF16), 5120)):
         st, plan = capi.make_plan(capi.Shape(*shp))
         assert st == 0
-        assert plan.saved_skew_bytes == 5120 and plan.dC_skew_bytes == want
-        for v in (plan.saved_skew_bytes, plan.dC_skew_bytes):
-            assert v % 256 == 0 and 0 < v < (2 << 20)
+        assert plan.dC_skew_bytes == want
+        assert plan.dC_skew_bytes % 256 == 0 and 0 < plan.dC_skew_bytes < (2 << 20)
 
 
 @pytest.mark.parametrize("H,W,ncx,ncy", [(56, 56, 7, 7), (14, 14, 2, 2), (200, 336, 42, 25), (1, 37, 5, 1), (512, 512, 64, 64),
