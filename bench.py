@@ -8,7 +8,9 @@ reference's fwd/bwd bindings would pay them) on synthetic inputs already residen
 Prints ONE JSON line.  `value` is the algorithmic HBM rate of the whole step:
     bytes = (2eP + 2eQ + 4P) + (4eP + 4eQ + 4P),  P = B*D*H*W, Q = B*K*N*H*W, e = input bytes
 (compulsory tensor I/O only) divided by the mean step time.  `roofline` is the same figure for the
-dominant kernel alone (the backward), from HIP events around its launches on the launch stream, with
+dominant kernel alone (the backward), from one pair of HIP events on the launch stream around K back-to-back
+launches of it through the C ABI (after W untimed ones; defaults K = 50, W = 20: the clocks settle over the first
+10-15 steps after the host-side input generation), with
 a second leg beside it: vector-ALU wave-instructions per second against the published FP32 vector peak
 (157.3 TFLOP/s = 1228.9 G wave-wide multiply-adds per second: a SIMD retires one 64-lane FP32 instruction
 per two cycles), with the rate `--issue-probe` measures for a pure multiply-add stream on all CUs beside
@@ -187,8 +189,10 @@ def placement_probe(torch, dev, workload):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (the clocks settle over the first 10-15 steps after the seconds of host-side input generation: c1 takes 2.25 ms
+    # for its second step and 1.89 ms from the fourteenth on; the warm-up covers that)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
@@ -269,22 +273,26 @@ def main():
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # kernel-only durations: HIP events on the launch stream around each launch through the C ABI
+    # kernel-only durations: HIP events on the launch stream around launches through the C ABI
     fcall = capi.FwdCall(u, delta, A, B, C, D, bias, True, True, None, True, sched)
     fcall.launch()
     bcall = capi.BwdCall(u, delta, A, B, C, D, bias, dout, fcall.x, fcall.x_v, True, None, fcall.x_sd, sched)
     stream = torch.cuda.current_stream()
-    kf, kb = [], []
-    for i in range(args.warmup + args.steps):
-        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-        bcall.zero()
-        e[0].record(stream); fcall.launch(); e[1].record(stream)
-        e[2].record(stream); bcall.launch_kernel_only(); e[3].record(stream)
+    # (each kernel launched back to back between ONE pair of events and divided by the count: a pair of events around
+    # every launch would add the event and launch gaps, a few microseconds, to every figure)
+    def kernel_ms(launch):
+        for _ in range(args.warmup):
+            launch()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(args.steps):
+            launch()
+        e1.record(stream)
         torch.cuda.synchronize()
-        if i >= args.warmup:
-            kf.append(e[0].elapsed_time(e[1]))
-            kb.append(e[2].elapsed_time(e[3]))
-    kf_ms, kb_ms = sum(kf) / len(kf), sum(kb) / len(kb)
+        return e0.elapsed_time(e1) / args.steps
+    kf_ms = kernel_ms(fcall.launch)
+    bcall.zero()
+    kb_ms = kernel_ms(bcall.launch_kernel_only)     # (the accumulated gradients are not cleared in between: timing only)
 
     value = (fb + bb) / (ms * 1e-3) / 1e9
     achieved = bb / (kb_ms * 1e-3) / 1e9
