@@ -35,6 +35,9 @@
 
 namespace snd {
 
+constexpr int kWaveShare = 4;                        // channels of a block that share their dB / dC atomics
+constexpr int kWaveShareWaves = 4;                   // waves of such a block (one segment per channel)
+
 __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -44,26 +47,42 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 // every path, and the waits the compiler derives for the prefetched loads count the instructions issued after them
 // instead of also waiting for the acknowledgement of the band's last stores and atomics (the counter is decremented
 // in order, and with a store on only some paths the wait has to assume it was not issued).
-template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN>
+//
+// CHB > 1: the block holds CHB channels of one (batch, group) pair, each with its own waves.  The channels' dB / dC
+// contributions of a band meet in LDS and leave as one atomic per element and block: the atomics are performed at
+// the memory side, line by line, and cost the kernel a third to a half of its time when every channel issues its own.
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
+    static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
+    constexpr int kItems = R * NS * 2;               // dB and dC rows of a band
+    constexpr int kXBuf = CHB == 1 ? 1 : NS == 4 ? 1 : 2;   // (with two buffers one barrier per band is enough)
+    constexpr int kXWaves = CHB == 1 ? 1 : kWaveShareWaves;
+    __shared__ float sX[kXBuf][kXWaves][CHB == 1 ? 1 : kItems][CHB == 1 ? 1 : 64];
     // load a band's inputs one band ahead (with four states, or two columns per lane, the registers are needed elsewhere)
     constexpr bool PF = NS <= 2 && CPL == 1;
     // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and
     // state.  Wave w writes slot w and reads slot w+1; the slot after the last wave stays zero.
-    __shared__ float4 sHO[2][kMaxSeg + 1][R][NS];
+    __shared__ float4 sHO[2][CHB][kMaxSeg + 1][R][NS];
 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
-    int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
-    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
-    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nseg = wg.nseg;
+    const int lane = threadIdx.x & 63, wi = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int kc = CHB > 1 ? wi / nseg : 0, w = wi - kc * nseg;     // channel of the block, segment of the channel
+    int pair, chunk;
+    if (!wave_job(blockIdx.x, sh.batch * G, (rg + CHB - 1) / CHB, pair, chunk)) return;
+    chunk = chunk * CHB + kc;
+    // A block past the last channel of its group repeats that channel (identical du / ddelta stores) and adds nothing.
+    const bool active = CHB == 1 || chunk < rg;
+    chunk = min(chunk, rg - 1);
+    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
     const bool multi = nseg > 1;
-    if (threadIdx.x < 2 * R * NS) (&sHO[0][0][0][0])[((threadIdx.x / (R * NS)) * (kMaxSeg + 1) + nseg) * R * NS + threadIdx.x % (R * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (threadIdx.x < 2 * R * NS)
+#pragma unroll
+        for (int q = 0; q < CHB; ++q) sHO[threadIdx.x / (R * NS)][q][nseg][threadIdx.x % (R * NS) / NS][threadIdx.x % NS] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     const bool fv = f.directions == SND_DIR_CORNERS && (g & 2), fh = f.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
@@ -310,7 +329,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
-                    const float4 in = sHO[(step + 1) & 1][w + 1][r][n];
+                    const float4 in = sHO[(step + 1) & 1][kc][w + 1][r][n];
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
                     const bool live = NS != 4 || n < N;
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
@@ -354,7 +373,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         ya[t] = dbu * dlu[t];                                          // dB, dC contributions (reusing the arrays)
                         ys[t] = dov[t] * fmaf(0.25f, bu[t], hs);
                     }
-                    if (jin && live && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
+                    if (CHB > 1) {
+                        sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2][lane] = active ? ya[0] : 0.f;
+                        sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2 + 1][lane] = active ? ys[0] : 0.f;
+                    } else if (jin && live && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
 #pragma unroll
                         for (int e = 0; e < CPL; ++e) {                                // memory order
                             const int t = fh ? e : CPL - 1 - e;
@@ -366,7 +388,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                     GdEdge[n] = in.x;
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) { Gd[n][t] = Gt[t]; ad[n][t] = a[t]; }
-                    if (hands_over && lane == 63) sHO[step & 1][w][r][n] = make_float4(Gt[CPL - 1], Gst[CPL - 1], a[CPL - 1], 0.f);
+                    if (hands_over && lane == 63) sHO[step & 1][kc][w][r][n] = make_float4(Gt[CPL - 1], Gst[CPL - 1], a[CPL - 1], 0.f);
                 }
                 if (jin) {
                     float duv[CPL], ddl[CPL];
@@ -391,7 +413,23 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                 o4 -= W4;
             }
         }
-        if (multi) { lds_barrier(); ++step; }
+        if (CHB > 1) {
+            // Wave kc of a segment adds up rows kc, kc + CHB, ... of what the segment's CHB waves left and issues
+            // their atomics.
+            lds_barrier();
+            if (!(SND_WAVE_ABLATE & 64))
+#pragma unroll
+            for (int m = 0; m < kItems / CHB; ++m) {
+                const int it = m * CHB + kc, r = it / (2 * NS), n = (it >> 1) % NS;
+                float v = 0.f;
+#pragma unroll
+                for (int q = 0; q < CHB; ++q) v += sX[kXBuf == 2 ? step & 1 : 0][w + q * nseg][it][lane];
+                float *dst = (float *)((char *)((it & 1) ? dCg : dBg) + n * HW4 + (int64_t)mad24(mad24(i0 + r, rs, r0m), W * 4, (int)col4));
+                if (jin && (EVEN || i0 + r < H) && (NS != 4 || n < N)) wave_glb_add(dst, v);
+            }
+            if (kXBuf == 1) lds_barrier();
+            ++step;
+        } else if (multi) { lds_barrier(); ++step; }
     };
 
     In sA;
@@ -400,7 +438,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     if (PF && EVEN) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     lds_barrier();                                   // the zeroed slot
     if (multi)
-        for (int e = 0; e < nseg - 1 - w; ++e) lds_barrier();
+        for (int e = 0; e < (nseg - 1 - w) * (CHB > 1 && kXBuf == 1 ? 2 : 1); ++e) lds_barrier();
     if (PF) {
         In sB;
         for (int band = wg.nBands - 1; band >= 0; band -= 2) {
@@ -411,17 +449,17 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         for (int band = wg.nBands - 1; band >= 0; --band) do_band(sA, sA, band);
     }
     if (multi)
-        for (int e = 0; e < w; ++e) lds_barrier();
+        for (int e = 0; e < w * (CHB > 1 && kXBuf == 1 ? 2 : 1); ++e) lds_barrier();
 
     // ---- per-channel sums leave the kernel: one atomic per wave and value
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
         const float t = wave_sum_to_last(dA_acc[n]);
-        if (lane == 63 && n < N) wave_glb_add(p.dA + (int64_t)c * N + n, t);
+        if (lane == 63 && n < N && active) wave_glb_add(p.dA + (int64_t)c * N + n, t);
     }
     {
         const float td = wave_sum_to_last(dD_acc), tb = wave_sum_to_last(dbias_acc);
-        if (lane == 63) {
+        if (lane == 63 && active) {
             if (p.dD) wave_glb_add(p.dD + c, td);
             if (p.ddelta_bias) wave_glb_add(p.ddelta_bias + c, tb);
         }
@@ -429,12 +467,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         // linear in u (D*u plus a recurrence linear in B*delta'*u) that inner product equals <du, u>.
         if (merge && p.dmerge) {
             const float tw = wave_sum_to_last(dw_acc);
-            if (lane == 63) wave_glb_add(p.dmerge + c, tw);
+            if (lane == 63 && active) wave_glb_add(p.dmerge + c, tw);
         }
     }
     if (want_decay) {
         const float t = wave_sum_to_last(dec_acc);
-        if (lane == 63) wave_glb_add(p.dA_decay, t / f.A_decay[0]);
+        if (lane == 63 && active) wave_glb_add(p.dA_decay, t / f.A_decay[0]);
     }
 }
 
@@ -445,23 +483,37 @@ static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::
     return true;
 }
 
-template <typename T, int NS, int CPL, bool VEC>
-static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+// Channels per block.  Sharing the atomics needs the channels' waves in one block, and a block may hold
+// kWaveShareWaves of them; with fewer planes than the GPU holds waves, one channel per block spreads them further.
+static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
+    const int64_t waves = (int64_t)sh.batch * sh.dim * wg.nseg;
+    return wg.cpl == 1 && wg.nseg * kWaveShare <= kWaveShareWaves && waves >= 2048 ? kWaveShare : 1;
+}
+
+template <typename T, int NS, int CPL, bool VEC, int CHB>
+static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
-    const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
+    const int rg = sh.dim / sh.n_groups;
+    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + CHB - 1) / CHB)), block(64 * wg.nseg * CHB);
     constexpr bool F32 = std::is_same<T, float>::value;
     constexpr int R = NS <= 1 ? 8 : 4;
     // (the even-plane variant only where the loads are prefetched: it is their waits that it makes exact)
     const bool even = NS <= 2 && CPL == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
     if (even) {
         constexpr bool E = NS <= 2 && CPL == 1;
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E>), grid, block, 0, stream, p, wg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E, CHB>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E, CHB>), grid, block, 0, stream, p, wg);
     } else {
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false>), grid, block, 0, stream, p, wg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false, CHB>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false, CHB>), grid, block, 0, stream, p, wg);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T, int NS, int CPL, bool VEC>
+static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+    if (CPL == 1 && wave_bwd_share(p.f.shape, wg) > 1) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? kWaveShare : 1>(p, wg, stream);
+    return launch_wave_bwd_c<T, NS, CPL, VEC, 1>(p, wg, stream);
 }
 
 template <typename T>

@@ -187,3 +187,42 @@ def test_wavefront_two_columns_per_lane_unaligned_and_flipped(gpu_device, dtype,
         r = {k: t[k].to(dtype).float().cpu().numpy() for k in ("u", "delta", "B", "C")}
         refo = OC.fwd(r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"], True, None, real="f64")
         assert relerr(res[("pitch", capi.SCHED_WAVEFRONT)][0].cpu().numpy(), refo) <= 1e-4
+
+
+SHARED = [
+    # Bt, Dm, H, W, N, K, dtype, kw: one segment per plane and at least 2048 planes - the backward's blocks hold four channels
+    (8, 264, 20, 24, 1, 4, torch.float32, {}),                 # 66 channels per group: the last block of a group repeats two
+    (16, 128, 16, 64, 1, 2, torch.bfloat16, {}),               # whole bands, whole segment
+    (8, 256, 12, 40, 2, 4, torch.float32, {}),
+    (8, 264, 8, 64, 2, 4, torch.bfloat16, {}),
+    (4, 516, 10, 33, 3, 4, torch.float32, {}),                 # four-state kernel with three states, 129 channels per group
+    (4, 512, 9, 20, 4, 4, torch.float16, {}),
+    (8, 264, 21, 30, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
+    (8, 256, 16, 64, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
+]
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,dtype,kw", SHARED)
+def test_wavefront_shared_atomics(gpu_device, Bt, Dm, H, W, N, K, dtype, kw):
+    """Backward blocks of four channels whose dB / dC contributions meet in LDS: against the tile kernels, and
+    against the oracle where it takes the options."""
+    print("wavefront shared atomics", Bt, Dm, H, W, N, K, dtype, kw, flush=True)
+    d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, None, dtype, capi.SCHED_WAVEFRONT, **kw)
+    _, _, f2, b2 = run(gpu_device, Bt, Dm, H, W, N, K, None, dtype, capi.SCHED_PLANE, **kw)
+    half = dtype != torch.float32
+    assert relerr(f.out.cpu().numpy(), f2.out.cpu().numpy()) <= 1e-5
+    for nm, a, w_ in zip(NAMES, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias, b.ddec], [b2.du, b2.ddelta, b2.dA, b2.dB, b2.dC, b2.dD, b2.dbias, b2.ddec]):
+        assert (a is None) == (w_ is None), nm
+        if a is None:
+            continue
+        tol = 1e-2 if (half and nm in ("du", "ddelta")) else (5e-4 if nm == "dA_decay" else 1e-4)
+        e = relerr(a.float().cpu().numpy(), w_.float().cpu().numpy())
+        assert e <= tol, (nm, e)
+    if not kw:
+        r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+        o = (r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"])
+        gref = OC.bwd(*o, d["dout"], True, None, real="f64")
+        for nm, a, w_ in zip(NAMES, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias], gref):
+            tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
+            e = relerr(a.float().cpu().numpy(), w_)
+            assert e <= tol, (nm, e)
