@@ -35,8 +35,7 @@
 
 namespace snd {
 
-constexpr int kWaveShare = 4;                        // channels of a block that share their dB / dC atomics
-constexpr int kWaveShareWaves = 4;                   // waves of such a block (one segment per channel)
+constexpr int kWaveShareWaves = 4;                   // waves of a block whose channels share their dB / dC atomics
 
 __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -487,7 +486,8 @@ static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::
 // kWaveShareWaves of them; with fewer planes than the GPU holds waves, one channel per block spreads them further.
 static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
     const int64_t waves = (int64_t)sh.batch * sh.dim * wg.nseg;
-    return wg.cpl == 1 && wg.nseg * kWaveShare <= kWaveShareWaves && waves >= 2048 ? kWaveShare : 1;
+    if (wg.cpl != 1 || waves < 2048) return 1;
+    return wg.nseg == 1 ? 4 : wg.nseg * 2 <= kWaveShareWaves ? 2 : 1;
 }
 
 template <typename T, int NS, int CPL, bool VEC, int CHB>
@@ -512,7 +512,9 @@ static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStre
 
 template <typename T, int NS, int CPL, bool VEC>
 static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
-    if (CPL == 1 && wave_bwd_share(p.f.shape, wg) > 1) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? kWaveShare : 1>(p, wg, stream);
+    const int share = CPL == 1 ? wave_bwd_share(p.f.shape, wg) : 1;
+    if (share == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1>(p, wg, stream);
+    if (share == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 2 : 1>(p, wg, stream);
     return launch_wave_bwd_c<T, NS, CPL, VEC, 1>(p, wg, stream);
 }
 

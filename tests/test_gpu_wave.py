@@ -199,12 +199,17 @@ SHARED = [
     (4, 512, 9, 20, 4, 4, torch.float16, {}),
     (8, 264, 21, 30, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
     (8, 256, 16, 64, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
+    # two segments per plane: blocks of two channels
+    (4, 264, 12, 100, 1, 4, torch.float32, {}),
+    (4, 256, 16, 128, 2, 4, torch.bfloat16, {}),
+    (2, 516, 9, 70, 3, 4, torch.float32, {}),
+    (4, 264, 13, 90, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
 ]
 
 
 @pytest.mark.parametrize("Bt,Dm,H,W,N,K,dtype,kw", SHARED)
 def test_wavefront_shared_atomics(gpu_device, Bt, Dm, H, W, N, K, dtype, kw):
-    """Backward blocks of four channels whose dB / dC contributions meet in LDS: against the tile kernels, and
+    """Backward blocks of four or two channels whose dB / dC contributions meet in LDS: against the tile kernels, and
     against the oracle where it takes the options."""
     print("wavefront shared atomics", Bt, Dm, H, W, N, K, dtype, kw, flush=True)
     d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, None, dtype, capi.SCHED_WAVEFRONT, **kw)
