@@ -125,7 +125,7 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 //   * row-segment wavefront: a plane is a block of nseg waves, 2048 waves fit the chip at once, a wave takes a
 //     row of its segment in about 1.0 us (one state), 1.6 (two), 2.9 (three or four), whatever the row's width:
 //     a 14-column row leaves 50 of its 64 lanes idle.  Where four channels share their dB / dC atomics (one
-//     segment per plane, a full load of waves) a row takes 0.85, 1.35, 2.55 us.
+//     segment per plane, 512 planes or more) a row takes 0.85, 1.35, 2.55 us.
 //   * tile kernels with four lanes per channel: a block is one wave of 16 channels, 1024 fit at once, and a block
 //     takes one 8x8 (7x7) tile in about 18.5 us - or, with few blocks and many strips, the strip pipeline takes
 //     (column tiles + strips - 1) steps of about 25 us per round of its jobs.
@@ -137,7 +137,7 @@ bool wave_family_pays(const snd_shape &s) {
     const snd::Geo g = snd::make_geo(s.nrows, s.ncols);
     const snd::WaveGeo wg = snd::make_wave_geo(s.nrows, s.ncols, s.dstate);
     const int64_t waves = (int64_t)s.batch * s.dim * wg.nseg;
-    const bool shared = wg.nseg == 1 && waves >= 2048;       // (wave_bwd_share() of the backward's launcher)
+    const bool shared = wg.nseg == 1 && waves >= 512;        // (wave_bwd_share() of the backward's launcher)
     const double t_row = shared ? (s.dstate <= 1 ? 0.85 : s.dstate == 2 ? 1.35 : 2.55) : (s.dstate <= 1 ? 1.0 : s.dstate == 2 ? 1.6 : 2.9);
     const double t_wave = (double)((waves + 2047) / 2048) * (wg.Hp + (wg.nseg - 1) * wg.R) * t_row;
     const int64_t blocks = plane_chunks(s);

@@ -483,11 +483,13 @@ static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::
 }
 
 // Channels per block.  Sharing the atomics needs the channels' waves in one block, and a block may hold
-// kWaveShareWaves of them; with fewer planes than the GPU holds waves, one channel per block spreads them further.
+// kWaveShareWaves of them; small launches spread further with one channel per block (measured at 56x56 and 112x112
+// planes: four one-wave channels pay from 512 planes on, two two-wave channels only once the waves fill the GPU).
 static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
     const int64_t waves = (int64_t)sh.batch * sh.dim * wg.nseg;
-    if (wg.cpl != 1 || waves < 2048) return 1;
-    return wg.nseg == 1 ? 4 : wg.nseg * 2 <= kWaveShareWaves ? 2 : 1;
+    if (wg.cpl != 1) return 1;
+    if (wg.nseg == 1) return waves >= 512 ? 4 : 1;
+    return wg.nseg * 2 <= kWaveShareWaves && waves >= 2048 ? 2 : 1;
 }
 
 template <typename T, int NS, int CPL, bool VEC, int CHB>

@@ -190,7 +190,7 @@ def test_wavefront_two_columns_per_lane_unaligned_and_flipped(gpu_device, dtype,
 
 
 SHARED = [
-    # Bt, Dm, H, W, N, K, dtype, kw: one segment per plane and at least 2048 planes - the backward's blocks hold four channels
+    # Bt, Dm, H, W, N, K, dtype, kw: one segment per plane and 512 planes or more - the backward's blocks hold four channels
     (8, 264, 20, 24, 1, 4, torch.float32, {}),                 # 66 channels per group: the last block of a group repeats two
     (16, 128, 16, 64, 1, 2, torch.bfloat16, {}),               # whole bands, whole segment
     (8, 256, 12, 40, 2, 4, torch.float32, {}),
@@ -199,7 +199,7 @@ SHARED = [
     (4, 512, 9, 20, 4, 4, torch.float16, {}),
     (8, 264, 21, 30, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
     (8, 256, 16, 64, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
-    # two segments per plane: blocks of two channels
+    # two segments per plane and a full load of waves (2048): blocks of two channels
     (4, 264, 12, 100, 1, 4, torch.float32, {}),
     (4, 256, 16, 128, 2, 4, torch.bfloat16, {}),
     (2, 516, 9, 70, 3, 4, torch.float32, {}),
