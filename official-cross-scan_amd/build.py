@@ -19,7 +19,7 @@ INC = os.path.join(ROOT, "include")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libsnd_scan.so")
 
-HIP_SOURCES = ["snd_bwd_f32.hip", "snd_bwd_bf16.hip", "snd_bwd_f16.hip", "snd_wave_bwd.hip", "snd_wave_fwd.hip", "snd_fwd_f32.hip", "snd_fwd_bf16.hip",
+HIP_SOURCES = ["snd_bwd_f32.hip", "snd_bwd_bf16.hip", "snd_bwd_f16.hip", "snd_wave_bwd_f32.hip", "snd_wave_bwd_bf16.hip", "snd_wave_bwd_f16.hip", "snd_wave_fwd_f32.hip", "snd_wave_fwd_bf16.hip", "snd_wave_fwd_f16.hip", "snd_fwd_f32.hip", "snd_fwd_bf16.hip",
                "snd_fwd_f16.hip", "snd_capi.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",

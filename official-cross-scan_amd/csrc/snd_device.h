@@ -474,6 +474,9 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][2][Wp]        h, then a, on the last row of every band
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
+// Planes per wave: narrow planes (one segment, at most 32 / 16 columns) are packed two / four to a wave, plane q of a
+// wave in lanes q*32.. / q*16.. (the saved state keeps its layout: either kernel of a pair may pack or not).
+__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all
@@ -572,13 +575,45 @@ __device__ __forceinline__ void wave_scan3(float &y, float &s, float &a) {
             SND_SCAN3_LVL("row_shr:8", "0xf") SND_SCAN3_LVL("row_bcast:15", "0xa") SND_SCAN3_LVL("row_bcast:31", "0xc")
         : "+v"(y), "+v"(s), "+v"(a));
 }
+// Packed planes: a wave holds PK = 2 or 4 planes of at most 32 or 16 columns, plane q in lanes q*64/PK ..; every
+// plane is scanned on its own.  The levels that would cross into the next plane are left out: row_shr never leaves a
+// 16-lane row, row_bcast:15 joins the two rows of a 32-lane plane.
+template <int PK> __device__ __forceinline__ void wave_scan3_pk(float &y, float &s, float &a) {
+    if (PK == 1) {
+        wave_scan3(y, s, a);
+    } else if (PK == 2) {
+        asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
+                SND_SCAN3_LVL("row_shr:8", "0xf") SND_SCAN3_LVL("row_bcast:15", "0xa")
+            : "+v"(y), "+v"(s), "+v"(a));
+    } else {
+        asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
+                SND_SCAN3_LVL("row_shr:8", "0xf")
+            : "+v"(y), "+v"(s), "+v"(a));
+    }
+}
+// v of the lane below inside the lane's plane; the plane's first lane (`first`) keeps `edge`.
+template <int PK> __device__ __forceinline__ float from_prev_lane_pk(float v, float edge, bool first) {
+    if (PK == 1) return from_prev_lane(v, edge);
+    if (PK == 4) return dpp_old<0x111, 0xF>(edge, v);                  // row_shr:1
+    const float t = from_prev_lane(v, edge);
+    return first ? edge : t;
+}
+// v of the lane above inside the lane's plane; the plane's last lane (`last`) keeps `edge`.
+template <int PK> __device__ __forceinline__ float from_next_lane_pk(float v, float edge, bool last) {
+    if (PK == 1) return from_next_lane(v, edge);
+    if (PK == 4) return dpp_old<0x101, 0xF>(edge, v);                  // row_shl:1
+    const float t = from_next_lane(v, edge);
+    return last ? edge : t;
+}
+
 // One row of a segment: t_j = a_j*t_{j-1} + y_j and the same with s_j, over the CPL columns of each of the 64
 // lanes, lanes ascending in the direction of the recurrence, cy / cs entering the first column of lane 0.
 // The CPL maps of a lane are composed first, one scan runs over the lanes, and the lane's columns are filled
 // in from the value entering the lane.  Returns the solutions per column (the lane's last: oy[CPL-1]).
-template <int CPL>
+template <int CPL, int PK = 1>
 __device__ __forceinline__ void wave_row_solve(const float (&a)[CPL], const float (&y)[CPL], const float (&sv)[CPL], float cy,
                                                float cs, float (&oy)[CPL], float (&os)[CPL]) {
+    static_assert(PK == 1 || CPL == 1, "packed planes: one column per lane");
     float Y = y[0], S = sv[0], Ap = a[0];
 #pragma unroll
     for (int k = 1; k < CPL; ++k) {
@@ -586,7 +621,7 @@ __device__ __forceinline__ void wave_row_solve(const float (&a)[CPL], const floa
         S = fmaf(a[k], S, sv[k]);
         Ap *= a[k];
     }
-    wave_scan3(Y, S, Ap);
+    wave_scan3_pk<PK>(Y, S, Ap);
     const float ey = fmaf(Ap, cy, Y), es = fmaf(Ap, cs, S);      // at the lane's last column
     if (CPL > 1) {
         float ty = from_prev_lane(ey, cy), ts = from_prev_lane(es, cs);   // entering the lane
@@ -602,6 +637,16 @@ __device__ __forceinline__ void wave_row_solve(const float (&a)[CPL], const floa
     os[CPL - 1] = es;
 }
 
+// Sum over the 64 / PK lanes of each packed plane; the total ends in the plane's last lane.
+template <int PK> __device__ __forceinline__ float wave_sum_to_plane_last(float v) {
+    v += dpp_old<0x111, 0xF>(0.f, v);
+    v += dpp_old<0x112, 0xF>(0.f, v);
+    v += dpp_old<0x114, 0xF>(0.f, v);
+    v += dpp_old<0x118, 0xF>(0.f, v);
+    if (PK <= 2) v += dpp_old<0x142, 0xA>(0.f, v);
+    if (PK == 1) v += dpp_old<0x143, 0xC>(0.f, v);
+    return v;
+}
 // Sum over the 64 lanes; the total ends in lane 63.
 __device__ __forceinline__ float wave_sum_to_last(float v) {
     v += dpp_old<0x111, 0xF>(0.f, v);

@@ -50,10 +50,15 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 // CHB > 1: the block holds CHB channels of one (batch, group) pair, each with its own waves.  The channels' dB / dC
 // contributions of a band meet in LDS and leave as one atomic per element and block: the atomics are performed at
 // the memory side, line by line, and cost the kernel a third to a half of its time when every channel issues its own.
-template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB>
+//
+// PK > 1 (with CHB > 1): narrow planes packed PK to a wave as in the forward (wave_pack() in snd_device.h); the block
+// then holds CHB * PK channels, and the planes of a wave are added up with the waves of the block.
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
     static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
+    static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
+    constexpr int S = 64 / PK;                       // lanes per plane
     constexpr int kItems = R * NS * 2;               // dB and dC rows of a band
     constexpr int kXBuf = CHB == 1 ? 1 : NS == 4 ? 1 : 2;   // (with two buffers one barrier per band is enough)
     constexpr int kXWaves = CHB == 1 ? 1 : kWaveShareWaves;
@@ -70,14 +75,18 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     const int nseg = wg.nseg;
     const int lane = threadIdx.x & 63, wi = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int kc = CHB > 1 ? wi / nseg : 0, w = wi - kc * nseg;     // channel of the block, segment of the channel
+    const int kc = CHB > 1 ? wi / nseg : 0, w = PK > 1 ? 0 : wi - kc * nseg;     // channel of the block, segment of the channel
+    const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
     int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, (rg + CHB - 1) / CHB, pair, chunk)) return;
-    chunk = chunk * CHB + kc;
-    // A block past the last channel of its group repeats that channel (identical du / ddelta stores) and adds nothing.
+    if (!wave_job(blockIdx.x, sh.batch * G, (rg + CHB * PK - 1) / (CHB * PK), pair, chunk)) return;
+    chunk = (chunk * CHB + kc) * PK + (PK > 1 ? lane / S : 0);       // (packed: a lane's own from here on)
+    // A wave (a plane of a wave) past the last channel of its group repeats that channel (identical du / ddelta
+    // stores) and adds nothing.
     const bool active = CHB == 1 || chunk < rg;
     chunk = min(chunk, rg - 1);
     const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
+    // channel offsets: in the scalar base pointers, or (packed) in the lanes' offsets
+    const int cB = PK > 1 ? 0 : c, chB = PK > 1 ? 0 : chunk, cL = PK > 1 ? c : 0, chL = PK > 1 ? chunk : 0;
     const bool multi = nseg > 1;
     if (threadIdx.x < 2 * R * NS)
 #pragma unroll
@@ -87,12 +96,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
     // Mirrored order: this lane owns scan columns jm0 .. jm0+CPL-1 and walks them downwards (its local index t is
     // scan column jm0 + CPL-1-t); in natural order (row checkpoints, recomputation) lane l owns columns jn0 ...
-    const int jm0 = (w * kSeg + 63 - lane) * CPL;
+    const int jm0 = PK > 1 ? S - 1 - sl : (w * kSeg + 63 - lane) * CPL;
     const bool jin = EVEN || jm0 < W;
     const int jc = jin ? jm0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
-    const int jn0 = (w * kSeg + lane) * CPL;
-    const int rev_addr = (63 - lane) * 4;
+    const int jn0 = (w * kSeg + sl) * CPL;
+    const int rev_addr = PK > 1 ? ((lane - sl) + S - 1 - sl) * 4 : (63 - lane) * 4;   // the mirror lane inside the plane
     auto mirror = [&](float v) {
         return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(rev_addr, __builtin_bit_cast(int, v)));
     };
@@ -117,21 +126,25 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     constexpr int DSZ = (int)sizeof(DoT);
     const T *Bb = (const T *)f.B + (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
     const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
-    const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chunk : c) * f.u_d_stride;
-    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(c / rd) * f.delta_d_stride;
+    const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chB : cB) * f.u_d_stride;
+    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(cB / rd) * f.delta_d_stride;
     // fused CrossMerge: dout is the gradient of the merged output, shared by the groups and scaled by the channel's weight
     const bool merge = f.merge != 0;
     const float wm = merge && f.merge_weights ? f.merge_weights[c] : 1.f;
-    const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)(merge ? chunk : c) * p.dout_d_stride;
-    T *dub = (T *)p.du + ((int64_t)b * Dm + c) * H * W;                 // du, ddelta: dense [b, c, H, W]
-    T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + c) * H * W;
+    const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)(merge ? chB : cB) * p.dout_d_stride;
+    T *dub = (T *)p.du + ((int64_t)b * Dm + cB) * H * W;                // du, ddelta: dense [b, c, H, W]
+    T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + cB) * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;               // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
     // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
     const int UhB = (int)f.u_h_stride * ESZ * rs, DhB = (int)f.delta_h_stride * ESZ * rs, BhB = (int)f.B_h_stride * ESZ * rs,
               ChB = (int)f.C_h_stride * ESZ * rs, DohB = (int)p.dout_h_stride * DSZ * rs, WB = W * ESZ * rs, W4 = W * 4 * rs;
     const int64_t BsB = f.B_dstate_stride * ESZ, CsB = f.C_dstate_stride * ESZ, HW4 = (int64_t)H * W * 4;
-    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc * DSZ, col4 = (uint32_t)mc * 4;
+    const uint32_t colB = (uint32_t)mc * ESZ, col4 = (uint32_t)mc * 4;
+    const uint32_t colU = colB + (uint32_t)(f.u_shared ? chL : cL) * (uint32_t)f.u_d_stride * ESZ,
+                   colD = colB + (uint32_t)(cL / rd) * (uint32_t)f.delta_d_stride * ESZ,
+                   colO = (uint32_t)mc * DSZ + (uint32_t)(merge ? chL : cL) * (uint32_t)p.dout_d_stride * DSZ,
+                   colG = colB + (uint32_t)cL * (uint32_t)(H * W) * ESZ;                  // du, ddelta
 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
@@ -151,7 +164,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     auto load_band = [&](In &q, int band) {
         const int i0 = band * R;
         const int m0 = mad24(i0, rs, r0m);           // memory row of the band's first scan row
-        uint32_t ou = mad24(m0, UhB * rs, colB), od = mad24(m0, DhB * rs, colB), oo = mad24(m0, DohB * rs, colO),
+        uint32_t ou = mad24(m0, UhB * rs, colU), od = mad24(m0, DhB * rs, colD), oo = mad24(m0, DohB * rs, colO),
                  ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -274,15 +287,15 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                             a[k] = fast_exp2(fmaf(dln[k], A2[n], ld));
                             bu[k] = bn_[r][n][k] * dlun[k];
                         }
-                        const float a_l = from_prev_lane(a[CPL - 1], ain);                 // a[i, j-1] of the lane's first column
-                        const float h_d = from_prev_lane(hp[n][CPL - 1], hdiag[n]);        // h[i-1, j-1]
+                        const float a_l = from_prev_lane_pk<PK>(a[CPL - 1], ain, sl == 0);                 // a[i, j-1] of the lane's first column
+                        const float h_d = from_prev_lane_pk<PK>(hp[n][CPL - 1], hdiag[n], sl == 0);        // h[i-1, j-1]
 #pragma unroll
                         for (int k = 0; k < CPL; ++k) {
                             const float al = k == 0 ? a_l : a[k > 0 ? k - 1 : 0], hd = k == 0 ? h_d : hp[n][k > 0 ? k - 1 : 0];
                             const float X = fmaf(-0.5f * (ap[n][k] + al), hd, hp[n][k]);
                             y[k] = fmaf(a[k], X, bu[k]);
                         }
-                        wave_row_solve<CPL>(a, y, bu, hin, sin_, h, s);
+                        wave_row_solve<CPL, PK>(a, y, bu, hin, sin_, h, s);
 #pragma unroll
                         for (int k = 0; k < CPL; ++k) {
                             hT[r][n][CPL - 1 - k] = mirror(h[k]);
@@ -312,7 +325,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
         const int rows = EVEN ? R : min(R, H - i0);  // rows of this band inside the plane
         const int mlast = mad24(i0 + rows - 1, rs, r0m);
-        uint32_t og = mad24(mlast, WB * rs, colB), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
+        uint32_t og = mad24(mlast, WB * rs, colG), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
 #pragma unroll
         for (int r = R - 1; r >= 0; --r) {
             if (EVEN || i0 + r < H) {
@@ -342,8 +355,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         bu[t] = Bv[t] * dlu[t];
                         dyC[t] = dov[t] * Cv[t];
                     }
-                    const float a_r0 = from_prev_lane(a[CPL - 1], in.z);               // a[i, j+1] of the lane's first column
-                    const float Gdg0 = from_prev_lane(Gd[n][CPL - 1], GdEdge[n]);      // G[i+1, j+1]
+                    const float a_r0 = from_prev_lane_pk<PK>(a[CPL - 1], in.z, sl == 0);               // a[i, j+1] of the lane's first column
+                    const float Gdg0 = from_prev_lane_pk<PK>(Gd[n][CPL - 1], GdEdge[n], sl == 0);      // G[i+1, j+1]
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
                         const float ar = t == 0 ? a_r0 : a[t > 0 ? t - 1 : 0], gdg = t == 0 ? Gdg0 : Gd[n][t > 0 ? t - 1 : 0];
@@ -351,9 +364,9 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         ya[t] = a[t] * z[t];
                         ys[t] = -a[t] * dyC[t];
                     }
-                    wave_row_solve<CPL>(a, ya, ys, in.x, in.y, Gt, Gst);               // G[i,j], Gs[i,j]
-                    const float Gr0 = from_prev_lane(Gt[CPL - 1], in.x), Gsr0 = from_prev_lane(Gst[CPL - 1], in.y);
-                    const float hl_last = from_next_lane(hT[r][n][0], hin);            // h[i, j-1] of the lane's last column
+                    wave_row_solve<CPL, PK>(a, ya, ys, in.x, in.y, Gt, Gst);           // G[i,j], Gs[i,j]
+                    const float Gr0 = from_prev_lane_pk<PK>(Gt[CPL - 1], in.x, sl == 0), Gsr0 = from_prev_lane_pk<PK>(Gst[CPL - 1], in.y, sl == 0);
+                    const float hl_last = from_next_lane_pk<PK>(hT[r][n][0], hin, sl == S - 1);   // h[i, j-1] of the lane's last column
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
                         const float Gr = t == 0 ? Gr0 : Gt[t > 0 ? t - 1 : 0], Gsr = t == 0 ? Gsr0 : Gst[t > 0 ? t - 1 : 0];
@@ -422,9 +435,11 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                 const int it = m * CHB + kc, r = it / (2 * NS), n = (it >> 1) % NS;
                 float v = 0.f;
 #pragma unroll
-                for (int q = 0; q < CHB; ++q) v += sX[kXBuf == 2 ? step & 1 : 0][w + q * nseg][it][lane];
+                for (int q = 0; q < CHB; ++q)
+#pragma unroll
+                    for (int k = 0; k < PK; ++k) v += sX[kXBuf == 2 ? step & 1 : 0][w + q * nseg][it][PK > 1 ? sl + k * S : lane];
                 float *dst = (float *)((char *)((it & 1) ? dCg : dBg) + n * HW4 + (int64_t)mad24(mad24(i0 + r, rs, r0m), W * 4, (int)col4));
-                if (jin && (EVEN || i0 + r < H) && (NS != 4 || n < N)) wave_glb_add(dst, v);
+                if (jin && (PK == 1 || lane < S) && (EVEN || i0 + r < H) && (NS != 4 || n < N)) wave_glb_add(dst, v);
             }
             if (kXBuf == 1) lds_barrier();
             ++step;
@@ -453,25 +468,25 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     // ---- per-channel sums leave the kernel: one atomic per wave and value
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
-        const float t = wave_sum_to_last(dA_acc[n]);
-        if (lane == 63 && n < N && active) wave_glb_add(p.dA + (int64_t)c * N + n, t);
+        const float t = wave_sum_to_plane_last<PK>(dA_acc[n]);
+        if (sl == S - 1 && n < N && active) wave_glb_add(p.dA + (int64_t)c * N + n, t);
     }
     {
-        const float td = wave_sum_to_last(dD_acc), tb = wave_sum_to_last(dbias_acc);
-        if (lane == 63 && active) {
+        const float td = wave_sum_to_plane_last<PK>(dD_acc), tb = wave_sum_to_plane_last<PK>(dbias_acc);
+        if (sl == S - 1 && active) {
             if (p.dD) wave_glb_add(p.dD + c, td);
             if (p.ddelta_bias) wave_glb_add(p.ddelta_bias + c, tb);
         }
         // Fused CrossMerge: weight * d(weight) = <weighted dout, result of the channel>, and since the result is
         // linear in u (D*u plus a recurrence linear in B*delta'*u) that inner product equals <du, u>.
         if (merge && p.dmerge) {
-            const float tw = wave_sum_to_last(dw_acc);
-            if (lane == 63 && active) wave_glb_add(p.dmerge + c, tw);
+            const float tw = wave_sum_to_plane_last<PK>(dw_acc);
+            if (sl == S - 1 && active) wave_glb_add(p.dmerge + c, tw);
         }
     }
     if (want_decay) {
-        const float t = wave_sum_to_last(dec_acc);
-        if (lane == 63 && active) wave_glb_add(p.dA_decay, t / f.A_decay[0]);
+        const float t = wave_sum_to_plane_last<PK>(dec_acc);
+        if (sl == S - 1 && active) wave_glb_add(p.dA_decay, t / f.A_decay[0]);
     }
 }
 
@@ -492,22 +507,22 @@ static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
     return wg.nseg * 2 <= kWaveShareWaves && waves >= 2048 ? 2 : 1;
 }
 
-template <typename T, int NS, int CPL, bool VEC, int CHB>
+template <typename T, int NS, int CPL, bool VEC, int CHB, int PK>
 static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const int rg = sh.dim / sh.n_groups;
-    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + CHB - 1) / CHB)), block(64 * wg.nseg * CHB);
+    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + CHB * PK - 1) / (CHB * PK))), block(64 * wg.nseg * CHB);
     constexpr bool F32 = std::is_same<T, float>::value;
     constexpr int R = NS <= 1 ? 8 : 4;
     // (the even-plane variant only where the loads are prefetched: it is their waits that it makes exact)
-    const bool even = NS <= 2 && CPL == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
+    const bool even = NS <= 2 && CPL == 1 && PK == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
     if (even) {
-        constexpr bool E = NS <= 2 && CPL == 1;
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E, CHB>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E, CHB>), grid, block, 0, stream, p, wg);
+        constexpr bool E = NS <= 2 && CPL == 1 && PK == 1;
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E, CHB, PK>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E, CHB, PK>), grid, block, 0, stream, p, wg);
     } else {
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false, CHB>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false, CHB>), grid, block, 0, stream, p, wg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false, CHB, PK>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false, CHB, PK>), grid, block, 0, stream, p, wg);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
@@ -515,9 +530,13 @@ static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStre
 template <typename T, int NS, int CPL, bool VEC>
 static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const int share = CPL == 1 ? wave_bwd_share(p.f.shape, wg) : 1;
-    if (share == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1>(p, wg, stream);
-    if (share == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 2 : 1>(p, wg, stream);
-    return launch_wave_bwd_c<T, NS, CPL, VEC, 1>(p, wg, stream);
+    const int pk = CPL == 1 ? wave_pack(wg, p.f.shape.ncols) : 1;
+    // (packed planes always in blocks of four waves: the planes of a wave are added up where the waves of a block are)
+    if (pk == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 4 : 1>(p, wg, stream);
+    if (pk == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 2 : 1>(p, wg, stream);
+    if (share == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, 1>(p, wg, stream);
+    if (share == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 2 : 1, 1>(p, wg, stream);
+    return launch_wave_bwd_c<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
 }
 
 template <typename T>

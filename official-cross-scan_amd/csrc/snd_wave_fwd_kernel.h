@@ -34,9 +34,14 @@
 
 namespace snd {
 
-template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32>
+// PK > 1: narrow planes packed PK to a wave (wave_pack() in snd_device.h): lane l works on column l % (64 / PK) of
+// channel PK * chunk + l / (64 / PK) of the group, every per-channel quantity is a lane's own, and the scan stays
+// inside the plane's lanes.  One segment per plane, so nothing is handed over between waves.
+template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK>
 __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band = rows per load group
+    static_assert(PK == 1 || CPL == 1, "packed planes: one column per lane");
+    constexpr int S = 64 / PK;                       // lanes per plane
 #ifndef SND_WAVE_RD
 #define SND_WAVE_RD 4
 #endif
@@ -54,9 +59,15 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
     const int rg = Dm / G, rd = Dm / sh.delta_dim;
     int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, rg, pair, chunk)) return;
+    if (!wave_job(blockIdx.x, sh.batch * G, (rg + PK - 1) / PK, pair, chunk)) return;
+    const int lane = threadIdx.x & 63, w = PK > 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
+    if (PK > 1) chunk = chunk * PK + lane / S;       // (a lane's own from here on)
+    const bool act = PK == 1 || chunk < rg;          // a wave past the last channel of its group repeats it and stores nothing
+    if (PK > 1) chunk = min(chunk, rg - 1);
     const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
-    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    // channel offsets: in the scalar base pointers, or (packed) in the lanes' offsets
+    const int cB = PK > 1 ? 0 : c, chB = PK > 1 ? 0 : chunk, cL = PK > 1 ? c : 0, chL = PK > 1 ? chunk : 0;
     const int nseg = wg.nseg;
     const bool multi = nseg > 1;
     if (threadIdx.x < 2 * RD * NS) (&sHO[0][0][0][0])[(threadIdx.x / (RD * NS)) * (kMaxSeg + 1) * RD * NS + threadIdx.x % (RD * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -64,7 +75,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     // scan origin of this group: memory row = r0m + rs*i; with fh the columns run against the memory order
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
-    const int j0 = (w * kSeg + lane) * CPL;          // this lane's first scan column
+    const int j0 = (w * kSeg + sl) * CPL;            // this lane's first scan column
     const bool jin = j0 < W;                         // (W is a multiple of CPL: a lane is inside or outside as a whole)
     const int jc = jin ? j0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
@@ -82,17 +93,20 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     constexpr int OSZ = (int)sizeof(OutT);
     const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
-    const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chunk : c) * p.u_d_stride;
-    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(c / rd) * p.delta_d_stride;
+    const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chB : cB) * p.u_d_stride;
+    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(cB / rd) * p.delta_d_stride;
     // fused CrossMerge (fp32 out only): the channel adds weight * result to the feature channel it belongs to
     const bool merge = p.merge != 0;
     const float wm = merge && p.merge_weights ? p.merge_weights[c] : 1.f;
-    OutT *outb = (OutT *)p.out + (int64_t)b * p.out_batch_stride + (int64_t)(merge ? chunk : c) * p.out_d_stride;
+    OutT *outb = (OutT *)p.out + (int64_t)b * p.out_batch_stride + (int64_t)(merge ? chB : cB) * p.out_d_stride;
     // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
     const int UhB = (int)p.u_h_stride * ESZ * rs, DhB = (int)p.delta_h_stride * ESZ * rs, BhB = (int)p.B_h_stride * ESZ * rs,
               ChB = (int)p.C_h_stride * ESZ * rs, OhB = (int)p.out_h_stride * OSZ * rs;
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
-    const uint32_t colB = (uint32_t)mc * ESZ, colO = (uint32_t)mc * OSZ;
+    const uint32_t colB = (uint32_t)mc * ESZ;
+    const uint32_t colU = colB + (uint32_t)(p.u_shared ? chL : cL) * (uint32_t)p.u_d_stride * ESZ,
+                   colD = colB + (uint32_t)(cL / rd) * (uint32_t)p.delta_d_stride * ESZ,
+                   colO = (uint32_t)mc * OSZ + (uint32_t)(merge ? chL : cL) * (uint32_t)p.out_d_stride * OSZ;
 
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
@@ -110,7 +124,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     auto load_band = [&](Stage &q, int band) {
         const int i0 = band * R;
         const int m0 = mad24(i0, rs, r0m);           // memory row of the band's first scan row
-        uint32_t ou = mad24(m0, UhB * rs, colB), od = mad24(m0, DhB * rs, colB), ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
+        uint32_t ou = mad24(m0, UhB * rs, colU), od = mad24(m0, DhB * rs, colD), ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             wave_ld(q.u[r], ub, ou);
@@ -210,8 +224,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                         a[k] = fast_exp2(fmaf(dl[k], A2[n], ld));
                         bu[k] = ((NS == 4 && n >= N) ? 0.f : bu[k]) * du[k];
                     }
-                    const float a_l = from_prev_lane(a[CPL - 1], in.z);                // a[i, j-1] of the lane's first column
-                    const float h_d = from_prev_lane(hprev[n][CPL - 1], hdiag[n]);     // h[i-1, j-1]
+                    const float a_l = from_prev_lane_pk<PK>(a[CPL - 1], in.z, sl == 0);                // a[i, j-1] of the lane's first column
+                    const float h_d = from_prev_lane_pk<PK>(hprev[n][CPL - 1], hdiag[n], sl == 0);     // h[i-1, j-1]
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) {
                         const float al = k == 0 ? a_l : a[k > 0 ? k - 1 : 0], hd = k == 0 ? h_d : hprev[n][k > 0 ? k - 1 : 0];
@@ -222,7 +236,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
 #pragma unroll
                         for (int k = 0; k < CPL; ++k) { h[k] = y[k]; s[k] = bu[k]; }
                     } else {
-                        wave_row_solve<CPL>(a, y, bu, in.x, in.y, h, s);
+                        wave_row_solve<CPL, PK>(a, y, bu, in.x, in.y, h, s);
                     }
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) {
@@ -241,7 +255,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                         ca[n] = mine ? in.z : ca[n];
                     }
                 }
-                if (jin && (!(SND_WAVE_ABLATE & 1) || acc[0] == 1234.5f)) {
+                if (jin && act && (!(SND_WAVE_ABLATE & 1) || acc[0] == 1234.5f)) {
                     float o[CPL];
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) o[k] = fmaf(Dv, u[k], acc[k]);
@@ -260,7 +274,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
-            if ((NS != 4 || n < N) && !(SND_WAVE_ABLATE & 16)) {
+            if ((NS != 4 || n < N) && act && !(SND_WAVE_ABLATE & 16)) {
                 float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
 #pragma unroll
                 for (int k = 0; k < CPL; ++k) {
@@ -311,17 +325,26 @@ static inline bool wave_aligned(const void *ptr, int64_t esz, int bytes, std::in
     return true;
 }
 
-template <typename T, int NS, int CPL, bool VEC>
-static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+template <typename T, int NS, int CPL, bool VEC, int PK>
+static int launch_wave_fwd_p(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.shape;
-    const dim3 grid(wave_grid(sh.batch * sh.n_groups, sh.dim / sh.n_groups)), block(64 * wg.nseg);
+    const int rg = sh.dim / sh.n_groups;
+    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + PK - 1) / PK)), block(64 * wg.nseg);
     const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
     constexpr bool F = std::is_same<T, float>::value;
-    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true>), grid, block, 0, stream, p, wg);
-    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F>), grid, block, 0, stream, p, wg);
-    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F>), grid, block, 0, stream, p, wg);
+    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK>), grid, block, 0, stream, p, wg);
+    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F, PK>), grid, block, 0, stream, p, wg);
+    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true, PK>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F, PK>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T, int NS, int CPL, bool VEC>
+static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+    const int pk = CPL == 1 ? wave_pack(wg, p.shape.ncols) : 1;
+    if (pk == 4) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 4 : 1>(p, wg, stream);
+    if (pk == 2) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 2 : 1>(p, wg, stream);
+    return launch_wave_fwd_p<T, NS, CPL, VEC, 1>(p, wg, stream);
 }
 
 template <typename T>

@@ -231,3 +231,50 @@ def test_wavefront_shared_atomics(gpu_device, Bt, Dm, H, W, N, K, dtype, kw):
             tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
             e = relerr(a.float().cpu().numpy(), w_)
             assert e <= tol, (nm, e)
+
+
+PACKED = [
+    # Bt, Dm, H, W, N, K, Dd, dtype, kw: planes of at most 32 / 16 columns, two / four to a wave
+    (2, 24, 14, 14, 1, 4, None, torch.float32, {}),            # 6 channels per group: the second wave of a group holds two
+    (2, 40, 7, 7, 2, 4, None, torch.bfloat16, {}),
+    (3, 36, 9, 16, 4, 2, 18, torch.float32, {}),               # 16 columns exactly; delta shared by pairs of channels
+    (2, 28, 20, 17, 1, 4, None, torch.float16, {}),            # two planes per wave, 7 channels per group
+    (1, 64, 33, 32, 3, 4, 16, torch.float32, {}),              # 32 columns exactly, three states, delta shared by four channels
+    (64, 96, 14, 14, 1, 4, None, torch.float32, {}),           # 6144 planes
+    (2, 24, 15, 13, 1, 4, None, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
+    (2, 20, 10, 29, 2, 4, None, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
+    (2, 24, 14, 14, 2, 4, None, torch.bfloat16, dict(out_float=False, use_D=False, use_bias=False)),
+    (1, 4, 5, 1, 1, 1, None, torch.float32, {}),               # one column, one group
+]
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,Dd,dtype,kw", PACKED)
+def test_wavefront_packed_planes(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, kw):
+    """Several narrow planes per wave, forward and backward: against the tile kernels, and against the oracle where
+    it takes the options."""
+    print("wavefront packed planes", Bt, Dm, H, W, N, K, Dd, dtype, kw, flush=True)
+    d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_WAVEFRONT, **kw)
+    _, _, f2, b2 = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_PLANE, **kw)
+    half = dtype != torch.float32
+    assert relerr(f.out.float().cpu().numpy(), f2.out.float().cpu().numpy()) <= (1e-2 if kw.get("out_float") is False else 1e-5)
+    for nm, a, w_ in zip(NAMES, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias, b.ddec], [b2.du, b2.ddelta, b2.dA, b2.dB, b2.dC, b2.dD, b2.dbias, b2.ddec]):
+        assert (a is None) == (w_ is None), nm
+        if a is None:
+            continue
+        tol = 1e-2 if (half and nm in ("du", "ddelta")) else (5e-4 if nm == "dA_decay" else 1e-4)
+        e = relerr(a.float().cpu().numpy(), w_.float().cpu().numpy())
+        assert e <= tol, (nm, e)
+    if not kw:
+        r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+        o = (r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"])
+        ref = OC.fwd(*o, True, None, real="f64")
+        gref = OC.bwd(*o, d["dout"], True, None, real="f64")
+        assert relerr(f.out.cpu().numpy(), ref) <= 1e-4
+        got = [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias]
+        if Dd is not None:                            # the C ABI returns ddelta / ddelta_bias per channel
+            got[1] = got[1].float().view(Bt, Dd, Dm // Dd, H, W).sum(2)
+            got[6] = got[6].view(Dd, Dm // Dd).sum(1)
+        for nm, a, w_ in zip(NAMES, got, gref):
+            tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
+            e = relerr(a.float().cpu().numpy(), w_)
+            assert e <= tol, (nm, e)

@@ -56,7 +56,7 @@ def test_placement_advice():
     an fp32 row for the row-segment kernels on rows of 2 KiB or more."""
     for shp, want in (((64, 192, 56, 56, 16, 4, 192, capi.SND_F32), 5120), ((1, 256, 512, 512, 1, 4, 256, capi.SND_BF16), 1024),
                       ((1, 64, 1024, 1024, 1, 4, 64, capi.SND_BF16), 2048), ((8, 192, 64, 64, 1, 4, 192, capi.SND_BF16), 16384),
-                      ((64, 768, 14, 14, 1, 4, 768, capi.SND_BF16), 5120)):
+                      ((64, 768, 14, 14, 16, 4, 768, capi.SND_BF16), 5120)):
         st, plan = capi.make_plan(capi.Shape(*shp))
         assert st == 0
         assert plan.dC_skew_bytes == want
@@ -223,8 +223,8 @@ def test_forward_job_split():
 
 
 def test_kernel_family_choice():
-    """1-4 states: large or few planes go to the row-segment wavefront, small planes of many channels to the tile
-    kernels (a 14-column row fills 14 of a wave's 64 lanes); 5-16 states always to the tile kernels."""
+    """1-4 states: the row-segment wavefront (narrow planes packed two or four to a wave), except for a few plane
+    sizes with four states where a wave's lanes stay too empty; 5-16 states always the tile kernels."""
     def family(Bt, Dm, H, W, N, K=4):
         st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, N, K, Dm, capi.SND_BF16))
         assert st == 0
@@ -233,9 +233,11 @@ def test_kernel_family_choice():
     assert family(1, 256, 512, 512, 1) == "wave"          # 256 planes: nothing else fills the chip
     assert family(64, 192, 56, 56, 1) == "wave"
     assert family(64, 384, 28, 28, 1) == "wave"
-    assert family(64, 768, 14, 14, 1) == "tile"
-    assert family(64, 1536, 7, 7, 1) == "tile"
-    assert family(64, 768, 14, 14, 4) == "tile"
+    assert family(64, 768, 14, 14, 1) == "wave"           # four planes per wave
+    assert family(64, 1536, 7, 7, 1) == "wave"
+    assert family(64, 768, 14, 14, 4) == "wave"
+    assert family(32, 12288, 7, 7, 4) == "tile"           # 7 of a packed plane's 16 lanes: 1.14 ms against 0.65
+    assert family(32, 1344, 21, 21, 4) == "tile"          # 21 of 32 lanes: 0.73 against 0.67
     assert family(32, 256, 40, 40, 4) == "tile"
     assert family(64, 192, 56, 56, 4) == "wave"           # (the two families within 2 % of each other)
     assert family(4, 192, 56, 56, 4) == "wave"            # 48 blocks: the strip pipeline's ramp costs more than the rows
