@@ -1,6 +1,6 @@
 """Benchmark of the 2D-CrossScan selective scan (selective_nd_scan fwd + bwd) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c4n1|c1n1] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c4n1|c1n1|c2n1] [--no-cpu]
 
 One step = one forward + one backward of the operator through the PyTorch extension (output,
 saved-state and gradient allocations, zero-fills and dtype casts included, as a caller of the
@@ -42,6 +42,7 @@ WORKLOADS = {                   # name: (B, D, H, W, N, K, input dtype)
     "c4": (1, 256, 512, 512, 16, 4, "bfloat16"),
     "c4n1": (1, 256, 512, 512, 1, 4, "bfloat16"),
     "c1n1": (64, 192, 56, 56, 1, 4, "float32"),     # c1's planes with one state per channel (the d_state = 1 variant)
+    "c2n1": (64, 768, 14, 14, 1, 4, "bfloat16"),    # c2's planes with one state per channel
 }
 
 
