@@ -21,6 +21,9 @@ FULL = [
     ("c3", 2, 192, 200, 336, 16, 4, torch.float32, capi.SCHED_STRIPS, 25),
     ("c4", 1, 256, 512, 512, 16, 4, torch.bfloat16, capi.SCHED_STRIPS, 64),
     ("c4n1", 1, 256, 512, 512, 1, 4, torch.bfloat16, None, None),
+    ("c1n1", 64, 192, 56, 56, 1, 4, torch.float32, None, None),       # four channels per backward block
+    ("c2n1", 64, 768, 14, 14, 1, 4, torch.bfloat16, None, None),      # four planes per wave
+    ("c2n4", 64, 768, 14, 14, 4, 4, torch.bfloat16, None, None),      # the same with four states
 ]
 
 
