@@ -474,9 +474,11 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][2][Wp]        h, then a, on the last row of every band
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
-// Planes per wave: narrow planes (one segment, at most 32 / 16 columns) are packed two / four to a wave, plane q of a
-// wave in lanes q*32.. / q*16.. (the saved state keeps its layout: either kernel of a pair may pack or not).
-__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
+// Planes per wave: narrow planes (one segment, at most 32 / 16 / 7 columns) are packed two / four / eight to a wave,
+// plane q of a wave in lanes q*32.. / q*16.. / q*8.. (the saved state keeps its layout: either kernel of a pair may
+// pack or not).  With eight planes the first lane of a plane is a barrier lane (wave_scan3_pk) and its columns are in
+// lanes 1..7.
+__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 7 ? 8 : W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all
@@ -585,23 +587,32 @@ template <int PK> __device__ __forceinline__ void wave_scan3_pk(float &y, float 
         asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
                 SND_SCAN3_LVL("row_shr:8", "0xf") SND_SCAN3_LVL("row_bcast:15", "0xa")
             : "+v"(y), "+v"(s), "+v"(a));
-    } else {
+    } else if (PK == 4) {
         asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
                 SND_SCAN3_LVL("row_shr:8", "0xf")
+            : "+v"(y), "+v"(s), "+v"(a));
+    } else {
+        // Eight planes of 8 lanes: row_shr carries lane 7 of a 16-lane row into lane 8, the first lane of the next
+        // plane.  That lane is a barrier: it holds the map (a, y, s) = (0, 0, 0), which stays what it is under every
+        // composition, and a lane whose range has reached it holds a = 0 and takes nothing from beyond it.  (Switching
+        // lanes off in EXEC instead does not work: a DPP read of a disabled lane is an invalid source.)
+        asm("s_nop 1\n\t" SND_SCAN3_LVL("row_shr:1", "0xf") SND_SCAN3_LVL("row_shr:2", "0xf") SND_SCAN3_LVL("row_shr:4", "0xf")
             : "+v"(y), "+v"(s), "+v"(a));
     }
 }
 // v of the lane below inside the lane's plane; the plane's first lane (`first`) keeps `edge`.
 template <int PK> __device__ __forceinline__ float from_prev_lane_pk(float v, float edge, bool first) {
     if (PK == 1) return from_prev_lane(v, edge);
-    if (PK == 4) return dpp_old<0x111, 0xF>(edge, v);                  // row_shr:1
+    // (eight planes: a plane's first lane is its barrier lane, whose own results are never used)
+    if (PK == 4 || PK == 8) return dpp_old<0x111, 0xF>(edge, v);       // row_shr:1
     const float t = from_prev_lane(v, edge);
     return first ? edge : t;
 }
 // v of the lane above inside the lane's plane; the plane's last lane (`last`) keeps `edge`.
 template <int PK> __device__ __forceinline__ float from_next_lane_pk(float v, float edge, bool last) {
     if (PK == 1) return from_next_lane(v, edge);
-    if (PK == 4) return dpp_old<0x101, 0xF>(edge, v);                  // row_shl:1
+    // (eight planes: the lane after a plane's last is the next plane's barrier lane, which holds the zero edge)
+    if (PK == 4 || PK == 8) return dpp_old<0x101, 0xF>(edge, v);       // row_shl:1
     const float t = from_next_lane(v, edge);
     return last ? edge : t;
 }
@@ -639,6 +650,12 @@ __device__ __forceinline__ void wave_row_solve(const float (&a)[CPL], const floa
 
 // Sum over the 64 / PK lanes of each packed plane; the total ends in the plane's last lane.
 template <int PK> __device__ __forceinline__ float wave_sum_to_plane_last(float v) {
+    if (PK == 8) {                                   // butterflies inside the 8 lanes: every lane ends with the total
+        v += dpp_old<0xB1, 0xF>(0.f, v);             // quad_perm:[1,0,3,2]
+        v += dpp_old<0x4E, 0xF>(0.f, v);             // quad_perm:[2,3,0,1]
+        v += dpp_old<0x141, 0xF>(0.f, v);            // row_half_mirror
+        return v;
+    }
     v += dpp_old<0x111, 0xF>(0.f, v);
     v += dpp_old<0x112, 0xF>(0.f, v);
     v += dpp_old<0x114, 0xF>(0.f, v);

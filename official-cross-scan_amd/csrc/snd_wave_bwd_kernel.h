@@ -96,12 +96,14 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
     // Mirrored order: this lane owns scan columns jm0 .. jm0+CPL-1 and walks them downwards (its local index t is
     // scan column jm0 + CPL-1-t); in natural order (row checkpoints, recomputation) lane l owns columns jn0 ...
+    const bool bar = PK == 8 && sl == 0;             // (eight planes per wave) the plane's barrier lane: mirrored column 7
     const int jm0 = PK > 1 ? S - 1 - sl : (w * kSeg + 63 - lane) * CPL;
     const bool jin = EVEN || jm0 < W;
     const int jc = jin ? jm0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
-    const int jn0 = (w * kSeg + sl) * CPL;
-    const int rev_addr = PK > 1 ? ((lane - sl) + S - 1 - sl) * 4 : (63 - lane) * 4;   // the mirror lane inside the plane
+    const int jn0 = PK == 8 ? max(sl - 1, 0) : (w * kSeg + sl) * CPL;
+    // the mirror lane inside the plane (eight planes: lanes 1..7 among themselves, the barrier lane stays)
+    const int rev_addr = PK == 8 ? ((lane - sl) + (sl == 0 ? 0 : 8 - sl)) * 4 : PK > 1 ? ((lane - sl) + S - 1 - sl) * 4 : (63 - lane) * 4;
     auto mirror = [&](float v) {
         return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(rev_addr, __builtin_bit_cast(int, v)));
     };
@@ -193,6 +195,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                     for (int k = 0; k < CPL; ++k) {
                         q.h0[n][k] = __builtin_nontemporal_load(src + k);
                         q.a0[n][k] = __builtin_nontemporal_load(src + wg.Wp + k);
+                        if (PK == 8) { q.h0[n][k] = bar ? 0.f : q.h0[n][k]; q.a0[n][k] = bar ? 0.f : q.a0[n][k]; }
                     }
                 }
                 if (w > 0 && lane <= R && row >= 0) {
@@ -286,6 +289,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
                         for (int k = 0; k < CPL; ++k) {
                             a[k] = fast_exp2(fmaf(dln[k], A2[n], ld));
                             bu[k] = bn_[r][n][k] * dlun[k];
+                            if (PK == 8) { a[k] = bar ? 0.f : a[k]; bu[k] = bar ? 0.f : bu[k]; }   // the barrier lane's map is (0, 0)
                         }
                         const float a_l = from_prev_lane_pk<PK>(a[CPL - 1], ain, sl == 0);                 // a[i, j-1] of the lane's first column
                         const float h_d = from_prev_lane_pk<PK>(hp[n][CPL - 1], hdiag[n], sl == 0);        // h[i-1, j-1]
@@ -370,7 +374,8 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_pa
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
                         const float Gr = t == 0 ? Gr0 : Gt[t > 0 ? t - 1 : 0], Gsr = t == 0 ? Gsr0 : Gst[t > 0 ? t - 1 : 0];
-                        const float g_ = Gr + z[t], gs = Gsr - dyC[t];
+                        float g_ = Gr + z[t], gs = Gsr - dyC[t];
+                        if (PK == 8) { g_ = bar ? 0.f : g_; gs = bar ? 0.f : gs; }         // (what the barrier lane fetched is another plane's)
                         const float dbu = fmaf(0.25f, dyC[t], g_ + gs);
                         const float hv = hT[r][n][t], sv = sT[r][n][t];
                         const float h_l = t == CPL - 1 ? hl_last : hT[r][n][t < CPL - 1 ? t + 1 : 0];
@@ -532,6 +537,7 @@ static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStre
     const int share = CPL == 1 ? wave_bwd_share(p.f.shape, wg) : 1;
     const int pk = CPL == 1 ? wave_pack(wg, p.f.shape.ncols) : 1;
     // (packed planes always in blocks of four waves: the planes of a wave are added up where the waves of a block are)
+    if (pk == 8) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 8 : 1>(p, wg, stream);
     if (pk == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 4 : 1>(p, wg, stream);
     if (pk == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 2 : 1>(p, wg, stream);
     if (share == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, 1>(p, wg, stream);

@@ -75,8 +75,9 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
     // scan origin of this group: memory row = r0m + rs*i; with fh the columns run against the memory order
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
-    const int j0 = (w * kSeg + sl) * CPL;            // this lane's first scan column
-    const bool jin = j0 < W;                         // (W is a multiple of CPL: a lane is inside or outside as a whole)
+    const bool bar = PK == 8 && sl == 0;             // (eight planes per wave) the plane's barrier lane
+    const int j0 = PK == 8 ? max(sl - 1, 0) : (w * kSeg + sl) * CPL;   // this lane's first scan column
+    const bool jin = j0 < W && !bar;                 // (W is a multiple of CPL: a lane is inside or outside as a whole)
     const int jc = jin ? j0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
 
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
                     for (int k = 0; k < CPL; ++k) {
                         a[k] = fast_exp2(fmaf(dl[k], A2[n], ld));
                         bu[k] = ((NS == 4 && n >= N) ? 0.f : bu[k]) * du[k];
+                        if (PK == 8) { a[k] = bar ? 0.f : a[k]; bu[k] = bar ? 0.f : bu[k]; }   // the barrier lane's map is (0, 0)
                     }
                     const float a_l = from_prev_lane_pk<PK>(a[CPL - 1], in.z, sl == 0);                // a[i, j-1] of the lane's first column
                     const float h_d = from_prev_lane_pk<PK>(hprev[n][CPL - 1], hdiag[n], sl == 0);     // h[i-1, j-1]
@@ -274,7 +276,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_pa
         // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
-            if ((NS != 4 || n < N) && act && !(SND_WAVE_ABLATE & 16)) {
+            if ((NS != 4 || n < N) && act && !bar && !(SND_WAVE_ABLATE & 16)) {
                 float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
 #pragma unroll
                 for (int k = 0; k < CPL; ++k) {
@@ -342,6 +344,7 @@ static int launch_wave_fwd_p(const snd_fwd_params &p, const WaveGeo &wg, hipStre
 template <typename T, int NS, int CPL, bool VEC>
 static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const int pk = CPL == 1 ? wave_pack(wg, p.shape.ncols) : 1;
+    if (pk == 8) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 8 : 1>(p, wg, stream);
     if (pk == 4) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 4 : 1>(p, wg, stream);
     if (pk == 2) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 2 : 1>(p, wg, stream);
     return launch_wave_fwd_p<T, NS, CPL, VEC, 1>(p, wg, stream);

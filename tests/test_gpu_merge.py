@@ -45,6 +45,7 @@ def _case(gpu_device, Bt, Dm, H, W, N, K, dtype, seed, shared_u):
     (1, 12, 17, 40, 3, 2, torch.float32, capi.SCHED_AUTO, capi.DIR_CORNERS, True, False),      # two groups, three states
     (2, 24, 14, 14, 1, 4, torch.float32, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, True, True),  # four planes per wave, 6 channels per group
     (2, 28, 9, 30, 2, 4, torch.bfloat16, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, False, True), # two planes per wave, 7 channels per group
+    (2, 40, 7, 7, 1, 4, torch.float32, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, True, True),    # eight planes per wave, 10 channels per group
 ])
 def test_fused_merge_matches_two_steps(gpu_device, Bt, Dm, H, W, N, K, dtype, sched, dirs, shared_u, weighted):
     print("merge", Bt, Dm, H, W, N, K, dtype, sched, dirs, shared_u, weighted, flush=True)

@@ -234,7 +234,7 @@ def test_wavefront_shared_atomics(gpu_device, Bt, Dm, H, W, N, K, dtype, kw):
 
 
 PACKED = [
-    # Bt, Dm, H, W, N, K, Dd, dtype, kw: planes of at most 32 / 16 columns, two / four to a wave
+    # Bt, Dm, H, W, N, K, Dd, dtype, kw: planes of at most 32 / 16 / 7 columns, two / four / eight to a wave
     (2, 24, 14, 14, 1, 4, None, torch.float32, {}),            # 6 channels per group: the second wave of a group holds two
     (2, 40, 7, 7, 2, 4, None, torch.bfloat16, {}),
     (3, 36, 9, 16, 4, 2, 18, torch.float32, {}),               # 16 columns exactly; delta shared by pairs of channels
@@ -245,6 +245,14 @@ PACKED = [
     (2, 20, 10, 29, 2, 4, None, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
     (2, 24, 14, 14, 2, 4, None, torch.bfloat16, dict(out_float=False, use_D=False, use_bias=False)),
     (1, 4, 5, 1, 1, 1, None, torch.float32, {}),               # one column, one group
+    # at most 7 columns: eight planes per wave
+    (2, 72, 7, 7, 1, 4, None, torch.float32, {}),              # 18 channels per group
+    (3, 36, 9, 6, 4, 2, 18, torch.float32, {}),                # delta shared by pairs of channels
+    (3, 36, 9, 8, 4, 2, 18, torch.float32, {}),                # 8 columns: four planes per wave again
+    (64, 384, 7, 7, 1, 4, None, torch.bfloat16, {}),
+    (2, 40, 6, 5, 2, 4, None, torch.float16, {}),
+    (2, 24, 7, 7, 1, 4, None, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
+    (2, 20, 10, 7, 3, 4, None, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
 ]
 
 
