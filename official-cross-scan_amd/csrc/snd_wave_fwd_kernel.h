@@ -37,8 +37,12 @@ namespace snd {
 // PK > 1: narrow planes packed PK to a wave (wave_pack() in snd_device.h): lane l works on column l % (64 / PK) of
 // channel PK * chunk + l / (64 / PK) of the group, every per-channel quantity is a lane's own, and the scan stays
 // inside the plane's lanes.  One segment per plane, so nothing is handed over between waves.
-template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK>
-__global__ __launch_bounds__(64 * kMaxSeg) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
+// EU: the waves per SIMD the registers are to leave room for (1: no limit asked for).  A plane of 4 to 8 segments
+// is a block of as many waves; at the 138 registers the kernel takes by itself a CU holds three such blocks of 4
+// waves and one of 6 (the second block's waves do not fit the SIMDs the first left half full), at 128 registers - a
+// few spilled - four and two.
+template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU>
+__global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     constexpr int R = NS <= 1 ? 8 : 4;               // rows per band = rows per load group
     static_assert(PK == 1 || CPL == 1, "packed planes: one column per lane");
     constexpr int S = 64 / PK;                       // lanes per plane
@@ -327,27 +331,34 @@ static inline bool wave_aligned(const void *ptr, int64_t esz, int bytes, std::in
     return true;
 }
 
-template <typename T, int NS, int CPL, bool VEC, int PK>
+template <typename T, int NS, int CPL, bool VEC, int PK, int EU>
 static int launch_wave_fwd_p(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int rg = sh.dim / sh.n_groups;
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + PK - 1) / PK)), block(64 * wg.nseg);
     const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
     constexpr bool F = std::is_same<T, float>::value;
-    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK>), grid, block, 0, stream, p, wg);
-    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F, PK>), grid, block, 0, stream, p, wg);
-    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true, PK>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F, PK>), grid, block, 0, stream, p, wg);
+    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK, EU>), grid, block, 0, stream, p, wg);
+    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F, PK, EU>), grid, block, 0, stream, p, wg);
+    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true, PK, EU>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F, PK, EU>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
 template <typename T, int NS, int CPL, bool VEC>
 static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const int pk = CPL == 1 ? wave_pack(wg, p.shape.ncols) : 1;
-    if (pk == 8) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 8 : 1>(p, wg, stream);
-    if (pk == 4) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 4 : 1>(p, wg, stream);
-    if (pk == 2) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 2 : 1>(p, wg, stream);
-    return launch_wave_fwd_p<T, NS, CPL, VEC, 1>(p, wg, stream);
+    if (pk == 8) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 8 : 1, 1>(p, wg, stream);
+    if (pk == 4) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, 1>(p, wg, stream);
+    if (pk == 2) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 2 : 1, 1>(p, wg, stream);
+    // Planes of 4 to 8 segments, one or two states, and more blocks than the GPU holds at three waves per SIMD (three
+    // blocks of 4 waves per CU, one of more): the instantiation that leaves room for four waves per SIMD.  Measured
+    // 2 x 192 x 200x336, one state: 0.159 -> 0.124 ms; 4 x 256 x 256x256: 0.183 -> 0.163; narrower planes lose 10 %
+    // to the spills and keep the other.
+    constexpr bool kRoomy = NS <= 2 && CPL == 1;
+    const int64_t blocks = (int64_t)p.shape.batch * p.shape.dim;
+    if (kRoomy && wg.nseg >= 4 && blocks > 256 * (wg.nseg == 4 ? 3 : 1)) return launch_wave_fwd_p<T, NS, CPL, VEC, 1, kRoomy ? 4 : 1>(p, wg, stream);
+    return launch_wave_fwd_p<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
 }
 
 template <typename T>

@@ -33,6 +33,9 @@ SHAPES = [
     (2, 8, 33, 256, 1, 4, 4, torch.bfloat16),        # two full segments, shared delta groups
     (1, 4, 12, 1024, 1, 1, None, torch.float16),     # the widest plane: eight segments of 128 columns
     (1, 8, 70, 200, 1, 4, None, torch.bfloat16),
+    # more blocks of 4 to 8 waves than fit at three waves per SIMD: the forward's instantiation with room for four
+    (2, 192, 20, 300, 1, 4, None, torch.float32),
+    (4, 256, 16, 256, 2, 4, None, torch.bfloat16),
 ]
 
 
