@@ -445,28 +445,41 @@ __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, in
 // the next wave through a few LDS words per row.
 struct WaveGeo {
     int nseg;                      // row segments (waves per plane): ceil(W / (64 * cpl))
-    int R;                         // rows per band: row-checkpoint spacing = rows the backward holds in registers
+    int R;                         // rows per band (wave_band_rows): row-checkpoint spacing = rows the backward holds in registers
     int nBands;                    // ceil(H / R)
-    int Hp, Wp;                    // nBands * R, nseg * 64 * cpl
+    int Hp, Wp;                    // nBands * R, nseg * 64 * cpl / planes per wave
     int cpl;                       // columns per lane: 1, or 2 (a lane owns two neighbouring columns: the scan and every
                                    // per-row overhead are paid once per two cells, and loads are twice as wide)
 };
 constexpr int kSeg = 64;
 constexpr int kMaxSeg = 8;
+// Rows per band of the backward = spacing of the forward's row checkpoints.  The backward keeps a band's h, s, a and
+// inputs of every state in registers, and what it gains from short bands is waves per SIMD: with one state 8 rows take
+// 172-190 registers (two waves per SIMD), 4 rows 114-120 (four) - measured 13 to 39 % off the backward from 56x56 down
+// to 7x7 planes, nothing at 512x512 x 256 channels (one block per CU either way), the forward within +-6 %; with two and
+// four states 2 rows instead of 4 take 10 to 20 % off the backward.  The forward walks bands of kWaveFwdRows rows
+// whatever the spacing (shorter bands cost it 5 to 30 %) and only stores the checkpoints more often.
+__host__ __device__ constexpr int wave_band_rows(int N) { return N <= 1 ? 4 : 2; }
+constexpr int kWaveFwdRows = 4;
 // Two columns per lane for one state and rows of 514 to 1024 columns (an even number): eight waves then still
 // cover a row.  Narrower rows keep one column per lane - measured at 256 planes of 512 x 512: the same forward
 // time and a 1.5 x slower backward with two, whose doubled per-lane state leaves one wave per SIMD.  Decided by
 // the shape alone, because the saved state's segment boundaries follow from it.
 __host__ __device__ inline int wave_cpl(int W, int N) { return (N <= 1 && W > kSeg * kMaxSeg && W % 2 == 0) ? 2 : 1; }
 __host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 && W <= kSeg * kMaxSeg * wave_cpl(W, N); }
+// Planes per wave: narrow planes (one segment, at most 32 / 16 / 7 columns) are packed two / four / eight to a wave,
+// plane q of a wave in lanes q*32.. / q*16.. / q*8.. (both kernels of a pair pack alike: the row checkpoints are as
+// wide as a plane's lanes).  With eight planes the first lane of a plane is a barrier lane (wave_scan3_pk) and its
+// columns are in lanes 1..7.
+__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 7 ? 8 : W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
 __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     WaveGeo g;
     g.cpl = wave_cpl(W, N);
     g.nseg = (W + kSeg * g.cpl - 1) / (kSeg * g.cpl);
-    g.R = N <= 1 ? 8 : 4;             // (the backward keeps a band's h, s, a and inputs of every state in registers)
+    g.R = wave_band_rows(N);
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
-    g.Wp = g.nseg * kSeg * g.cpl;
+    g.Wp = g.nseg * kSeg * g.cpl / wave_pack(g, W);   // (packed planes: a row checkpoint is the plane's own lanes wide)
     return g;
 }
 // Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):
@@ -474,11 +487,6 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][2][Wp]        h, then a, on the last row of every band
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
-// Planes per wave: narrow planes (one segment, at most 32 / 16 / 7 columns) are packed two / four / eight to a wave,
-// plane q of a wave in lanes q*32.. / q*16.. / q*8.. (the saved state keeps its layout: either kernel of a pair may
-// pack or not).  With eight planes the first lane of a plane is a barrier lane (wave_scan3_pk) and its columns are in
-// lanes 1..7.
-__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 7 ? 8 : W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all

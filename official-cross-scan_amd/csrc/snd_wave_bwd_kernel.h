@@ -53,14 +53,9 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 //
 // PK > 1 (with CHB > 1): narrow planes packed PK to a wave as in the forward (wave_pack() in snd_device.h); the block
 // then holds CHB * PK channels, and the planes of a wave are added up with the waves of the block.
-//
-// Registers: the one-state fp32 kernel of four-channel blocks is held to 168 (three waves per SIMD; it takes 172 by
-// itself and fits with at most two spilled): 64x192x56x56 0.295 -> 0.268 ms.  The 16-bit variants take 188 and lose
-// 45 % to the spills under the same limit, so they and everything else keep what the compiler gives them.
 template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK>
-__global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(CHB == 4 && PK == 1 && NS == 1 && sizeof(T) == 4 ? 3 : 1)))
-void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
-    constexpr int R = NS <= 1 ? 8 : 4;               // rows per band
+__global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
+    constexpr int R = wave_band_rows(NS);            // rows per band
     static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
     static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
     constexpr int S = 64 / PK;                       // lanes per plane
@@ -523,7 +518,7 @@ static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStre
     const int rg = sh.dim / sh.n_groups;
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + CHB * PK - 1) / (CHB * PK))), block(64 * wg.nseg * CHB);
     constexpr bool F32 = std::is_same<T, float>::value;
-    constexpr int R = NS <= 1 ? 8 : 4;
+    constexpr int R = wave_band_rows(NS);
     // (the even-plane variant only where the loads are prefetched: it is their waits that it makes exact)
     const bool even = NS <= 2 && CPL == 1 && PK == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
     if (even) {

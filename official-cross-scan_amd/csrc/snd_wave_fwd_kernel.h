@@ -18,7 +18,7 @@
 // 2(e-w)+1 and reads what wave w-1 left for those rows in LDS in step e-1 (h, s, a of its last column);
 // one block barrier per step, no polling.  Global loads are whole rows of 64 consecutive elements per
 // wave (one or two full memory lines per instruction), issued a band of rows ahead; nothing is staged
-// through LDS.  Saved for the backward: h, a on the last row of every band of R rows (x_v) and h, s, a
+// through LDS.  Saved for the backward: h, a on the last row of every band of its R rows (x_v) and h, s, a
 // entering every segment on every row (x, x_sd), so that the backward can recompute any band of any
 // segment on its own.
 #pragma once
@@ -43,7 +43,9 @@ namespace snd {
 // few spilled - four and two.
 template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU>
 __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
-    constexpr int R = NS <= 1 ? 8 : 4;               // rows per band = rows per load group
+    constexpr int R = kWaveFwdRows;                  // rows per band of this kernel = rows per load group
+    constexpr int RC = wave_band_rows(NS);           // spacing of the row checkpoints (the backward's bands)
+    static_assert(R % RC == 0, "a band ends on a checkpoint row");
     static_assert(PK == 1 || CPL == 1, "packed planes: one column per lane");
     constexpr int S = 64 / PK;                       // lanes per plane
 #ifndef SND_WAVE_RD
@@ -160,6 +162,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
         for (int k = 0; k < CPL; ++k) { hprev[n][k] = 0.f; aprev[n][k] = 0.f; }
     }
 
+    const int nFB = (H + R - 1) / R;                 // bands of this kernel
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     const bool hands_over = multi && w + 1 < nseg;
     const bool writer = hands_over && lane == 63;
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     // (MERGE_: whether out is accumulated with atomics - decided once around the band loop, not at every row's store)
     auto do_band = [&](auto MERGE_, Stage &cur, Stage &nxt, int band) {
         constexpr bool MERGE = decltype(MERGE_)::value;
-        load_band(nxt, min(band + 1, wg.nBands - 1));   // unconditionally (the last band once more): a skipped load would leave two
+        load_band(nxt, min(band + 1, nFB - 1));   // unconditionally (the last band once more): a skipped load would leave two
                                                         // paths with different numbers of loads in flight, and the waits follow the smaller
         const int i0 = band * R;
         uint32_t oo = mad24(mad24(i0, rs, r0m), OhB * rs, colO);
@@ -274,23 +277,26 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                     }
                 }
                 oo += OhB;
+                // row checkpoint: h, a on the last row of a band of the backward (what its next band starts from; the
+                // last row of the plane is nobody's, and a ragged last band leaves none)
+                if (r % RC == RC - 1) {
+#pragma unroll
+                    for (int n = 0; n < NS; ++n) {
+                        if ((NS != 4 || n < N) && act && !bar && !(SND_WAVE_ABLATE & 16)) {
+                            float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band * (R / RC) + r / RC) * 2 * wg.Wp;
+#pragma unroll
+                            for (int k = 0; k < CPL; ++k) {
+                                __builtin_nontemporal_store(hprev[n][k], dst + k);
+                                __builtin_nontemporal_store(aprev[n][k], dst + wg.Wp + k);
+                            }
+                        }
+                    }
+                }
             }
             if (multi && r % RD == RD - 1) { if (!(SND_WAVE_ABLATE & 2)) lds_barrier(); ++step; }
         }
-        // row checkpoint: h, a on the band's last row (what the next band starts from in the backward)
-#pragma unroll
-        for (int n = 0; n < NS; ++n) {
-            if ((NS != 4 || n < N) && act && !bar && !(SND_WAVE_ABLATE & 16)) {
-                float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)band * 2 * wg.Wp;
-#pragma unroll
-                for (int k = 0; k < CPL; ++k) {
-                    __builtin_nontemporal_store(hprev[n][k], dst + k);
-                    __builtin_nontemporal_store(aprev[n][k], dst + wg.Wp + k);
-                }
-            }
-        }
         // column checkpoints: lanes 0..R-1 hold what entered the segment on the band's rows
-        if (SAVE && w > 0 && lane < R && !(SND_WAVE_ABLATE & 16)) {
+        if (SAVE && w > 0 && lane < R && band * R + lane < wg.Hp && !(SND_WAVE_ABLATE & 16)) {
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 if (NS != 4 || n < N) {
@@ -309,14 +315,14 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     if (multi)
         for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
     if (OUT32 && merge) {
-        for (int band = 0; band < wg.nBands; band += 2) {
+        for (int band = 0; band < nFB; band += 2) {
             do_band(std::true_type{}, sA, sB, band);
-            if (band + 1 < wg.nBands) do_band(std::true_type{}, sB, sA, band + 1);
+            if (band + 1 < nFB) do_band(std::true_type{}, sB, sA, band + 1);
         }
     } else {
-        for (int band = 0; band < wg.nBands; band += 2) {
+        for (int band = 0; band < nFB; band += 2) {
             do_band(std::false_type{}, sA, sB, band);
-            if (band + 1 < wg.nBands) do_band(std::false_type{}, sB, sA, band + 1);
+            if (band + 1 < nFB) do_band(std::false_type{}, sB, sA, band + 1);
         }
     }
     if (multi)
