@@ -35,7 +35,7 @@
 
 namespace snd {
 
-constexpr int kWaveShareWaves = 4;                   // waves of a block whose channels share their dB / dC atomics
+constexpr int kWaveShareWaves = 8;                   // waves of a block whose channels share their dB / dC atomics
 
 __device__ __forceinline__ void wave_glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -503,13 +503,18 @@ static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::
 }
 
 // Channels per block.  Sharing the atomics needs the channels' waves in one block, and a block may hold
-// kWaveShareWaves of them; small launches spread further with one channel per block (measured at 56x56 and 112x112
-// planes: four one-wave channels pay from 512 planes on, two two-wave channels only once the waves fill the GPU).
+// kWaveShareWaves of them; small launches spread further with one channel per block.  Measured: four one-wave
+// channels pay from 512 planes on (56x56); with a full load of waves, one or two states, four channels of two segments
+// (64x96x112x112, two states: 0.85 -> 0.78 ms over two channels) and two channels of three or four segments
+// (4x256x256x256, one state: 0.50 -> 0.33 ms, two states 0.99 -> 0.59; 16x96x160x160: 0.36 -> 0.32); with three or
+// four states two channels of two segments, and no more (blocks of 6 or 8 waves lost 14 to 50 %).
 static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
     const int64_t waves = (int64_t)sh.batch * sh.dim * wg.nseg;
     if (wg.cpl != 1) return 1;
     if (wg.nseg == 1) return waves >= 512 ? 4 : 1;
-    return wg.nseg * 2 <= kWaveShareWaves && waves >= 2048 ? 2 : 1;
+    if (waves < 2048) return 1;
+    if (sh.dstate > 2) return wg.nseg == 2 ? 2 : 1;
+    return wg.nseg * 4 <= kWaveShareWaves ? 4 : wg.nseg * 2 <= kWaveShareWaves ? 2 : 1;
 }
 
 template <typename T, int NS, int CPL, bool VEC, int CHB, int PK>

@@ -202,11 +202,15 @@ SHARED = [
     (4, 512, 9, 20, 4, 4, torch.float16, {}),
     (8, 264, 21, 30, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
     (8, 256, 16, 64, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
-    # two segments per plane and a full load of waves (2048): blocks of two channels
+    # two segments per plane and a full load of waves (2048): blocks of four channels (two with three or four states)
     (4, 264, 12, 100, 1, 4, torch.float32, {}),
     (4, 256, 16, 128, 2, 4, torch.bfloat16, {}),
     (2, 516, 9, 70, 3, 4, torch.float32, {}),
     (4, 264, 13, 90, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
+    # three and four segments per plane, one or two states: blocks of two channels
+    (4, 264, 9, 200, 1, 4, torch.float32, {}),
+    (8, 128, 10, 130, 2, 4, torch.bfloat16, {}),
+    (4, 264, 11, 250, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS)),
 ]
 
 
