@@ -53,15 +53,18 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 //
 // PK > 1 (with CHB > 1): narrow planes packed PK to a wave as in the forward (wave_pack() in snd_device.h); the block
 // then holds CHB * PK channels, and the planes of a wave are added up with the waves of the block.
-template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK>
-__global__ __launch_bounds__(64 * kMaxSeg) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
+//
+// XW: the most waves a block may have, 8 or (two channels of five to eight segments) 16.
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW>
+__global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = wave_band_rows(NS);            // rows per band
     static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
     static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
     constexpr int S = 64 / PK;                       // lanes per plane
     constexpr int kItems = R * NS * 2;               // dB and dC rows of a band
-    constexpr int kXBuf = CHB == 1 ? 1 : NS == 4 ? 1 : 2;   // (with two buffers one barrier per band is enough)
-    constexpr int kXWaves = CHB == 1 ? 1 : kWaveShareWaves;
+    static_assert(XW == kMaxSeg || (CHB == 2 && NS <= 2 && PK == 1), "blocks of 16 waves: two channels, one or two states");
+    constexpr int kXBuf = CHB == 1 ? 1 : (NS == 4 || XW > 8) ? 1 : 2;   // (with two buffers one barrier per band is enough)
+    constexpr int kXWaves = CHB == 1 ? 1 : XW;
     __shared__ float sX[kXBuf][kXWaves][CHB == 1 ? 1 : kItems][CHB == 1 ? 1 : 64];
     // load a band's inputs one band ahead (with four states, or two columns per lane, the registers are needed elsewhere)
     constexpr bool PF = NS <= 2 && CPL == 1;
@@ -507,17 +510,21 @@ static inline bool wave_aligned_b(const void *ptr, int64_t esz, int bytes, std::
 // channels pay from 512 planes on (56x56); with a full load of waves, one or two states, four channels of two segments
 // (64x96x112x112, two states: 0.85 -> 0.78 ms over two channels) and two channels of three or four segments
 // (4x256x256x256, one state: 0.50 -> 0.33 ms, two states 0.99 -> 0.59; 16x96x160x160: 0.36 -> 0.32); with three or
-// four states two channels of two segments, and no more (blocks of 6 or 8 waves lost 14 to 50 %).
+// four states two channels of two segments, and no more (blocks of 6 or 8 waves lost 14 to 50 %).  Planes of five to
+// eight segments, one or two states: two channels in a block of 10 to 16 waves once there are more planes than CUs
+// (2x256x512x512, one state: 1.00 -> 0.67 ms; 4x192x300x300: 0.75 -> 0.71; with 256 planes the blocks would fill half
+// the CUs: 0.46 -> 0.62).
 static inline int wave_bwd_share(const snd_shape &sh, const WaveGeo &wg) {
     const int64_t waves = (int64_t)sh.batch * sh.dim * wg.nseg;
     if (wg.cpl != 1) return 1;
     if (wg.nseg == 1) return waves >= 512 ? 4 : 1;
     if (waves < 2048) return 1;
     if (sh.dstate > 2) return wg.nseg == 2 ? 2 : 1;
-    return wg.nseg * 4 <= kWaveShareWaves ? 4 : wg.nseg * 2 <= kWaveShareWaves ? 2 : 1;
+    if (wg.nseg > 4) return (int64_t)sh.batch * sh.dim > 256 ? 2 : 1;       // blocks of 10 to 16 waves
+    return wg.nseg * 4 <= kWaveShareWaves ? 4 : 2;
 }
 
-template <typename T, int NS, int CPL, bool VEC, int CHB, int PK>
+template <typename T, int NS, int CPL, bool VEC, int CHB, int PK, int XW = kMaxSeg>
 static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const int rg = sh.dim / sh.n_groups;
@@ -528,11 +535,11 @@ static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStre
     const bool even = NS <= 2 && CPL == 1 && PK == 1 && sh.nrows % R == 0 && sh.ncols % (kSeg * CPL) == 0;
     if (even) {
         constexpr bool E = NS <= 2 && CPL == 1 && PK == 1;
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E, CHB, PK>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E, CHB, PK>), grid, block, 0, stream, p, wg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, E, CHB, PK, XW>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, E, CHB, PK, XW>), grid, block, 0, stream, p, wg);
     } else {
-        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false, CHB, PK>), grid, block, 0, stream, p, wg);
-        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false, CHB, PK>), grid, block, 0, stream, p, wg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, true, false, CHB, PK, XW>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, CPL, VEC, F32, false, CHB, PK, XW>), grid, block, 0, stream, p, wg);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
@@ -546,6 +553,7 @@ static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStre
     if (pk == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 4 : 1>(p, wg, stream);
     if (pk == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, CPL == 1 ? 2 : 1>(p, wg, stream);
     if (share == 4) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, 1>(p, wg, stream);
+    if (share == 2 && wg.nseg > 4) return launch_wave_bwd_c<T, NS, CPL, VEC, (CPL == 1 && NS <= 2) ? 2 : 1, 1, (CPL == 1 && NS <= 2) ? 16 : kMaxSeg>(p, wg, stream);
     if (share == 2) return launch_wave_bwd_c<T, NS, CPL, VEC, CPL == 1 ? 2 : 1, 1>(p, wg, stream);
     return launch_wave_bwd_c<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
 }

@@ -211,6 +211,10 @@ SHARED = [
     (4, 264, 9, 200, 1, 4, torch.float32, {}),
     (8, 128, 10, 130, 2, 4, torch.bfloat16, {}),
     (4, 264, 11, 250, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS)),
+    # five to eight segments per plane and more planes than CUs: two channels in a block of 10 to 16 waves
+    (2, 260, 10, 330, 1, 4, torch.float32, {}),                # 65 channels per group: the last block of a group repeats one
+    (2, 264, 8, 512, 2, 4, torch.bfloat16, {}),                # whole bands, whole segments
+    (1, 516, 9, 450, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
 ]
 
 
