@@ -485,7 +485,9 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 // Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):
 //   x    [segment w][2][Hp]   h, then a, at column S*w-1 of every row (what segment w needs from its left)
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
-//   x_v  [band][2][Wp]        h, then a, on the last row of every band
+//   x_v  [band][Wp][2]        (h, a) on the last row of every band: one 8-byte access per column
+typedef float wave_f2 __attribute__((ext_vector_type(2)));
+typedef float wave_f4 __attribute__((ext_vector_type(4)));
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
 

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn0;
+    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + 2 * jn0;
     const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
     const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
 
@@ -194,12 +194,16 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
             if (NS != 4 || n < N) {
                 if (band > 0) {
                     const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
-#pragma unroll
-                    for (int k = 0; k < CPL; ++k) {
-                        q.h0[n][k] = __builtin_nontemporal_load(src + k);
-                        q.a0[n][k] = __builtin_nontemporal_load(src + wg.Wp + k);
-                        if (PK == 8) { q.h0[n][k] = bar ? 0.f : q.h0[n][k]; q.a0[n][k] = bar ? 0.f : q.a0[n][k]; }
+                    if (CPL == 2) {
+                        const wave_f4 v = __builtin_nontemporal_load((const wave_f4 *)src);
+                        q.h0[n][0] = v.x; q.a0[n][0] = v.y; q.h0[n][CPL - 1] = v.z; q.a0[n][CPL - 1] = v.w;
+                    } else {
+                        const wave_f2 v = __builtin_nontemporal_load((const wave_f2 *)src);
+                        q.h0[n][0] = v.x; q.a0[n][0] = v.y;
                     }
+#pragma unroll
+                    for (int k = 0; k < CPL; ++k)
+                        if (PK == 8) { q.h0[n][k] = bar ? 0.f : q.h0[n][k]; q.a0[n][k] = bar ? 0.f : q.a0[n][k]; }
                 }
                 if (w > 0 && lane <= R && row >= 0) {
                     const int64_t o = (int64_t)n * wave_x_plane(wg) + row;

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
 
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j0;
+    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + 2 * j0;
     float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
     float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
 
@@ -284,10 +284,12 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                     for (int n = 0; n < NS; ++n) {
                         if ((NS != 4 || n < N) && act && !bar && !(SND_WAVE_ABLATE & 16)) {
                             float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band * (R / RC) + r / RC) * 2 * wg.Wp;
-#pragma unroll
-                            for (int k = 0; k < CPL; ++k) {
-                                __builtin_nontemporal_store(hprev[n][k], dst + k);
-                                __builtin_nontemporal_store(aprev[n][k], dst + wg.Wp + k);
+                            if (CPL == 2) {
+                                const wave_f4 v = {hprev[n][0], aprev[n][0], hprev[n][CPL - 1], aprev[n][CPL - 1]};
+                                __builtin_nontemporal_store(v, (wave_f4 *)dst);
+                            } else {
+                                const wave_f2 v = {hprev[n][0], aprev[n][0]};
+                                __builtin_nontemporal_store(v, (wave_f2 *)dst);
                             }
                         }
                     }
