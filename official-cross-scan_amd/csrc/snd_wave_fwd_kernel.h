@@ -38,9 +38,9 @@ namespace snd {
 // channel PK * chunk + l / (64 / PK) of the group, every per-channel quantity is a lane's own, and the scan stays
 // inside the plane's lanes.  One segment per plane, so nothing is handed over between waves.
 // EU: the waves per SIMD the registers are to leave room for (1: no limit asked for).  A plane of 4 to 8 segments
-// is a block of as many waves; at the 138 registers the kernel takes by itself a CU holds three such blocks of 4
-// waves and one of 6 (the second block's waves do not fit the SIMDs the first left half full), at 128 registers - a
-// few spilled - four and two.
+// is a block of as many waves; at the 134 registers the two-state kernel takes by itself (three waves per SIMD) a CU
+// holds three such blocks of 4 waves and one of 6 (the second block's waves do not fit the SIMDs the first left half
+// full), at 128 registers - a few spilled - four and two.  (The one-state kernel takes 94 and needs no such variant.)
 template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU>
 __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     constexpr int R = kWaveFwdRows;                  // rows per band of this kernel = rows per load group
@@ -359,11 +359,10 @@ static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStre
     if (pk == 8) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 8 : 1, 1>(p, wg, stream);
     if (pk == 4) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 4 : 1, 1>(p, wg, stream);
     if (pk == 2) return launch_wave_fwd_p<T, NS, CPL, VEC, CPL == 1 ? 2 : 1, 1>(p, wg, stream);
-    // Planes of 4 to 8 segments, one or two states, and more blocks than the GPU holds at three waves per SIMD (three
-    // blocks of 4 waves per CU, one of more): the instantiation that leaves room for four waves per SIMD.  Measured
-    // 2 x 192 x 200x336, one state: 0.159 -> 0.124 ms; 4 x 256 x 256x256: 0.183 -> 0.163; narrower planes lose 10 %
-    // to the spills and keep the other.
-    constexpr bool kRoomy = NS <= 2 && CPL == 1;
+    // Planes of 4 to 8 segments, two states, and more blocks than the GPU holds at three waves per SIMD (three blocks
+    // of 4 waves per CU, one of more): the instantiation that leaves room for four waves per SIMD.  Measured
+    // 2 x 192 x 200x336, two states: 0.242 -> 0.199 ms; narrower planes lose 10 % to the spills and keep the other.
+    constexpr bool kRoomy = NS == 2 && CPL == 1;
     const int64_t blocks = (int64_t)p.shape.batch * p.shape.dim;
     if (kRoomy && wg.nseg >= 4 && blocks > 256 * (wg.nseg == 4 ? 3 : 1)) return launch_wave_fwd_p<T, NS, CPL, VEC, 1, kRoomy ? 4 : 1>(p, wg, stream);
     return launch_wave_fwd_p<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
