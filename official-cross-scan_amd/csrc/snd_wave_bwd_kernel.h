@@ -579,7 +579,7 @@ int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
         return vec ? launch_wave_bwd_v<T, 1, 2, true>(p, wg, stream) : launch_wave_bwd_v<T, 1, 2, false>(p, wg, stream);
     }
     return N == 1 ? launch_wave_bwd_v<T, 1, 1, true>(p, wg, stream) : N == 2 ? launch_wave_bwd_v<T, 2, 1, true>(p, wg, stream)
-                                                                              : launch_wave_bwd_v<T, 4, 1, true>(p, wg, stream);
+         : N == 3 ? launch_wave_bwd_v<T, 3, 1, true>(p, wg, stream) : launch_wave_bwd_v<T, 4, 1, true>(p, wg, stream);
 }
 
 }  // namespace snd
