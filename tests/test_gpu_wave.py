@@ -20,7 +20,7 @@ SHAPES = [
     (1, 4, 1, 200, 2, 2, None, torch.float32),       # single row: 1D scan across four segments
     (1, 4, 33, 1, 2, 1, None, torch.float32),        # single column
     (1, 8, 30, 130, 2, 4, 4, torch.float32),         # three segments, shared delta groups
-    (2, 6, 21, 100, 3, 2, None, torch.float32),      # three states run on the four-state kernels
+    (2, 6, 21, 100, 3, 2, None, torch.float32),      # three states
     (1, 8, 13, 150, 4, 2, None, torch.float32),      # four states: bands of four rows
     (1, 8, 40, 512, 1, 4, None, torch.float32),      # the widest plane: eight segments
     (1, 8, 64, 512, 1, 4, None, torch.bfloat16),
@@ -198,7 +198,7 @@ SHARED = [
     (16, 128, 16, 64, 1, 2, torch.bfloat16, {}),               # whole bands, whole segment
     (8, 256, 12, 40, 2, 4, torch.float32, {}),
     (8, 264, 8, 64, 2, 4, torch.bfloat16, {}),
-    (4, 516, 10, 33, 3, 4, torch.float32, {}),                 # four-state kernel with three states, 129 channels per group
+    (4, 516, 10, 33, 3, 4, torch.float32, {}),                 # three states, 129 channels per group
     (4, 512, 9, 20, 4, 4, torch.float16, {}),
     (8, 264, 21, 30, 1, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, decay=0.9)),
     (8, 256, 16, 64, 2, 4, torch.float32, dict(dirs=capi.DIR_CORNERS, softplus=False)),
