@@ -178,7 +178,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
             wave_ld(q.o[r], dob, oo);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                const int sn = (NS == 4 && n >= N) ? 0 : n;
+                const int sn = n;
                 wave_ld(q.b[r][n], (const T *)((const char *)Bb + sn * BsB), ob);
                 wave_ld(q.c[r][n], (const T *)((const char *)Cb + sn * CsB), oc);
             }
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
             q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
 #pragma unroll
             for (int k = 0; k < CPL; ++k) { q.h0[n][k] = 0.f; q.a0[n][k] = 0.f; }
-            if (NS != 4 || n < N) {
+            {
                 if (band > 0) {
                     const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
                     if (CPL == 2) {
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                     float bm[CPL];
                     unpack(cur.b[r][n], bm);
 #pragma unroll
-                    for (int t = 0; t < CPL; ++t) bn_[r][n][CPL - 1 - t] = (NS == 4 && n >= N) ? 0.f : mirror(bm[t]);
+                    for (int t = 0; t < CPL; ++t) bn_[r][n][CPL - 1 - t] = mirror(bm[t]);
                 }
             }
 #pragma unroll
@@ -354,14 +354,11 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
                     const float4 in = sHO[(step + 1) & 1][kc][w + 1][r][n];
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
-                    const bool live = NS != 4 || n < N;
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
                     unpack(cur.b[r][n], Bv);
                     unpack(cur.c[r][n], Cv);
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
-                        Bv[t] = live ? Bv[t] : 0.f;
-                        Cv[t] = live ? Cv[t] : 0.f;
                         a[t] = aT[r][n][t];
                         bu[t] = Bv[t] * dlu[t];
                         dyC[t] = dov[t] * Cv[t];
@@ -400,7 +397,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                     if (CHB > 1) {
                         sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2][lane] = active ? ya[0] : 0.f;
                         sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2 + 1][lane] = active ? ys[0] : 0.f;
-                    } else if (jin && live && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
+                    } else if (jin && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
 #pragma unroll
                         for (int e = 0; e < CPL; ++e) {                                // memory order
                             const int t = fh ? e : CPL - 1 - e;
@@ -451,7 +448,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                     for (int k = 0; k < PK; ++k) v += sX[kXBuf == 2 ? step & 1 : 0][w + q * nseg][it][PK > 1 ? sl + k * S : lane];
                 float *dst = (float *)((char *)((it & 1) ? dCg : dBg) + n * HW4 + (int64_t)mad24(mad24(i0 + r, rs, r0m), W * 4, (int)col4));
-                if (jin && (PK == 1 || lane < S) && (EVEN || i0 + r < H) && (NS != 4 || n < N)) wave_glb_add(dst, v);
+                if (jin && (PK == 1 || lane < S) && (EVEN || i0 + r < H)) wave_glb_add(dst, v);
             }
             if (kXBuf == 1) lds_barrier();
             ++step;

@@ -138,7 +138,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
             wave_ld(q.d[r], db, od);
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                const int sn = (NS == 4 && n >= N) ? 0 : n;
+                const int sn = n;
                 wave_ld(q.b[r][n], (const T *)((const char *)Bb + sn * BsB), ob);
                 wave_ld(q.c[r][n], (const T *)((const char *)Cb + sn * CsB), oc);
             }
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
 #pragma unroll
                     for (int k = 0; k < CPL; ++k) {
                         a[k] = fast_exp2(fmaf(dl[k], A2[n], ld));
-                        bu[k] = ((NS == 4 && n >= N) ? 0.f : bu[k]) * du[k];
+                        bu[k] = bu[k] * du[k];
                         if (PK == 8) { a[k] = bar ? 0.f : a[k]; bu[k] = bar ? 0.f : bu[k]; }   // the barrier lane's map is (0, 0)
                     }
                     const float a_l = from_prev_lane_pk<PK>(a[CPL - 1], in.z, sl == 0);                // a[i, j-1] of the lane's first column
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                 if (r % RC == RC - 1) {
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
-                        if ((NS != 4 || n < N) && act && !bar && !(SND_WAVE_ABLATE & 16)) {
+                        if (act && !bar && !(SND_WAVE_ABLATE & 16)) {
                             float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band * (R / RC) + r / RC) * 2 * wg.Wp;
                             if (CPL == 2) {
                                 const wave_f4 v = {hprev[n][0], aprev[n][0], hprev[n][CPL - 1], aprev[n][CPL - 1]};
@@ -301,12 +301,10 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
         if (SAVE && w > 0 && lane < R && band * R + lane < wg.Hp && !(SND_WAVE_ABLATE & 16)) {
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
-                if (NS != 4 || n < N) {
-                    const int64_t o = (int64_t)n * wave_x_plane(wg) + band * R + lane;
-                    xh[o] = ch[n];
-                    xh[o + wg.Hp] = ca[n];
-                    xs[o] = cs[n];
-                }
+                const int64_t o = (int64_t)n * wave_x_plane(wg) + band * R + lane;
+                xh[o] = ch[n];
+                xh[o + wg.Hp] = ca[n];
+                xs[o] = cs[n];
             }
         }
     };
