@@ -62,11 +62,13 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
     constexpr int S = 64 / PK;                       // lanes per plane
     constexpr int kItems = R * NS * 2;               // dB and dC rows of a band
+    static_assert(kItems % CHB == 0, "the waves of a segment take equal shares of a band's dB / dC rows");
     static_assert(XW == kMaxSeg || (CHB == 2 && NS <= 2 && PK == 1), "blocks of 16 waves: two channels, one or two states");
     constexpr int kXBuf = CHB == 1 ? 1 : (NS == 4 || XW > 8) ? 1 : 2;   // (with two buffers one barrier per band is enough)
     constexpr int kXWaves = CHB == 1 ? 1 : XW;
     __shared__ float sX[kXBuf][kXWaves][CHB == 1 ? 1 : kItems][CHB == 1 ? 1 : 64];
-    // load a band's inputs one band ahead (with four states, or two columns per lane, the registers are needed elsewhere)
+    // load a band's inputs one band ahead (with three or four states it measured 20 % slower, and with two columns per
+    // lane the registers are needed elsewhere)
     constexpr bool PF = NS <= 2 && CPL == 1;
     // what a wave leaves for the wave on its left: {G, Gs, a, -} at its first column, per band parity, row and
     // state.  Wave w writes slot w and reads slot w+1; the slot after the last wave stays zero.
