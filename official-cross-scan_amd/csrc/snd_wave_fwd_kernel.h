@@ -14,8 +14,8 @@
 // affine maps (a_j, y_j) (and (a_j, bu_j) for s) in six DPP steps, then adds the value entering from
 // the segment on its left: h = Y + A*h[i, 64w-1].  h[i-1,j] and a[i-1,j] are the lane's own registers
 // from the previous row, h[i-1,j-1] and a[i,j-1] come from the lane below (wave_shr:1).
-// The segments of a plane form an anti-diagonal wavefront: in step e wave w works on rows 2(e-w),
-// 2(e-w)+1 and reads what wave w-1 left for those rows in LDS in step e-1 (h, s, a of its last column);
+// The segments of a plane form an anti-diagonal wavefront: in step e wave w works on the four rows 4(e-w) ..
+// 4(e-w)+3 and reads what wave w-1 left for those rows in LDS in step e-1 (h, s, a of its last column);
 // one block barrier per step, no polling.  Global loads are whole rows of 64 consecutive elements per
 // wave (one or two full memory lines per instruction), issued a band of rows ahead; nothing is staged
 // through LDS.  Saved for the backward: h, a on the last row of every band of its R rows (x_v) and h, s, a
