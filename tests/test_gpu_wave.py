@@ -297,3 +297,40 @@ def test_wavefront_packed_planes(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, kw):
             tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
             e = relerr(a.float().cpu().numpy(), w_)
             assert e <= tol, (nm, e)
+
+
+def _draw_large(seed):
+    r = np.random.RandomState(7000 + seed)
+    K = int(r.choice([2, 4]))
+    rg = int(r.randint(33, 131))
+    W = int(r.choice([r.randint(1, 8), r.randint(8, 17), r.randint(17, 33), r.randint(33, 65), r.randint(65, 257), r.randint(257, 513)]))
+    Bt = int(r.choice([1, 2, 4]))
+    if seed % 8 == 7:                                 # wide planes, more of them than CUs: blocks of 10 to 16 waves
+        W, Bt = int(r.randint(257, 513)), 4
+    return dict(Bt=Bt, K=K, Dm=K * rg, H=int(r.randint(1, 41)), W=W, N=int(r.choice([1, 2, 3, 4])),
+                dtype=[torch.float32, torch.bfloat16, torch.float16][int(r.randint(3))], dirs=int(r.randint(2)),
+                decay=0.9 if r.randint(4) == 0 else None)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_wavefront_random_many_planes(gpu_device, seed):
+    """Hundreds to thousands of planes of random size: every way the backward groups channels into blocks (one, two
+    or four channels, two to eight planes per wave, blocks of up to 16 waves) with channel counts that leave ragged
+    last blocks, against the tile kernels on the same inputs."""
+    c = _draw_large(seed)
+    print("wavefront random, many planes", seed, c, flush=True)
+    kw = dict(dirs=c["dirs"], decay=c["decay"], seed=seed)
+    d, t, f, b = run(gpu_device, c["Bt"], c["Dm"], c["H"], c["W"], c["N"], c["K"], None, c["dtype"], capi.SCHED_WAVEFRONT, **kw)
+    _, _, f2, b2 = run(gpu_device, c["Bt"], c["Dm"], c["H"], c["W"], c["N"], c["K"], None, c["dtype"], capi.SCHED_PLANE, **kw)
+    half = c["dtype"] != torch.float32
+    assert relerr(f.out.cpu().numpy(), f2.out.cpu().numpy()) <= 1e-5
+    for nm, a, w_ in zip(NAMES, [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias, b.ddec], [b2.du, b2.ddelta, b2.dA, b2.dB, b2.dC, b2.dD, b2.dbias, b2.ddec]):
+        assert (a is None) == (w_ is None), nm
+        if a is None:
+            continue
+        tol = 1e-2 if (half and nm in ("du", "ddelta")) else (5e-4 if nm == "dA_decay" else 1e-4)
+        # (a single row or column makes some sums identically zero: both families then return rounding noise)
+        ref = w_.float().cpu().numpy()
+        scale = max(float(np.abs(ref).max()), 1e-6)
+        e = float(np.abs(a.float().cpu().numpy().astype(np.float64) - ref).max()) / scale
+        assert e <= tol or float(np.abs(ref).max()) < 1e-9, (nm, e)
