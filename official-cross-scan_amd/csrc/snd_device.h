@@ -485,11 +485,11 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 // Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):
 //   x    [segment w][2][Hp]   h, then a, at column S*w-1 of every row (what segment w needs from its left)
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
-//   x_v  [band][Wp][2]        (h, a) on the last row of every band: one 8-byte access per column
+//   x_v  [band][Wp]           h on the last row of every band (the backward recomputes a of that row from delta)
 typedef float wave_f2 __attribute__((ext_vector_type(2)));
 typedef float wave_f4 __attribute__((ext_vector_type(4)));
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
-__host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * 2 * g.Wp; }
+__host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all
 // channels of a pair share an XCD (and its L2 copy of the pair's B / C planes) as in xcd_job; with few pairs

@@ -155,17 +155,18 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + 2 * jn0;
+    const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn0;
     const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
     const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
 
     // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
     // last columns (always in bounds) and only their dout is masked to zero where it is used, which makes every
-    // adjoint there exactly zero.  h0, a0: the row above the band in natural order.  ch, cs, ca: what entered
+    // adjoint there exactly zero.  h0: h of the row above the band in natural order; dtop: that row's delta (its a is
+    // recomputed).  ch, cs, ca: what entered
     // the segment from the left on rows i0-1 .. i0+R-1, one row per lane.
     typedef WaveRaw<T, CPL, VEC> Raw;
     typedef WaveRaw<DoT, CPL, VEC> RawO;
-    struct In { Raw u[R], d[R], b[R][NS], c[R][NS]; RawO o[R]; float h0[NS][CPL], a0[NS][CPL], ch[NS], cs[NS], ca[NS]; };
+    struct In { Raw u[R], d[R], b[R][NS], c[R][NS]; RawO o[R]; Raw dtop; float h0[NS][CPL], ch[NS], cs[NS], ca[NS]; };
     // Every band issues the same loads on every path (the wait counters the compiler derives for the prefetch
     // need that): rows past the end of a ragged last band read the last row again and are never used.
     auto load_band = [&](In &q, int band) {
@@ -173,6 +174,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         const int m0 = mad24(i0, rs, r0m);           // memory row of the band's first scan row
         uint32_t ou = mad24(m0, UhB * rs, colU), od = mad24(m0, DhB * rs, colD), oo = mad24(m0, DohB * rs, colO),
                  ob = mad24(m0, BhB * rs, colB), oc = mad24(m0, ChB * rs, colB);
+        wave_ld(q.dtop, db, band > 0 ? od - DhB : od);   // (the first band has no row above: any row, never used)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             wave_ld(q.u[r], ub, ou);
@@ -192,20 +194,19 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         for (int n = 0; n < NS; ++n) {
             q.ch[n] = 0.f; q.cs[n] = 0.f; q.ca[n] = 0.f;
 #pragma unroll
-            for (int k = 0; k < CPL; ++k) { q.h0[n][k] = 0.f; q.a0[n][k] = 0.f; }
+            for (int k = 0; k < CPL; ++k) q.h0[n][k] = 0.f;
             {
                 if (band > 0) {
-                    const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * 2 * wg.Wp;
+                    const float *src = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band - 1) * wg.Wp;
                     if (CPL == 2) {
-                        const wave_f4 v = __builtin_nontemporal_load((const wave_f4 *)src);
-                        q.h0[n][0] = v.x; q.a0[n][0] = v.y; q.h0[n][CPL - 1] = v.z; q.a0[n][CPL - 1] = v.w;
-                    } else {
                         const wave_f2 v = __builtin_nontemporal_load((const wave_f2 *)src);
-                        q.h0[n][0] = v.x; q.a0[n][0] = v.y;
+                        q.h0[n][0] = v.x; q.h0[n][CPL - 1] = v.y;
+                    } else {
+                        q.h0[n][0] = __builtin_nontemporal_load(src);
                     }
 #pragma unroll
                     for (int k = 0; k < CPL; ++k)
-                        if (PK == 8) { q.h0[n][k] = bar ? 0.f : q.h0[n][k]; q.a0[n][k] = bar ? 0.f : q.a0[n][k]; }
+                        if (PK == 8) q.h0[n][k] = bar ? 0.f : q.h0[n][k];
                 }
                 if (w > 0 && lane <= R && row >= 0) {
                     const int64_t o = (int64_t)n * wave_x_plane(wg) + row;
@@ -245,13 +246,24 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         float hT[R][NS][CPL], sT[R][NS][CPL], aT[R][NS][CPL], dl[R][CPL], dsp[R][CPL], uu[R][CPL], hTop[NS][CPL];
         {
             float hp[NS][CPL], ap[NS][CPL], hdiag[NS];
+            // a of the row above the band, from that row's delta (zero above the first band, and in a barrier lane)
+            float dtop[CPL];
+            unpack(cur.dtop, dtop);
+#pragma unroll
+            for (int t = 0; t < CPL; ++t) {
+                const float raw = dtop[t] + bias;
+                float sg;
+                dtop[t] = softplus ? softplus20(raw, sg) : raw;
+            }
 #pragma unroll
             for (int n = 0; n < NS; ++n) {
                 hdiag[n] = bcast(cur.ch[n], 0);
 #pragma unroll
                 for (int k = 0; k < CPL; ++k) {
                     hp[n][k] = cur.h0[n][k];
-                    ap[n][k] = cur.a0[n][k];
+                    const float at = band > 0 ? fast_exp2(fmaf(dtop[CPL - 1 - k], A2[n], ld)) : 0.f;
+                    ap[n][k] = mirror(at);
+                    if (PK == 8) ap[n][k] = bar ? 0.f : ap[n][k];
                     hTop[n][CPL - 1 - k] = mirror(cur.h0[n][k]);
                 }
             }

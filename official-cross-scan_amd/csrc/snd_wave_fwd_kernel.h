@@ -18,7 +18,7 @@
 // 4(e-w)+3 and reads what wave w-1 left for those rows in LDS in step e-1 (h, s, a of its last column);
 // one block barrier per step, no polling.  Global loads are whole rows of 64 consecutive elements per
 // wave (one or two full memory lines per instruction), issued a band of rows ahead; nothing is staged
-// through LDS.  Saved for the backward: h, a on the last row of every band of its R rows (x_v) and h, s, a
+// through LDS.  Saved for the backward: h on the last row of every band of its R rows (x_v) and h, s, a
 // entering every segment on every row (x, x_sd), so that the backward can recompute any band of any
 // segment on its own.
 #pragma once
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
 
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
-    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + 2 * j0;
+    float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j0;
     float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
     float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
 
@@ -277,19 +277,18 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                     }
                 }
                 oo += OhB;
-                // row checkpoint: h, a on the last row of a band of the backward (what its next band starts from; the
+                // row checkpoint: h on the last row of a band of the backward (what its next band starts from; the
                 // last row of the plane is nobody's, and a ragged last band leaves none)
                 if (r % RC == RC - 1) {
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
                         if (act && !bar && !(SND_WAVE_ABLATE & 16)) {
-                            float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band * (R / RC) + r / RC) * 2 * wg.Wp;
+                            float *dst = xv + (int64_t)n * wave_xv_plane(wg) + (int64_t)(band * (R / RC) + r / RC) * wg.Wp;
                             if (CPL == 2) {
-                                const wave_f4 v = {hprev[n][0], aprev[n][0], hprev[n][CPL - 1], aprev[n][CPL - 1]};
-                                __builtin_nontemporal_store(v, (wave_f4 *)dst);
-                            } else {
-                                const wave_f2 v = {hprev[n][0], aprev[n][0]};
+                                const wave_f2 v = {hprev[n][0], hprev[n][CPL - 1]};
                                 __builtin_nontemporal_store(v, (wave_f2 *)dst);
+                            } else {
+                                __builtin_nontemporal_store(hprev[n][0], dst);
                             }
                         }
                     }
