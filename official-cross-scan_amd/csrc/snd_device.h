@@ -487,7 +487,6 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][Wp]           h on the last row of every band (the backward recomputes a of that row from delta)
 typedef float wave_f2 __attribute__((ext_vector_type(2)));
-typedef float wave_f4 __attribute__((ext_vector_type(4)));
 __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * g.Wp; }
 
