@@ -11,10 +11,13 @@ from test_gpu_fwd import relerr
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("sched", [capi.SCHED_PLANE, capi.SCHED_STRIPS, capi.SCHED_BANDS])
-def test_graph_replays_match_eager(gpu_device, sched):
-    print("graph", sched, flush=True)
-    d = O.make_inputs(2, 16, 40, 24, N=16, K=4, seed=13)
+@pytest.mark.parametrize("sched,dims", [(capi.SCHED_PLANE, (2, 16, 40, 24, 16)), (capi.SCHED_STRIPS, (2, 16, 40, 24, 16)),
+                                        (capi.SCHED_BANDS, (2, 16, 40, 24, 16)),
+                                        # the row-segment kernels: packed planes in four-wave blocks; three segments
+                                        (capi.SCHED_WAVEFRONT, (4, 160, 14, 14, 1)), (capi.SCHED_WAVEFRONT, (2, 16, 40, 150, 2))])
+def test_graph_replays_match_eager(gpu_device, sched, dims):
+    print("graph", sched, dims, flush=True)
+    d = O.make_inputs(*dims[:4], N=dims[4], K=4, seed=13)
     t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
     args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
 
@@ -51,5 +54,5 @@ def test_graph_replays_match_eager(gpu_device, sched):
         for i, (a, w) in enumerate(zip(got, want)):
             tol = 0.0 if i < 3 else 1e-5                 # atomic sums may differ in order
             assert relerr(a.cpu().numpy(), w.cpu().numpy()) <= tol, (rep, i)
-        if sched != capi.SCHED_PLANE:
+        if sched not in (capi.SCHED_PLANE, capi.SCHED_WAVEFRONT):
             assert int(f.ws.view(torch.int32)[1]) == 0 and int(b.ws.view(torch.int32)[1]) == 0
