@@ -457,10 +457,12 @@ constexpr int kMaxSeg = 8;
 // inputs of every state in registers, and what it gains from short bands is waves per SIMD: with one state 8 rows take
 // 172-190 registers (two waves per SIMD), 4 rows 114-120 (four) - measured 13 to 39 % off the backward from 56x56 down
 // to 7x7 planes, nothing at 512x512 x 256 channels (one block per CU either way), the forward within +-6 %; with two and
-// four states 2 rows instead of 4 take 10 to 20 % off the backward.  The forward walks bands of kWaveFwdRows rows
-// whatever the spacing (shorter bands cost it 5 to 30 %) and only stores the checkpoints more often.
+// four states 2 rows instead of 4 take 10 to 20 % off the backward.  The forward walks bands of its own height
+// (load groups and wavefront steps) whatever the spacing and only stores the checkpoints more often: 4 rows with one
+// and two states (2-row bands cost it 5 to 30 %), 2 rows with three and four, where the registers of a 4-row load
+// group leave two waves per SIMD (192-245 registers; 64x192x56x56, four states: 0.352 -> 0.303 ms).
 __host__ __device__ constexpr int wave_band_rows(int N) { return N <= 1 ? 4 : 2; }
-constexpr int kWaveFwdRows = 4;
+__host__ __device__ constexpr int wave_fwd_rows(int N) { return N <= 2 ? 4 : 2; }
 // Two columns per lane for one state and rows of 514 to 1024 columns (an even number): eight waves then still
 // cover a row.  Narrower rows keep one column per lane - measured at 256 planes of 512 x 512: the same forward
 // time and a 1.5 x slower backward with two, whose doubled per-lane state leaves one wave per SIMD.  Decided by

@@ -43,7 +43,7 @@ namespace snd {
 // full), at 128 registers - a few spilled - four and two.  (The one-state kernel takes 94 and needs no such variant.)
 template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU>
 __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
-    constexpr int R = kWaveFwdRows;                  // rows per band of this kernel = rows per load group
+    constexpr int R = wave_fwd_rows(NS);             // rows per band of this kernel = rows per load group
     constexpr int RC = wave_band_rows(NS);           // spacing of the row checkpoints (the backward's bands)
     static_assert(R % RC == 0, "a band ends on a checkpoint row");
     static_assert(PK == 1 || CPL == 1, "packed planes: one column per lane");
