@@ -126,21 +126,21 @@ bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 //     row of its segment in about 0.85 us (one state), 1.5 (two), 2.95 (three or four), whatever the row's width.
 //     Where four channels share their dB / dC atomics (one segment per plane, 512 planes or more) a row takes 0.7,
 //     1.15, 2.4 us.  Planes of at most 32 / 16 columns are packed two / four to a wave, whose row then takes 0.65,
-//     1.05, 2.05 us; planes of at most 7 columns eight to a wave, 0.75, 1.15, 2.4 us.
+//     1.05, 2.05 us; planes of at most 7 columns eight to a wave, 0.75, 1.15, 2.2 us.
 //   * tile kernels with four lanes per channel: a block is one wave of 16 channels, 1024 fit at once, and a block
 //     takes one 8x8 (7x7) tile in about 18.5 us - or, with few blocks and many strips, the strip pipeline takes
 //     (column tiles + strips - 1) steps of about 25 us per round of its jobs.
-// With four states, planes of 7x7 and of 33 to 40 columns go to the tile kernels (32 x 12288 x 7x7: 0.65 ms forward +
-// backward instead of 0.69; 32 x 384 x 40x40: 0.65 instead of 0.80), everything else to the wavefront (32 x 3072 x
-// 14x14, one state: 0.18 ms instead of 0.60; 32 x 192 x 56x56, one state: 0.18 instead of 0.67; 512x512 x 256
-// channels, one state: 0.65 instead of 3.2).
+// With four states, planes of 33 to 40 columns go to the tile kernels (32 x 384 x 40x40: 0.65 ms forward + backward
+// instead of 0.73), everything else to the wavefront (32 x 12288 x 7x7, four states: 0.59 ms instead of 0.65; 32 x 3072
+// x 14x14, one state: 0.18 instead of 0.60; 32 x 192 x 56x56, one state: 0.18 instead of 0.67; 512x512 x 256 channels,
+// one state: 0.65 instead of 3.2).
 bool wave_family_pays(const snd_shape &s) {
     const snd::Geo g = snd::make_geo(s.nrows, s.ncols);
     const snd::WaveGeo wg = snd::make_wave_geo(s.nrows, s.ncols, s.dstate);
     const int pk = snd::wave_pack(wg, s.ncols);
     const int64_t waves = ((int64_t)s.batch * s.dim + pk - 1) / pk * wg.nseg;
     const bool shared = wg.nseg == 1 && waves >= 512;        // (wave_bwd_share() of the backward's launcher)
-    const double t_row = pk == 8 ? (s.dstate <= 1 ? 0.75 : s.dstate == 2 ? 1.15 : 2.4) : pk > 1 ? (s.dstate <= 1 ? 0.65 : s.dstate == 2 ? 1.05 : 2.05)
+    const double t_row = pk == 8 ? (s.dstate <= 1 ? 0.75 : s.dstate == 2 ? 1.15 : 2.2) : pk > 1 ? (s.dstate <= 1 ? 0.65 : s.dstate == 2 ? 1.05 : 2.05)
                        : shared ? (s.dstate <= 1 ? 0.7 : s.dstate == 2 ? 1.15 : 2.4) : (s.dstate <= 1 ? 0.85 : s.dstate == 2 ? 1.5 : 2.95);
     const double t_wave = (double)((waves + 2047) / 2048) * (wg.Hp + (wg.nseg - 1) * wg.R) * t_row;
     const int64_t blocks = plane_chunks(s);
