@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     // Only lane 63 of a wave has something to hand over.  Instead of masking the other lanes off (a compare, two
     // exec writes and a branch around every hand-over store), every lane stores: lane 63 to the slot, the others to
     // a word of their own that nobody reads.  One wave instruction costs the wave the same issue time either way.
-    __shared__ float4 sDump[64 * kMaxSeg + RD * NS];
+    __shared__ float4 sDump[PK > 1 ? 1 : 64 * kMaxSeg + RD * NS];      // (packed planes: one wave per block, nothing to hand over)
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     const bool hands_over = multi && w + 1 < nseg;
     const bool writer = hands_over && lane == 63;
-    float4 *const dump = &sDump[threadIdx.x];
+    float4 *const dump = &sDump[PK > 1 ? 0 : threadIdx.x];
 
     // one band of rows from `cur`, with the next band's loads issued into `nxt` first
     // (MERGE_: whether out is accumulated with atomics - decided once around the band loop, not at every row's store)
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
         float4 *wr = dump;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (r % RD == 0 && HOIST_IN && !(SND_WAVE_ABLATE & 32)) {
+            if (r % RD == 0 && HOIST_IN && PK == 1 && !(SND_WAVE_ABLATE & 32)) {
 #pragma unroll
                 for (int q = 0; q < RD; ++q)
 #pragma unroll
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column S*w-1
-                    const float4 in = (SND_WAVE_ABLATE & 32) ? make_float4(0.f, 0.f, 0.f, 0.f)
+                    const float4 in = ((SND_WAVE_ABLATE & 32) || PK > 1) ? make_float4(0.f, 0.f, 0.f, 0.f)
                                       : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
                     float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
                     unpack(cur.b[r][n], bu);
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                         aprev[n][k] = a[k];
                     }
                     hdiag[n] = in.x;
-                    if (!(SND_WAVE_ABLATE & 32)) {
+                    if (PK == 1 && !(SND_WAVE_ABLATE & 32)) {
                         wr[(r % RD) * NS + n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
                     }
                     if (SAVE) {                     // lane r keeps what entered the segment on row r (selects, no branch)
