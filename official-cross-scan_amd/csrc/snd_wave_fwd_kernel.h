@@ -41,8 +41,11 @@ namespace snd {
 // is a block of as many waves; at the 134 registers the two-state kernel takes by itself (three waves per SIMD) a CU
 // holds three such blocks of 4 waves and one of 6 (the second block's waves do not fit the SIMDs the first left half
 // full), at 128 registers - a few spilled - four and two.  (The one-state kernel takes 94 and needs no such variant.)
-template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU>
-__global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
+// ONE: the plane is one segment wide (always so with packed planes): one wave per block, nothing is handed over and
+// no LDS is used.
+template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU, bool ONE>
+__global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
+    static_assert(ONE || PK == 1, "packed planes are one segment wide");
     constexpr int R = wave_fwd_rows(NS);             // rows per band of this kernel = rows per load group
     constexpr int RC = wave_band_rows(NS);           // spacing of the row checkpoints (the backward's bands)
     static_assert(R % RC == 0, "a band ends on a checkpoint row");
@@ -59,7 +62,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     // Only lane 63 of a wave has something to hand over.  Instead of masking the other lanes off (a compare, two
     // exec writes and a branch around every hand-over store), every lane stores: lane 63 to the slot, the others to
     // a word of their own that nobody reads.  One wave instruction costs the wave the same issue time either way.
-    __shared__ float4 sDump[PK > 1 ? 1 : 64 * kMaxSeg + RD * NS];      // (packed planes: one wave per block, nothing to hand over)
+    __shared__ float4 sDump[ONE ? 1 : 64 * kMaxSeg + RD * NS];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
     int step = w;                                    // wavefront step this wave is in (parity selects the LDS buffer)
     const bool hands_over = multi && w + 1 < nseg;
     const bool writer = hands_over && lane == 63;
-    float4 *const dump = &sDump[PK > 1 ? 0 : threadIdx.x];
+    float4 *const dump = &sDump[ONE ? 0 : threadIdx.x];
 
     // one band of rows from `cur`, with the next band's loads issued into `nxt` first
     // (MERGE_: whether out is accumulated with atomics - decided once around the band loop, not at every row's store)
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
         float4 *wr = dump;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (r % RD == 0 && HOIST_IN && PK == 1 && !(SND_WAVE_ABLATE & 32)) {
+            if (r % RD == 0 && HOIST_IN && !ONE && !(SND_WAVE_ABLATE & 32)) {
 #pragma unroll
                 for (int q = 0; q < RD; ++q)
 #pragma unroll
@@ -222,7 +225,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column S*w-1
-                    const float4 in = ((SND_WAVE_ABLATE & 32) || PK > 1) ? make_float4(0.f, 0.f, 0.f, 0.f)
+                    const float4 in = ((SND_WAVE_ABLATE & 32) || ONE) ? make_float4(0.f, 0.f, 0.f, 0.f)
                                       : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
                     float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
                     unpack(cur.b[r][n], bu);
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU
                         aprev[n][k] = a[k];
                     }
                     hdiag[n] = in.x;
-                    if (PK == 1 && !(SND_WAVE_ABLATE & 32)) {
+                    if (!ONE && !(SND_WAVE_ABLATE & 32)) {
                         wr[(r % RD) * NS + n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
                     }
                     if (SAVE) {                     // lane r keeps what entered the segment on row r (selects, no branch)
@@ -336,18 +339,25 @@ static inline bool wave_aligned(const void *ptr, int64_t esz, int bytes, std::in
     return true;
 }
 
-template <typename T, int NS, int CPL, bool VEC, int PK, int EU>
-static int launch_wave_fwd_p(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+template <typename T, int NS, int CPL, bool VEC, int PK, int EU, bool ONE>
+static int launch_wave_fwd_o(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int rg = sh.dim / sh.n_groups;
     const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + PK - 1) / PK)), block(64 * wg.nseg);
     const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
     constexpr bool F = std::is_same<T, float>::value;
-    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK, EU>), grid, block, 0, stream, p, wg);
-    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F, PK, EU>), grid, block, 0, stream, p, wg);
-    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true, PK, EU>), grid, block, 0, stream, p, wg);
-    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F, PK, EU>), grid, block, 0, stream, p, wg);
+    if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK, EU, ONE>), grid, block, 0, stream, p, wg);
+    else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, F, PK, EU, ONE>), grid, block, 0, stream, p, wg);
+    else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, true, PK, EU, ONE>), grid, block, 0, stream, p, wg);
+    else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, false, F, PK, EU, ONE>), grid, block, 0, stream, p, wg);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+template <typename T, int NS, int CPL, bool VEC, int PK, int EU>
+static int launch_wave_fwd_p(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
+    constexpr bool kOne = CPL == 1 && EU == 1;       // (the one-segment instantiation exists where it can be asked for)
+    if (PK > 1 || (kOne && wg.nseg == 1)) return launch_wave_fwd_o<T, NS, CPL, VEC, PK, EU, (PK > 1 || kOne)>(p, wg, stream);
+    return launch_wave_fwd_o<T, NS, CPL, VEC, PK, EU, (PK > 1)>(p, wg, stream);
 }
 
 template <typename T, int NS, int CPL, bool VEC>
