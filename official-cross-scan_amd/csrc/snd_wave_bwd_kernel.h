@@ -368,7 +368,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
-                    const float4 in = sHO[(step + 1) & 1][kc][w + 1][r][n];
+                    const float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
                     unpack(cur.b[r][n], Bv);
