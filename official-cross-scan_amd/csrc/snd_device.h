@@ -450,9 +450,13 @@ struct WaveGeo {
     int Hp, Wp;                    // nBands * R, nseg * 64 * cpl / planes per wave
     int cpl;                       // columns per lane: 1, or 2 (a lane owns two neighbouring columns: the scan and every
                                    // per-row overhead are paid once per two cells, and loads are twice as wide)
+    int rg, rd, gshift, xcd;       // set by the launchers (wave_geo_channels): channels per group, channels per delta
+                                   // channel, log2(groups) or -1, the block mapping (wave_job2) - divisions a wave
+                                   // of a 7-row plane would spend a fifth of its instructions on
 };
 constexpr int kSeg = 64;
 constexpr int kMaxSeg = 8;
+constexpr int kOneWaves = 4;         // waves per block of the forward's one-segment instantiation
 // Rows per band of the backward = spacing of the forward's row checkpoints.  The backward keeps a band's h, s, a and
 // inputs of every state in registers, and what it gains from short bands is waves per SIMD: with one state 8 rows take
 // 172-190 registers (two waves per SIMD), 4 rows 114-120 (four) - measured 13 to 39 % off the backward from 56x56 down
@@ -482,6 +486,7 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
     g.Wp = g.nseg * kSeg * g.cpl / wave_pack(g, W);   // (packed planes: a row checkpoint is the plane's own lanes wide)
+    g.rg = g.rd = 1; g.gshift = 0; g.xcd = 0;
     return g;
 }
 // Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):
@@ -495,13 +500,38 @@ __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all
 // channels of a pair share an XCD (and its L2 copy of the pair's B / C planes) as in xcd_job; with few pairs
 // that would leave XCDs idle, so the channels are dealt over all of them (B / C of few pairs are small).
-__device__ __forceinline__ bool wave_job(int bid, int nPairs, int rg, int &pair, int &chunk) {
-    if (nPairs >= 16 || (nPairs & 7) == 0) return xcd_job(bid, nPairs, rg, pair, chunk);
-    pair = bid / rg;
-    chunk = bid - pair * rg;
+__host__ inline int wave_grid(int nPairs, int rg) { return (nPairs >= 16 || (nPairs & 7) == 0) ? xcd_grid(nPairs, rg) : nPairs * rg; }
+// The same mapping without a division: a grid of (8 * chunks, ceil(pairs / 8)) blocks is dispatched x first, so block
+// (x, y) is the (8 * (y * chunks + x / 8) + x % 8)-th and lands on XCD x % 8 like block 8 * k + xcd of the flat grid.
+// (WaveGeo.xcd says which of the two mappings the launcher chose.)
+__host__ inline bool wave_grid_xcd(int nPairs) { return (nPairs >= 16 || (nPairs & 7) == 0) && (nPairs + 7) / 8 <= 65535; }
+__host__ inline dim3 wave_grid2(int nPairs, int nChunks) {
+    if (wave_grid_xcd(nPairs)) return dim3(8 * nChunks, (nPairs + 7) / 8);
+    return dim3(nChunks, nPairs < 65535 ? nPairs : 65535, (nPairs + 65534) / 65535);
+}
+__device__ __forceinline__ bool wave_job2(const WaveGeo &g, int nPairs, int &pair, int &chunk) {
+    if (g.xcd) {
+        pair = blockIdx.y * 8 + (blockIdx.x & 7);
+        chunk = blockIdx.x >> 3;
+    } else {
+        pair = blockIdx.z * 65535 + blockIdx.y;
+        chunk = blockIdx.x;
+    }
     return pair < nPairs;
 }
-__host__ inline int wave_grid(int nPairs, int rg) { return (nPairs >= 16 || (nPairs & 7) == 0) ? xcd_grid(nPairs, rg) : nPairs * rg; }
+__host__ inline void wave_geo_channels(WaveGeo &g, int batch, int dim, int n_groups, int delta_dim) {
+    g.xcd = wave_grid_xcd(batch * n_groups) ? 1 : 0;
+    g.rg = dim / n_groups;
+    g.rd = dim / delta_dim;
+    g.gshift = -1;
+    for (int k = 0; k < 16; ++k)
+        if (n_groups == 1 << k) g.gshift = k;
+}
+// (batch, group) of a pair
+__device__ __forceinline__ void wave_pair_split(const WaveGeo &g, int pair, int G, int &b, int &grp) {
+    b = g.gshift >= 0 ? pair >> g.gshift : pair / G;
+    grp = pair - b * G;
+}
 // Row inputs of the wavefront kernels wait in registers as raw bits for a band of rows and are converted
 // where they are used (a conversion at the load would put the wait for the load there).  They are loaded
 // without any lane condition: a load whose result is only needed under a lane condition is sunk into that

@@ -79,19 +79,21 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
-    const int rg = Dm / G, rd = Dm / sh.delta_dim;
+    const int rg = wg.rg, rd = wg.rd;
     const int nseg = wg.nseg;
     const int lane = threadIdx.x & 63, wi = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int kc = CHB > 1 ? wi / nseg : 0, w = PK > 1 ? 0 : wi - kc * nseg;     // channel of the block, segment of the channel
     const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
     int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, (rg + CHB * PK - 1) / (CHB * PK), pair, chunk)) return;
+    if (!wave_job2(wg, sh.batch * G, pair, chunk)) return;
     chunk = (chunk * CHB + kc) * PK + (PK > 1 ? lane / S : 0);       // (packed: a lane's own from here on)
     // A wave (a plane of a wave) past the last channel of its group repeats that channel (identical du / ddelta
     // stores) and adds nothing.
     const bool active = CHB == 1 || chunk < rg;
     chunk = min(chunk, rg - 1);
-    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
+    int b, g;
+    wave_pair_split(wg, pair, G, b, g);
+    const int c = g * rg + chunk, cd = rd == 1 ? c : c / rd;   // channel of u, of delta
     // channel offsets: in the scalar base pointers, or (packed) in the lanes' offsets
     const int cB = PK > 1 ? 0 : c, chB = PK > 1 ? 0 : chunk, cL = PK > 1 ? c : 0, chL = PK > 1 ? chunk : 0;
     const bool multi = nseg > 1;
@@ -121,12 +123,12 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     float Av[NS], A2[NS];
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
-        Av[n] = n < N ? f.A[(int64_t)c * f.A_d_stride + (int64_t)n * f.A_dstate_stride] : 0.f;
+        Av[n] = f.A[(int64_t)c * f.A_d_stride + (int64_t)n * f.A_dstate_stride];   // (NS == N)
         A2[n] = Av[n] * kLog2e;
     }
     const float ld = f.A_decay ? __log2f(f.A_decay[0]) : 0.f;
     const float Dv = f.D ? f.D[c] : 0.f;
-    const float bias = f.delta_bias ? f.delta_bias[c / rd] : 0.f;
+    const float bias = f.delta_bias ? f.delta_bias[cd] : 0.f;
     const bool softplus = f.delta_softplus != 0;
     const bool want_decay = p.dA_decay != nullptr;
 
@@ -136,7 +138,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const T *Bb = (const T *)f.B + (int64_t)b * f.B_batch_stride + (int64_t)g * f.B_group_stride;
     const T *Cb = (const T *)f.C + (int64_t)b * f.C_batch_stride + (int64_t)g * f.C_group_stride;
     const T *ub = (const T *)f.u + (int64_t)b * f.u_batch_stride + (int64_t)(f.u_shared ? chB : cB) * f.u_d_stride;
-    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(cB / rd) * f.delta_d_stride;
+    const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(PK > 1 ? 0 : cd) * f.delta_d_stride;
     // fused CrossMerge: dout is the gradient of the merged output, shared by the groups and scaled by the channel's weight
     const bool merge = f.merge != 0;
     const float wm = merge && f.merge_weights ? f.merge_weights[c] : 1.f;
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const int64_t BsB = f.B_dstate_stride * ESZ, CsB = f.C_dstate_stride * ESZ, HW4 = (int64_t)H * W * 4;
     const uint32_t colB = (uint32_t)mc * ESZ, col4 = (uint32_t)mc * 4;
     const uint32_t colU = colB + (uint32_t)(f.u_shared ? chL : cL) * (uint32_t)f.u_d_stride * ESZ,
-                   colD = colB + (uint32_t)(cL / rd) * (uint32_t)f.delta_d_stride * ESZ,
+                   colD = colB + (uint32_t)(PK > 1 ? cd : 0) * (uint32_t)f.delta_d_stride * ESZ,
                    colO = (uint32_t)mc * DSZ + (uint32_t)(merge ? chL : cL) * (uint32_t)p.dout_d_stride * DSZ,
                    colG = colB + (uint32_t)cL * (uint32_t)(H * W) * ESZ;                  // du, ddelta
 
@@ -545,7 +547,7 @@ template <typename T, int NS, int CPL, bool VEC, int CHB, int PK, int XW = kMaxS
 static int launch_wave_bwd_c(const snd_bwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const int rg = sh.dim / sh.n_groups;
-    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + CHB * PK - 1) / (CHB * PK))), block(64 * wg.nseg * CHB);
+    const dim3 grid = wave_grid2(sh.batch * sh.n_groups, (rg + CHB * PK - 1) / (CHB * PK)), block(64 * wg.nseg * CHB);
     constexpr bool F32 = std::is_same<T, float>::value;
     constexpr int R = wave_band_rows(NS);
     // (the even-plane variant only where the loads are prefetched: it is their waits that it makes exact)
@@ -580,7 +582,8 @@ int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
     const int N = sh.dstate;
-    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.dout_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned_b(f.u, e, 2 * e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&

@@ -41,10 +41,12 @@ namespace snd {
 // is a block of as many waves; at the 134 registers the two-state kernel takes by itself (three waves per SIMD) a CU
 // holds three such blocks of 4 waves and one of 6 (the second block's waves do not fit the SIMDs the first left half
 // full), at 128 registers - a few spilled - four and two.  (The one-state kernel takes 94 and needs no such variant.)
-// ONE: the plane is one segment wide (always so with packed planes): one wave per block, nothing is handed over and
-// no LDS is used.
+// ONE: the plane is one segment wide (always so with packed planes): nothing is handed over and no LDS is used.  A
+// block is kOneWaves independent waves, each with a channel (PK channels) of its own, a quarter of the blocks to hand
+// out (measured against blocks of one wave, bf16, one state: 64 x 1536 x 14x14 0.055 -> 0.049 ms, 64 x 768 x 14x14
+// 0.035 -> 0.031, 64 x 3072 x 7x7 unchanged at 0.051).
 template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU, bool ONE>
-__global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
+__global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     static_assert(ONE || PK == 1, "packed planes are one segment wide");
     constexpr int R = wave_fwd_rows(NS);             // rows per band of this kernel = rows per load group
     constexpr int RC = wave_band_rows(NS);           // spacing of the row checkpoints (the backward's bands)
@@ -66,20 +68,26 @@ __global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_wave
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
-    const int rg = Dm / G, rd = Dm / sh.delta_dim;
+    const int rg = wg.rg, rd = wg.rd;
     int pair, chunk;
-    if (!wave_job(blockIdx.x, sh.batch * G, (rg + PK - 1) / PK, pair, chunk)) return;
-    const int lane = threadIdx.x & 63, w = PK > 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (!wave_job2(wg, sh.batch * G, pair, chunk)) return;
+    const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), w = ONE ? 0 : wv;
+    if (ONE) {                                       // (independent waves: one past the group's last channel just leaves)
+        chunk = chunk * kOneWaves + wv;
+        if (chunk * PK >= rg) return;
+    }
     const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
     if (PK > 1) chunk = chunk * PK + lane / S;       // (a lane's own from here on)
     const bool act = PK == 1 || chunk < rg;          // a wave past the last channel of its group repeats it and stores nothing
     if (PK > 1) chunk = min(chunk, rg - 1);
-    const int b = pair / G, g = pair - b * G, c = g * rg + chunk;
+    int b, g;
+    wave_pair_split(wg, pair, G, b, g);
+    const int c = g * rg + chunk, cd = rd == 1 ? c : c / rd;   // channel of u, of delta
     // channel offsets: in the scalar base pointers, or (packed) in the lanes' offsets
     const int cB = PK > 1 ? 0 : c, chB = PK > 1 ? 0 : chunk, cL = PK > 1 ? c : 0, chL = PK > 1 ? chunk : 0;
     const int nseg = wg.nseg;
-    const bool multi = nseg > 1;
-    if (threadIdx.x < 2 * RD * NS) (&sHO[0][0][0][0])[(threadIdx.x / (RD * NS)) * (kMaxSeg + 1) * RD * NS + threadIdx.x % (RD * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool multi = !ONE && nseg > 1;
+    if (!ONE && threadIdx.x < 2 * RD * NS) (&sHO[0][0][0][0])[(threadIdx.x / (RD * NS)) * (kMaxSeg + 1) * RD * NS + threadIdx.x % (RD * NS)] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     // scan origin of this group: memory row = r0m + rs*i; with fh the columns run against the memory order
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
@@ -92,10 +100,10 @@ __global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_wave
 
     float A2[NS];
 #pragma unroll
-    for (int n = 0; n < NS; ++n) A2[n] = n < N ? p.A[(int64_t)c * p.A_d_stride + (int64_t)n * p.A_dstate_stride] * kLog2e : 0.f;
-    const float ld = p.A_decay ? __log2f(p.A_decay[0]) : 0.f;
+    for (int n = 0; n < NS; ++n) A2[n] = p.A[(int64_t)c * p.A_d_stride + (int64_t)n * p.A_dstate_stride];   // (NS == N; scaled below)
+    float ld = p.A_decay ? p.A_decay[0] : 1.f;
     const float Dv = p.D ? p.D[c] : 0.f;
-    const float bias = p.delta_bias ? p.delta_bias[c / rd] : 0.f;
+    const float bias = p.delta_bias ? p.delta_bias[cd] : 0.f;
     const bool softplus = p.delta_softplus != 0;
 
     constexpr int ESZ = (int)sizeof(T);
@@ -104,7 +112,7 @@ __global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_wave
     const T *Bb = (const T *)p.B + (int64_t)b * p.B_batch_stride + (int64_t)g * p.B_group_stride;
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
     const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chB : cB) * p.u_d_stride;
-    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(cB / rd) * p.delta_d_stride;
+    const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(PK > 1 ? 0 : cd) * p.delta_d_stride;
     // fused CrossMerge (fp32 out only): the channel adds weight * result to the feature channel it belongs to
     const bool merge = p.merge != 0;
     const float wm = merge && p.merge_weights ? p.merge_weights[c] : 1.f;
@@ -115,7 +123,7 @@ __global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_wave
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
     const uint32_t colB = (uint32_t)mc * ESZ;
     const uint32_t colU = colB + (uint32_t)(p.u_shared ? chL : cL) * (uint32_t)p.u_d_stride * ESZ,
-                   colD = colB + (uint32_t)(cL / rd) * (uint32_t)p.delta_d_stride * ESZ,
+                   colD = colB + (uint32_t)(PK > 1 ? cd : 0) * (uint32_t)p.delta_d_stride * ESZ,
                    colO = (uint32_t)mc * OSZ + (uint32_t)(merge ? chL : cL) * (uint32_t)p.out_d_stride * OSZ;
 
     // saved state of this plane set
@@ -313,7 +321,12 @@ __global__ __launch_bounds__(ONE ? 64 : 64 * kMaxSeg) __attribute__((amdgpu_wave
 
     Stage sA, sB;
     load_band(sA, 0);
-    lds_barrier();                                   // the zeroed slot
+    // the per-channel parameters are first used here, behind the first band's loads: a wave of a small plane lives
+    // for a few microseconds, and a wait for them in front of those loads would be a round trip of its own
+#pragma unroll
+    for (int n = 0; n < NS; ++n) A2[n] *= kLog2e;
+    ld = __log2f(ld);
+    if (!ONE) lds_barrier();                         // the zeroed slot
     if (multi)
         for (int e = 0; e < w; ++e) lds_barrier(); // the waves on the left go first
     if (OUT32 && merge) {
@@ -343,7 +356,8 @@ template <typename T, int NS, int CPL, bool VEC, int PK, int EU, bool ONE>
 static int launch_wave_fwd_o(const snd_fwd_params &p, const WaveGeo &wg, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int rg = sh.dim / sh.n_groups;
-    const dim3 grid(wave_grid(sh.batch * sh.n_groups, (rg + PK - 1) / PK)), block(64 * wg.nseg);
+    const int waves = (rg + PK - 1) / PK;            // per (batch, group) pair
+    const dim3 grid = wave_grid2(sh.batch * sh.n_groups, ONE ? (waves + kOneWaves - 1) / kOneWaves : waves), block(ONE ? 64 * kOneWaves : 64 * wg.nseg);
     const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
     constexpr bool F = std::is_same<T, float>::value;
     if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, CPL, VEC, true, true, PK, EU, ONE>), grid, block, 0, stream, p, wg);
@@ -379,7 +393,8 @@ template <typename T>
 int launch_wave_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int N = sh.dstate;
-    const WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
+    wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.out_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned(p.u, e, 2 * e, {p.u_batch_stride, p.u_d_stride, p.u_h_stride}) &&

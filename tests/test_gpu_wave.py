@@ -36,6 +36,11 @@ SHAPES = [
     # more blocks of 4 to 8 waves than fit at three waves per SIMD: the forward's instantiation with room for four
     (2, 192, 20, 300, 1, 4, None, torch.float32),
     (4, 256, 16, 256, 2, 4, None, torch.bfloat16),
+    # group counts that are no power of two (the pair -> (batch, group) split divides), with 18 and 30 pairs dealt to
+    # the XCDs and 3 pairs not; one-segment planes whose channels do not fill the forward's blocks of four waves
+    (6, 15, 9, 20, 1, 3, None, torch.float32),
+    (6, 30, 11, 70, 2, 5, 15, torch.bfloat16),
+    (1, 18, 6, 12, 1, 3, 9, torch.float32),
 ]
 
 
