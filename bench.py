@@ -142,52 +142,6 @@ def profile_counters(workload):
     return out
 
 
-def placement_probe(torch, dev, workload):
-    """Kernel time against where the second buffer of a pair lies (median of 9 launches each, everything else fixed):
-    x_sd at x + 2 MiB-rounded size + skew for the forward, dC at dB + 2 MiB-rounded size + skew for the backward,
-    both inside one allocation.  Results do not depend on placement; the time does (memory banks)."""
-    from selective_nd_scan import capi
-    Bt, Dm, H, W, N, K, dtn = WORKLOADS[workload]
-    u, delta, A, B, C, D, bias, dout = make_inputs(torch, Bt, Dm, H, W, N, K, getattr(torch, dtn), dev)
-    f = capi.FwdCall(u, delta, A, B, C, D, bias, True, True, None, True, 0)
-    f.launch()
-    b = capi.BwdCall(u, delta, A, B, C, D, bias, dout, f.x, f.x_v, True, None, f.x_sd, 0)
-    b.launch()
-
-    def median_ms(fn, n=9):
-        ts = []
-        for i in range(n + 3):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(); fn(); e1.record()
-            torch.cuda.synchronize()
-            if i >= 3:
-                ts.append(e0.elapsed_time(e1))
-        return round(sorted(ts)[len(ts) // 2], 4)
-
-    mib2 = 2 << 20
-    r2 = lambda v: (v + mib2 - 1) // mib2 * mib2
-    nx, nb = f.x.numel() * 4, b.dB.numel() * 4
-    pool = torch.zeros(2 * r2(nx) + 2 * r2(nb) + 4 * mib2, dtype=torch.uint8, device=dev)
-    base = r2(pool.data_ptr())
-    skews = [0, 256, 512, 1024, 2048, 3072, 4096, 5120, 16384, 17408, (1 << 20) + 1024]
-    keep = (f.params.x, f.params.x_sd, b.params.dB, b.params.dC)
-    fwd, bwd = {}, {}
-    for _ in range(20):                               # clocks settled before the first figure
-        f.launch(); b.launch_kernel_only()
-    for sk in skews:                                  # the forward writes x and x_sd; the backward only reads them
-        f.params.x, f.params.x_sd = base, base + r2(nx) + sk
-        fwd[sk] = median_ms(f.launch)
-    f.params.x, f.params.x_sd = keep[0], keep[1]
-    f.launch()
-    pb = base + 2 * r2(nx) + mib2
-    for sk in skews:
-        b.params.dB, b.params.dC = pb, pb + r2(nb) + sk
-        bwd[sk] = median_ms(b.launch_kernel_only)
-    b.params.dB, b.params.dC = keep[2], keep[3]
-    print(json.dumps({"placement_probe": workload, "skew_bytes": skews, "fwd_ms_by_x_sd_skew": fwd, "bwd_ms_by_dC_skew": bwd,
-                      "advice": {"dC_skew_bytes": f.plan.dC_skew_bytes}}))
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,16 +154,6 @@ def main():
     ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
                     help="kernel family and block mapping: chosen by shape (default), one block per plane chunk, "
                          "pipelined row strips / bands, or the row-segment wavefront kernels (1-4 states)")
-    ap.add_argument("--issue-probe", action="store_true",
-                    help="only time register-only instruction streams (library hook snd_debug_issue_probe) at 1-4 "
-                         "waves per SIMD on every CU and exit: the vector-ALU rate the roofline's second leg uses")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="only run a plain 256 MiB device copy a few times (scale reference for rocprofv3 "
-                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
-    ap.add_argument("--placement-probe", action="store_true",
-                    help="only time the backward against the distance between dB and dC (accumulated at equal offsets at "
-                         "the same time) and, for comparison, the forward against the distance between x and x_sd, for "
-                         "--workload, and exit: the measurement behind snd_plan.dC_skew_bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this operator is measured on ONE GPU (every (batch, channel, state) plane is an "
@@ -218,40 +162,6 @@ def main():
 
     import torch
     dev = torch.device("cuda:0")
-    if args.copy_probe:
-        x = torch.randn(64 * 1024 * 1024, device=dev)          # 256 MiB read + 256 MiB written per copy
-        y = torch.empty_like(x)
-        for _ in range(5):
-            y.copy_(x)
-        torch.cuda.synchronize()
-        print(json.dumps({"copy_probe_bytes_each_way": x.numel() * 4}))
-        return
-    if args.issue_probe:
-        from selective_nd_scan import capi
-        lib = capi.lib()
-        sink = torch.empty(256 * 1024, device=dev)
-        stream = torch.cuda.current_stream()
-        iters = 4000
-        kinds = ["v_fma_f32", "v_fma_f32 + s_nop 0", "v_exp_f32", "v_add_f32 (DPP operand)", "v_permlane32_swap_b32"]
-        res = {}
-        for kind, name in enumerate(kinds):
-            row = []
-            for wps in (1, 2, 3, 4):
-                capi.check(lib.snd_debug_issue_probe(kind, wps, 200, sink.data_ptr(), stream.cuda_stream))
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(stream)
-                capi.check(lib.snd_debug_issue_probe(kind, wps, iters, sink.data_ptr(), stream.cuda_stream))
-                e1.record(stream)
-                torch.cuda.synchronize()
-                # a SIMD hosts wps waves, each issuing iters x 64 probe instructions
-                row.append(round(e0.elapsed_time(e1) * 1e6 / (iters * 64.0 * wps), 3))
-            res[name] = row
-        print(json.dumps({"issue_probe_ns_per_instruction_per_simd": res, "waves_per_simd": [1, 2, 3, 4],
-                          "note": "256 blocks (one per CU); kind 1 counts only its v_fma_f32"}))
-        return
-    if args.placement_probe:
-        placement_probe(torch, dev, args.workload)
-        return
     import selective_nd_scan as snd
     from selective_nd_scan import capi
 

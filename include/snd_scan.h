@@ -88,7 +88,7 @@ typedef struct snd_plan {
      * 0.55-0.63 ms that way and 0.46-0.50 ms with dC half an fp32 row further on.  Put both in one allocation,
      * dC at dB + round_up(bytes of dB, 2 MiB) + dC_skew_bytes (a multiple of 256; the distance the advice was
      * measured at).  Results do not depend on placement, and no other pair of buffers shows the effect
-     * (`python bench.py --placement-probe`). */
+     * (timed with dC moved step by step inside one large allocation). */
     int64_t dC_skew_bytes;
 } snd_plan;
 
@@ -237,14 +237,6 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream);
  * With a limit of a few polls the time-out path above can be exercised from the host while every
  * kernel still runs to completion. */
 void snd_debug_set_spin_limit(int polls);
-
-/* Measurement hook (bench.py --issue-probe): launches, on every CU, blocks of `waves_per_simd` x 4 waves that
- * each issue `iters` x 64 register-only instructions of one kind on eight independent accumulators:
- * kind 0 v_fma_f32, 1 v_fma_f32 alternating with s_nop 0, 2 v_exp_f32, 3 v_add_f32 with a DPP operand,
- * 4 v_permlane32_swap_b32.  `sink` (>= 4 bytes per launched thread: 256 x waves_per_simd x 256 floats) takes
- * the accumulators.  The caller times the launch; the time per instruction and SIMD is what the vector-ALU
- * leg of the roofline is priced with.  No counterpart in the reference. */
-int snd_debug_issue_probe(int kind, int waves_per_simd, int iters, float *sink, snd_stream_t stream);
 
 /* snd_bwd for callers that cannot allocate device memory (code under HIP-graph capture, serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference, which allocates its scratch with

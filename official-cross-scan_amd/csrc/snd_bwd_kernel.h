@@ -26,6 +26,7 @@
 // As in the forward, tiles are computed in full on zero-padded staging (dout = B = C = 0 outside
 // the plane makes every adjoint there exactly zero), so the inner loops have no bounds checks.
 #pragma once
+#include <initializer_list>
 #include <type_traits>
 #include "snd_device.h"
 
@@ -60,8 +61,16 @@ __device__ __forceinline__ void rows_scatter4x2(float &b0, float &b1, float &b2,
 #ifndef SND_BWD_WAVES
 #define SND_BWD_WAVES 2
 #endif
-template <typename T, int NP, bool PIPE, int TE>
+#ifndef SND_KA8
+#define SND_KA8 2
+#endif
+// VEC: the tile's inputs are staged, and du / ddelta stored, four columns at a time with one 16-byte (fp32) or
+// 8-byte (16-bit) access per thread and tensor instead of one access per element - a quarter of the memory
+// instructions and of their address arithmetic.  Needs 8x8 tiles, a width that is a multiple of four and tensors
+// whose rows start on such boundaries (bwd_vec_ok); everything else takes the element-wise staging.
+template <typename T, int NP, bool PIPE, int TE, bool VEC>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD_WAVES, SND_BWD_WAVES))) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
+    static_assert(!VEC || TE == 8, "vector staging needs 8x8 tiles");
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;
@@ -76,8 +85,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     constexpr int NSD = NP == 16 ? kTile + 2 : kTile + 4;
     constexpr int NBC = 4;
     constexpr int NPX = kTile / NP;
-    constexpr int HG = 10, DLP = HG * HG;           // delta' on the tile plus a one-cell halo
+    // delta' on the tile plus a one-cell halo: rows -1..8 at a pitch of 12 floats, column j at element DLO + j, so
+    // that columns 0-3 and 4-7 of a row are each one aligned 16-byte read (channels of a wave 24 banks apart)
+    constexpr int HG = 12, DLO = 4, DLP = 10 * HG;
     constexpr int NHALO = 4 * TE + 4, NHK = (NHALO + NP - 1) / NP;   // ring around the TE x TE tile
+    constexpr int NCH = VEC ? kTile / 4 / NP : 0;   // (VEC) four-column chunks of a channel's tile per thread
+    constexpr int NHV = (24 + NP - 1) / NP;         // (VEC) halo cells per thread: row above, row below, column to the left
 
     // A wave's channels (four with 16 states per channel, eight with 8) are reduced in registers and
     // every wave owns a partial dB/dC tile, written with plain stores.
@@ -204,12 +217,57 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const int qrow = (tid & 63) >> 4;               // 16-lane row of this lane inside its wave
 
     // ---- register staging of one tile's raw inputs (loaded at the start of the tile, then committed to LDS)
-    float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qdo[NPX], qh[NHK];
+    float qb[VEC ? 1 : NBC], qc[VEC ? 1 : NBC], qdl[VEC ? 1 : NPX], qu[VEC ? 1 : NPX], qdo[VEC ? 1 : NPX], qh[VEC ? 1 : NHK];
+    Raw4<T> vb, vc, vdl[VEC ? NCH : 1], vu[VEC ? NCH : 1];     // (VEC) one chunk of B and C, NCH chunks of delta, u, dout
+    uint32_t vdo[VEC ? NCH : 1][4];
+    uint32_t vh[VEC ? NHV : 1];
+    // (VEC) halo cell k of this thread: cells 0-7 the row above, 8-15 the row below, 16-23 the column to the left
+    auto halo_cell = [&](int hidx, int &rr, int &jj) {
+        if (hidx < 8) { rr = -1; jj = hidx; }
+        else if (hidx < 16) { rr = TE; jj = hidx - 8; }
+        else { rr = hidx - 16; jj = -1; }
+    };
     auto prefetch = [&](int I, int J) {
         const int r0 = (SND_TILE_ABLATE & 2) ? 0 : I * TE, j0 = (SND_TILE_ABLATE & 2) ? 0 : J * TE;
         // The thread's element maps are re-derived here from an opaque copy of the thread id, so that
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
+        if constexpr (VEC) {
+            // loads are always in bounds (clamped coordinates); commit() zeroes what lies outside the plane.
+            // Chunk q of a tile = row q / 2, columns 4 * (q % 2) .. + 3; under a mirrored column order the same four
+            // memory columns in reverse (the chunk then starts at the memory column of its last scan column).
+            auto chunk_off = [&](int q, int hB, int esz) {
+                const int row = min(r0 + (q >> 1), H - 1), col = min(j0 + (q & 1) * 4, W - 4);
+                return (uint32_t)mad24(mrow(row), hB, mcol(col + (fh ? 3 : 0)) * esz);
+            };
+            {
+                const int sn = min(t_ >> 4, N - 1), q = t_ & 15;
+                ldraw4_b(vb, (const T *)((const char *)Bb + sn * BsB), chunk_off(q, BhB, ESZ));
+                ldraw4_b(vc, (const T *)((const char *)Cb + sn * CsB), chunk_off(q, ChB, ESZ));
+            }
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                const int q = n + NP * k;
+                ldraw4_b(vdl[k], db, cDb + chunk_off(q, DhB, ESZ));
+                ldraw4_b(vu[k], ub, cUb + chunk_off(q, UhB, ESZ));
+                const char *src = (const char *)dob + (cDob + chunk_off(q, DohB, esz_do));
+                if (sizeof(T) == 4 || sh_do == 2) {
+                    const uint4 v = *(const uint4 *)src;
+                    vdo[k][0] = v.x; vdo[k][1] = v.y; vdo[k][2] = v.z; vdo[k][3] = v.w;
+                } else {
+                    const uint2 v = *(const uint2 *)src;
+                    vdo[k][0] = v.x; vdo[k][1] = v.y;
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < NHV; ++k) {
+                int rr, jj;
+                halo_cell(n + NP * k, rr, jj);
+                const int row = min(max(r0 + rr, 0), H - 1), col = min(max(j0 + jj, 0), W - 1);
+                vh[k] = ldraw_b(db, cDb + mad24(mrow(row), DhB, mcol(col) * ESZ));
+            }
+            return;
+        }
         // loads are always in bounds (clamped coordinates); values outside the plane become zero
         {
             const int row = r0 + pr, col = j0 + pj;
@@ -219,10 +277,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
                 const int sn = wave_u + WPB * k, sc = min(sn, N - 1);       // scalar: folded into the base
-                const float vb = ldg_b((const T *)((const char *)Bb + sc * BsB), ob);
-                const float vc = ldg_b((const T *)((const char *)Cb + sc * CsB), oc);
-                qb[k] = (in && sn < N) ? vb : 0.f;
-                qc[k] = (in && sn < N) ? vc : 0.f;
+                const float vb_ = ldg_b((const T *)((const char *)Bb + sc * BsB), ob);
+                const float vc_ = ldg_b((const T *)((const char *)Cb + sc * CsB), oc);
+                qb[k] = (in && sn < N) ? vb_ : 0.f;
+                qc[k] = (in && sn < N) ? vc_ : 0.f;
             }
         }
 #pragma unroll
@@ -231,10 +289,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
             const bool ok = cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W;
             const int mr = mrow(min(row, H - 1)), mc = mcol(min(col, W - 1));
-            const float vd = ldg_b(db, cDb + mad24(mr, DhB, mc * ESZ)), vu = ldg_b(ub, cUb + mad24(mr, UhB, mc * ESZ));
+            const float vd = ldg_b(db, cDb + mad24(mr, DhB, mc * ESZ)), vu_ = ldg_b(ub, cUb + mad24(mr, UhB, mc * ESZ));
             const float vo = ld_f32_b(dob, cDob + mad24(mr, DohB, mc << sh_do), p.dout_dtype);
             qdl[k] = ok ? vd : 0.f;
-            qu[k] = ok ? vu : 0.f;
+            qu[k] = ok ? vu_ : 0.f;
             qdo[k] = ok ? vo : 0.f;
         }
 #pragma unroll
@@ -251,8 +309,67 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             qh[k] = ok ? vd : 0.f;
         }
     };
-    auto commit = [&]() {
+    auto commit = [&](int I, int J) {
         SND_THREAD_MAPS(NP);
+        if constexpr (VEC) {
+            const int r0 = I * TE, j0 = J * TE;
+            auto flip4 = [&](float (&v)[4]) {                     // memory order -> scan order under a mirrored column order
+                if (fh) { const float a0 = v[0], a1 = v[1]; v[0] = v[3]; v[1] = v[2]; v[2] = a1; v[3] = a0; }
+            };
+            {
+                const int sn = t_ >> 4, q = t_ & 15;
+                const bool ok = sn < N && r0 + (q >> 1) < H && j0 + (q & 1) * 4 < W;
+                float b4[4], c4[4];
+                raw4_to_f32(vb, b4); raw4_to_f32(vc, c4);
+                flip4(b4); flip4(c4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { b4[e] = ok ? b4[e] : 0.f; c4[e] = ok ? c4[e] : 0.f; }
+                *(float4 *)(sB + sn * NSTR + q * 4) = make_float4(b4[0], b4[1], b4[2], b4[3]);
+                *(float4 *)(sC + sn * NSTR + q * 4) = make_float4(c4[0], c4[1], c4[2], c4[3]);
+            }
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                const int q = n + NP * k;
+                const bool ok = cvalid && r0 + (q >> 1) < H && j0 + (q & 1) * 4 < W;
+                float d4[4], u4[4], o4[4], dl4[4], du4[4], sg4[4];
+                raw4_to_f32(vdl[k], d4); raw4_to_f32(vu[k], u4);
+                if (sizeof(T) == 4 || sh_do == 2) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o4[e] = __builtin_bit_cast(float, vdo[k][e]);
+                } else {
+                    Raw4<T> t4;
+                    t4.w[0] = vdo[k][0]; t4.w[sizeof(T) == 4 ? 0 : 1] = vdo[k][1];
+                    raw4_to_f32(t4, o4);
+                }
+                flip4(d4); flip4(u4); flip4(o4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float raw = (ok ? d4[e] : 0.f) + bias;
+                    float dsp = 1.f;
+                    dl4[e] = softplus ? softplus20(raw, dsp) : raw;
+                    u4[e] = ok ? u4[e] : 0.f;
+                    du4[e] = dl4[e] * u4[e];
+                    o4[e] = ok ? wm * o4[e] : 0.f;
+                    sg4[e] = dsp;
+                }
+                *(float4 *)(sDl + cl * DLP + ((q >> 1) + 1) * HG + DLO + (q & 1) * 4) = make_float4(dl4[0], dl4[1], dl4[2], dl4[3]);
+                *(float4 *)(sDu + cl * PCH + q * 4) = make_float4(du4[0], du4[1], du4[2], du4[3]);
+                *(float4 *)(sU + cl * PCS + q * 4) = make_float4(u4[0], u4[1], u4[2], u4[3]);
+                *(float4 *)(sDo + cl * PCH + q * 4) = make_float4(o4[0], o4[1], o4[2], o4[3]);
+                *(float4 *)(sSg + cl * PCS + q * 4) = make_float4(sg4[0], sg4[1], sg4[2], sg4[3]);
+            }
+#pragma unroll
+            for (int k = 0; k < NHV; ++k) {
+                const int hidx = n + NP * k;
+                int rr, jj;
+                halo_cell(hidx, rr, jj);
+                const bool ok = cvalid && r0 + rr >= 0 && r0 + rr < H && j0 + jj >= 0 && j0 + jj < W;
+                const float raw = (ok ? raw_to_f32((const T *)nullptr, vh[k]) : 0.f) + bias;
+                float dsp;
+                if (hidx < 24) sDl[cl * DLP + (rr + 1) * HG + DLO + jj] = softplus ? softplus20(raw, dsp) : raw;
+            }
+            return;
+        }
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
             const int sn = wave + WPB * k;
@@ -266,7 +383,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             float dsp = 1.f;
             const float dl = softplus ? softplus20(raw, dsp) : raw;
             if (TE == 8 || ((pp >> 3) < TE && (pp & 7) < TE))     // slots beyond the tile belong to the halo ring
-                sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1] = dl;
+                sDl[cl * DLP + ((pp >> 3) + 1) * HG + DLO + (pp & 7)] = dl;
             sDu[cl * PCH + pp] = dl * qu[k];
             sU[cl * PCS + pp] = qu[k];
             sDo[cl * PCH + pp] = wm * qdo[k];
@@ -282,11 +399,18 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             else { rr = hidx - (3 * TE + 3); jj = TE + 1; }
             const float raw = qh[k] + bias;
             float dsp;
-            if (hidx < NHALO) sDl[cl * DLP + rr * HG + jj] = softplus ? softplus20(raw, dsp) : raw;
+            if (hidx < NHALO && DLO - 1 + jj < HG)      // (the column right of an 8-column tile is never read)
+                sDl[cl * DLP + rr * HG + DLO - 1 + jj] = softplus ? softplus20(raw, dsp) : raw;
         }
     };
-#define DL(r, j) myDl[((r) + 1) * HG + (j) + 1]
-#define AEXP(r, j) fast_exp2(fmaf(DL(r, j), A2, ld))
+#define DL(r, j) myDl[((r) + 1) * HG + DLO + (j)]
+#define AEXP(r, j) EXPA(DL(r, j))
+    // delta' of columns c0 .. c0+3 (c0 = 0 or 4) of tile row r (-1 .. 8): one aligned 16-byte read
+    auto dl_row4 = [&](int r, int c0, float (&o)[4]) __attribute__((always_inline)) {
+        const float4 v = *(const float4 *)(myDl + (r + 1) * HG + DLO + c0);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    };
+#define EXPA(x) fast_exp2(fmaf((x), A2, ld))
 
     float dA_acc = 0.f, dec_acc = 0.f;              // per lane: sum delta'*da*a, sum da*a
     const bool want_decay = p.dA_decay != nullptr;  // the second sum is skipped when nobody reads it
@@ -382,7 +506,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
             }
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
-            commit();
+            commit(I, J);
             if (pI >= 0) flush_bc(pI, pJ);          // the previous tile's dB, dC
             pI = I; pJ = J;
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
@@ -415,17 +539,19 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // swept: 32 extra cell updates per tile buy about 60 registers).
             float hmid[kRows] = {}, smid[kRows] = {}, amid[kRows] = {};   // h, s, a at column 3
             {
-                float aprev[4], hprev[4];
+                float aprev[4], hprev[4], dlr[4];
+                dl_row4(-1, 0, dlr);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) { aprev[j] = AEXP(-1, j); hprev[j] = hu[j]; }
+                for (int j = 0; j < 4; ++j) { aprev[j] = EXPA(dlr[j]); hprev[j] = hu[j]; }
                 float diag0 = hc;
 #pragma unroll
                 for (int r = 0; r < TE; ++r) {
                     float al = AEXP(r, -1), left = hlft[r], sl = slft[r], diag = diag0;
                     diag0 = hlft[r];
+                    dl_row4(r, 0, dlr);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float a = AEXP(r, j);
+                        const float a = EXPA(dlr[j]);
                         const float bu = myB[r * kCkX + j] * myDu[r * kCkX + j];
                         const float up = hprev[j];
                         const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
@@ -449,20 +575,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 float hT[kRows][4];
                 // the left half keeps a of its first KA columns from this pass for the sweep (as many as
                 // fit under 256 registers without spilling); everything else is recomputed there
-                constexpr int KA = C0 == 0 ? (TE == 7 ? 4 : 2) : 0;
+                constexpr int KA = C0 == 0 ? (TE == 7 ? 4 : SND_KA8) : 0;
                 float aT[KA ? kRows : 1][KA ? KA : 1];
                 {
-                    float aprev[4], hprev[4];
+                    float aprev[4], hprev[4], dlr[4];
+                    dl_row4(-1, C0, dlr);
 #pragma unroll
-                    for (int j = 0; j < HW; ++j) { aprev[j] = AEXP(-1, C0 + j); hprev[j] = top[j]; }
+                    for (int j = 0; j < HW; ++j) { aprev[j] = EXPA(dlr[j]); hprev[j] = top[j]; }
                     float diag0 = corner;
 #pragma unroll
                     for (int r = 0; r < TE; ++r) {
                         float al = C0 == 0 ? AEXP(r, C0 - 1) : amid[r], left = hL[r], diag = diag0;
                         diag0 = hL[r];
+                        dl_row4(r, C0, dlr);
 #pragma unroll
                         for (int j = 0; j < HW; ++j) {
-                            const float a = AEXP(r, C0 + j);
+                            const float a = EXPA(dlr[j]);
                             const float bu = myB[r * kCkX + C0 + j] * myDu[r * kCkX + C0 + j];
                             const float up = hprev[j];
                             const float X = fmaf(-0.5f * (aprev[j] + al), diag, up);
@@ -476,19 +604,36 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
                 float adn[4];
                 float Gd8 = gdiag0;
+                {
+                    float dlr[4];
+                    dl_row4(TE, C0, dlr);
 #pragma unroll
-                for (int j = 0; j < HW; ++j) adn[j] = AEXP(TE, C0 + j);
+                    for (int j = 0; j < HW; ++j) adn[j] = EXPA(dlr[j]);
+                }
+                // The five LDS operands of a row (delta', B, C, delta'*u, dout; 16 bytes each) are requested one row ahead.
+                // With 7x7 tiles, 16 states and whole-plane blocks the request sits behind the row's cell updates and in front of its
+                // cross-lane sums (the registers of the row just finished are free there, and the reads complete under
+                // the sums: 64 x 768 channels of 14x14, bf16, 0.347 -> 0.336 ms); every other variant has no register
+                // left for that (12 to 16 spilled, nothing gained) and requests the next row behind the sums.
+                constexpr bool ROWPF = TE == 7 && NP == 16 && !PIPE;
+                float4 nD4, nB4, nC4, nU4, nO4;
+                auto request_row = [&](int r) __attribute__((always_inline)) {
+                    nD4 = *(const float4 *)(myDl + (r + 1) * HG + DLO + C0);
+                    nB4 = *(const float4 *)(myB + r * kCkX + C0);
+                    nU4 = *(const float4 *)(myDu + r * kCkX + C0);
+                    nC4 = *(const float4 *)(myC + r * kCkX + C0); nO4 = *(const float4 *)(myDo + r * kCkX + C0);
+                };
+                request_row(TE - 1);
 #pragma unroll
                 for (int r = TE - 1; r >= 0; --r) {
                     __builtin_amdgcn_sched_barrier(0);
                     float arow[5], s[4], buv[4];
+                    const float dlr[4] = {nD4.x, nD4.y, nD4.z, nD4.w};
 #pragma unroll
-                    for (int j = 0; j < HW; ++j) arow[j] = j < KA ? aT[KA ? r : 0][j < KA ? j : 0] : AEXP(r, C0 + j);
+                    for (int j = 0; j < HW; ++j) arow[j] = j < KA ? aT[KA ? r : 0][j < KA ? j : 0] : EXPA(dlr[j]);
                     arow[HW] = aR[r];
-                    const float4 vB4 = *(const float4 *)(myB + r * kCkX + C0), vC4 = *(const float4 *)(myC + r * kCkX + C0);
-                    const float4 vU4 = *(const float4 *)(myDu + r * kCkX + C0), vO4 = *(const float4 *)(myDo + r * kCkX + C0);
-                    const float aB[4] = {vB4.x, vB4.y, vB4.z, vB4.w}, aC[4] = {vC4.x, vC4.y, vC4.z, vC4.w};
-                    const float aU[4] = {vU4.x, vU4.y, vU4.z, vU4.w}, aO[4] = {vO4.x, vO4.y, vO4.z, vO4.w};
+                    const float aB[4] = {nB4.x, nB4.y, nB4.z, nB4.w}, aC[4] = {nC4.x, nC4.y, nC4.z, nC4.w};
+                    const float aU[4] = {nU4.x, nU4.y, nU4.z, nU4.w}, aO[4] = {nO4.x, nO4.y, nO4.z, nO4.w};
                     {
                         float sp = sL[r];
 #pragma unroll
@@ -517,7 +662,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         const float hs = hT[r][j] - s[j], sb = s[j] - bu;
                         const float cross = fmaf(GdH[j], h_l, Gr * h_u);
                         const float da = fmaf(-0.5f * a, cross, fmaf(g_, hs, (g_ + gs) * sb));
-                        dA_acc = fmaf(DL(r, C0 + j), da, dA_acc);
+                        dA_acc = fmaf(dlr[j], da, dA_acc);
                         dsum[j] = da;
                         const float Gn = a * g_;
                         Gdiag = GdH[j];
@@ -529,7 +674,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                         vB[j] = dbu * duv;                         // dB, dC contributions
                         vC[j] = dov * fmaf(0.25f, bu, hs);
                     }
+                    // The two running sums are pinned to their row: left to itself the compiler sinks the whole chain of
+                    // multiply-adds to the end of the tile and keeps delta' and da of all 64 cells in registers until then.
                     if (want_decay) dec_acc += (dsum[0] + dsum[1]) + (dsum[2] + dsum[3]);
+                    if (ROWPF) {
+                        if (r > 0) request_row(r - 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     if (NP == 16) {
                         // sums over the channel's 16 states: quads 0,1 of the lane group end with
                         // q[0..1], q[2..3], quads 2,3 with pp_[0..1], pp_[2..3]
@@ -558,6 +709,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                             mydC[r * kCkX + C0 + qrow] = tc;
                         }
                     }
+                    if (!ROWPF && r > 0) request_row(r - 1);
                     Gd8 = GR[r];                    // G[r][C0+4]: diagonal neighbour for the row above
                     GR[r] = Gr;                     // G[r][C0]: right neighbour for the half on the left
                     GsR[r] = Gsr;
@@ -588,12 +740,51 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // ---- once per pixel: du, ddelta (thread that staged the pixel), dD, ddelta_bias
             {
             SND_THREAD_MAPS(NP);
+            if constexpr (VEC) {
+#pragma unroll
+                for (int k = 0; k < NCH; ++k) {
+                    const int q = n + NP * k;
+                    const int row = r0 + (q >> 1), col = j0 + (q & 1) * 4;
+                    const float4 q4 = *(const float4 *)(sQ + cl * PCH + q * 4), p4 = *(const float4 *)(sP + cl * PCH + q * 4);
+                    const float4 l4 = *(const float4 *)(sDl + cl * DLP + ((q >> 1) + 1) * HG + DLO + (q & 1) * 4);
+                    const float4 u4 = *(const float4 *)(sU + cl * PCS + q * 4), o4 = *(const float4 *)(sDo + cl * PCH + q * 4);
+                    const float4 g4 = *(const float4 *)(sSg + cl * PCS + q * 4);
+                    const float aq[4] = {q4.x, q4.y, q4.z, q4.w}, ap[4] = {p4.x, p4.y, p4.z, p4.w}, al[4] = {l4.x, l4.y, l4.z, l4.w};
+                    const float au[4] = {u4.x, u4.y, u4.z, u4.w}, ao[4] = {o4.x, o4.y, o4.z, o4.w}, ag[4] = {g4.x, g4.y, g4.z, g4.w};
+                    float duv[4], ddl[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        duv[e] = fmaf(Dv, ao[e], al[e] * aq[e]);
+                        ddl[e] = fmaf(au[e], aq[e], ap[e]) * ag[e];
+                    }
+                    if (cvalid && row < H && col < W) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            dD_acc = fmaf(ao[e], au[e], dD_acc);
+                            dw_acc = fmaf(duv[e], au[e], dw_acc);
+                            dbias_acc += ddl[e];
+                        }
+                        if (fh) {                   // scan order -> memory order
+                            const float a0 = duv[0], a1 = duv[1], b0 = ddl[0], b1 = ddl[1];
+                            duv[0] = duv[3]; duv[1] = duv[2]; duv[2] = a1; duv[3] = a0;
+                            ddl[0] = ddl[3]; ddl[1] = ddl[2]; ddl[2] = b1; ddl[3] = b0;
+                        }
+                        const uint32_t o = cGb + mad24(mrow(row), WB, mcol(col + (fh ? 3 : 0)) * ESZ);
+                        if (!(SND_TILE_ABLATE & 4)) {
+                            stg4_b(dub, o, duv);
+                            stg4_b(ddb, o, ddl);
+                        } else {
+                            dD_acc += duv[0] + ddl[0];  // keeps the values live
+                        }
+                    }
+                }
+            } else {
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                 const float qv = sQ[cl * PCH + pp], pv = sP[cl * PCH + pp];
-                const float dl = sDl[cl * DLP + ((pp >> 3) + 1) * HG + (pp & 7) + 1];
+                const float dl = sDl[cl * DLP + ((pp >> 3) + 1) * HG + DLO + (pp & 7)];
                 const float uv = sU[cl * PCS + pp], dov = sDo[cl * PCH + pp], sg = sSg[cl * PCS + pp];
                 const float duv = fmaf(Dv, dov, dl * qv);
                 const float ddl = fmaf(uv, qv, pv) * sg;
@@ -611,11 +802,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
             }
             }
+            }
         }
     }
     if (pI >= 0) flush_bc(pI, pJ);
 #undef DL
 #undef AEXP
+#undef EXPA
 
 #ifdef SND_PIPE_TRACE
     if (PIPE && threadIdx.x == 0) { trace_[1] = (int)wall_clock64(); trace_[2] = trace_wait_; }
@@ -650,23 +843,50 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 // Dynamic LDS of one backward block (more than the 64 KB a kernel gets without asking).
 template <int NP> constexpr size_t bwd_lds_bytes() {
     constexpr int PCH = kTile + (NP == 16 ? 8 : 4), PCS = kTile + NP, NSD = NP == 16 ? kTile + 2 : kTile + 4;
-    return sizeof(float) * (2 * NP * (kTile + 4) + 2 * (NP / 4) * NP * NSD + 16 * 100 + 16 * (4 * PCH + 2 * PCS) + 4 + NP / 4);
+    return sizeof(float) * (2 * NP * (kTile + 4) + 2 * (NP / 4) * NP * NSD + 16 * 120 + 16 * (4 * PCH + 2 * PCS) + 4 + NP / 4);
 }
 // Raise the dynamic LDS limit of every backward instantiation of one input dtype on the current device.
 // hipFuncSetAttribute is not stream-ordered and must not run under a stream capture, which is why it is
 // done once per device at set-up and not inside the launch path.
-template <typename T, int NP, int TE> static bool configure_bwd_one() {
+template <typename T, int NP, int TE, bool VEC> static bool configure_bwd_one() {
     const int lds = (int)bwd_lds_bytes<NP>();
-    return hipFuncSetAttribute((const void *)bwd_kernel<T, NP, true, TE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
-           hipFuncSetAttribute((const void *)bwd_kernel<T, NP, false, TE>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
+    return hipFuncSetAttribute((const void *)bwd_kernel<T, NP, true, TE, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
+           hipFuncSetAttribute((const void *)bwd_kernel<T, NP, false, TE, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
 }
 template <typename T> int configure_bwd_t() {
-    const bool ok = configure_bwd_one<T, 16, 8>() && configure_bwd_one<T, 16, 7>() && configure_bwd_one<T, 8, 8>() &&
-                    configure_bwd_one<T, 8, 7>() && configure_bwd_one<T, 4, 8>() && configure_bwd_one<T, 4, 7>();
+    const bool ok = configure_bwd_one<T, 16, 8, false>() && configure_bwd_one<T, 16, 7, false>() && configure_bwd_one<T, 8, 8, false>() &&
+                    configure_bwd_one<T, 8, 7, false>() && configure_bwd_one<T, 4, 8, false>() && configure_bwd_one<T, 4, 7, false>() &&
+                    configure_bwd_one<T, 16, 8, true>() && configure_bwd_one<T, 8, 8, true>() && configure_bwd_one<T, 4, 8, true>();
     return ok ? SND_OK : SND_ERR_LAUNCH;
 }
 
-template <typename T, int NP, int TE>
+// Whether a call can stage four columns per access (bwd_kernel's VEC): every row of every tensor the staging touches
+// must start on a four-element boundary (16 bytes of fp32, 8 bytes of 16-bit values), and so must the rows of the dense
+// du / ddelta; a state's plane of B / C must lie within 2^31 bytes of the first (the state offset is per lane there).
+inline bool vec4_ok(const void *ptr, int esz, std::initializer_list<int64_t> strides) {
+    if (((uintptr_t)ptr & (uintptr_t)(4 * esz - 1)) != 0) return false;
+    for (int64_t s : strides)
+        if (s % 4 != 0) return false;
+    return true;
+}
+inline bool bwd_vec_ok(const snd_bwd_params &p) {
+    const snd_fwd_params &f = p.f;
+    const snd_shape &sh = f.shape;
+    const int e = sh.in_dtype == SND_F32 ? 4 : 2, eo = p.dout_dtype == SND_F32 ? 4 : 2;
+    if (sh.ncols % 4 != 0) return false;
+    const int64_t span = (int64_t)(sh.dstate - 1) * e;
+    if (span * f.B_dstate_stride + (int64_t)sh.nrows * f.B_h_stride * e >= ((int64_t)1 << 31) ||
+        span * f.C_dstate_stride + (int64_t)sh.nrows * f.C_h_stride * e >= ((int64_t)1 << 31))
+        return false;
+    return vec4_ok(f.u, e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&
+           vec4_ok(f.delta, e, {f.delta_batch_stride, f.delta_d_stride, f.delta_h_stride}) &&
+           vec4_ok(f.B, e, {f.B_batch_stride, f.B_group_stride, f.B_dstate_stride, f.B_h_stride}) &&
+           vec4_ok(f.C, e, {f.C_batch_stride, f.C_group_stride, f.C_dstate_stride, f.C_h_stride}) &&
+           vec4_ok(p.dout, eo, {p.dout_batch_stride, p.dout_d_stride, p.dout_h_stride}) &&
+           vec4_ok(p.du, e, {}) && vec4_ok(p.ddelta, e, {});
+}
+
+template <typename T, int NP, int TE, bool VEC>
 static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t stream) {
     const snd_shape &sh = p.f.shape;
     const int rg = sh.dim / sh.n_groups;
@@ -684,10 +904,10 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
         gb.spinLimit = spin_limit();
         gb.nBands = bands;
         gb.nQueues = job_queues(sh.batch * sh.n_groups);
-        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE, VEC>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
-        hipLaunchKernelGGL((bwd_kernel<T, NP, false, TE>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
+        hipLaunchKernelGGL((bwd_kernel<T, NP, false, TE, VEC>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
@@ -695,7 +915,8 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
 template <typename T, int NP>
 static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
     const Geo geo = make_geo(p.f.shape.nrows, p.f.shape.ncols);
-    return geo.te == 7 ? launch_bwd_te<T, NP, 7>(p, geo, stream) : launch_bwd_te<T, NP, 8>(p, geo, stream);
+    if (geo.te == 7) return launch_bwd_te<T, NP, 7, false>(p, geo, stream);
+    return bwd_vec_ok(p) ? launch_bwd_te<T, NP, 8, true>(p, geo, stream) : launch_bwd_te<T, NP, 8, false>(p, geo, stream);
 }
 
 // One instantiation per input dtype, each in its own translation unit.

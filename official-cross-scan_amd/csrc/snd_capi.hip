@@ -35,37 +35,6 @@ __global__ void zero_words_kernel(int *p, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0;
 }
-// Issue-rate probe (snd_debug_issue_probe): 64 register-only instructions of one kind per loop pass, on eight
-// independent accumulators so that no instruction waits for the one before it.
-#define SND_P8(op, tail)                                                                                          \
-    op " %0, %0" tail "\n\t" op " %1, %1" tail "\n\t" op " %2, %2" tail "\n\t" op " %3, %3" tail "\n\t"            \
-    op " %4, %4" tail "\n\t" op " %5, %5" tail "\n\t" op " %6, %6" tail "\n\t" op " %7, %7" tail "\n\t"
-#define SND_PROBE(text) asm volatile(text : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3), "+v"(x4), "+v"(x5), "+v"(x6), "+v"(x7) : "v"(a), "v"(b))
-template <int KIND> __global__ void issue_probe_kernel(float *sink, int iters) {
-    float x0 = threadIdx.x * 1e-3f, x1 = x0 + 1.f, x2 = x0 + 2.f, x3 = x0 + 3.f, x4 = x0 + 4.f, x5 = x0 + 5.f, x6 = x0 + 6.f, x7 = x0 + 7.f;
-    const float a = 0.999f, b = 1e-3f;
-    for (int i = 0; i < iters; ++i) {
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (KIND == 0) SND_PROBE(SND_P8("v_fma_f32", ", %8, %9"));
-            if (KIND == 1)
-                SND_PROBE("v_fma_f32 %0, %0, %8, %9\n\ts_nop 0\n\tv_fma_f32 %1, %1, %8, %9\n\ts_nop 0\n\t"
-                          "v_fma_f32 %2, %2, %8, %9\n\ts_nop 0\n\tv_fma_f32 %3, %3, %8, %9\n\ts_nop 0\n\t"
-                          "v_fma_f32 %4, %4, %8, %9\n\ts_nop 0\n\tv_fma_f32 %5, %5, %8, %9\n\ts_nop 0\n\t"
-                          "v_fma_f32 %6, %6, %8, %9\n\ts_nop 0\n\tv_fma_f32 %7, %7, %8, %9\n\ts_nop 0\n\t");
-            if (KIND == 2) SND_PROBE(SND_P8("v_exp_f32_e32", ""));
-            if (KIND == 3) SND_PROBE(SND_P8("v_add_f32_dpp", ", %8 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"));
-            if (KIND == 4)
-                SND_PROBE("v_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\tv_permlane32_swap_b32 %4, %5\n\t"
-                          "v_permlane32_swap_b32 %6, %7\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\t"
-                          "v_permlane32_swap_b32 %4, %5\n\tv_permlane32_swap_b32 %6, %7\n\t");
-        }
-    }
-    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = ((x0 + x1) + (x2 + x3)) + ((x4 + x5) + (x6 + x7));
-}
-#undef SND_PROBE
-#undef SND_P8
-
 int zero_words(int *p, int64_t n, hipStream_t stream) {
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
@@ -371,20 +340,6 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream) {
         return SND_ERR_LAUNCH;
     if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return SND_ERR_LAUNCH;
     return word != 0 ? SND_ERR_PIPELINE : SND_OK;
-}
-
-int snd_debug_issue_probe(int kind, int waves_per_simd, int iters, float *sink, snd_stream_t stream) {
-    if (!sink) return SND_ERR_NULL;
-    if (kind < 0 || kind > 4 || waves_per_simd < 1 || waves_per_simd > 4 || iters < 1) return SND_ERR_SHAPE;
-    const dim3 grid(256), block(256 * waves_per_simd);
-    switch (kind) {
-    case 0: hipLaunchKernelGGL(snd::issue_probe_kernel<0>, grid, block, 0, (hipStream_t)stream, sink, iters); break;
-    case 1: hipLaunchKernelGGL(snd::issue_probe_kernel<1>, grid, block, 0, (hipStream_t)stream, sink, iters); break;
-    case 2: hipLaunchKernelGGL(snd::issue_probe_kernel<2>, grid, block, 0, (hipStream_t)stream, sink, iters); break;
-    case 3: hipLaunchKernelGGL(snd::issue_probe_kernel<3>, grid, block, 0, (hipStream_t)stream, sink, iters); break;
-    default: hipLaunchKernelGGL(snd::issue_probe_kernel<4>, grid, block, 0, (hipStream_t)stream, sink, iters); break;
-    }
-    return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
 }
 
 void snd_debug_set_spin_limit(int polls) { snd::g_spin_limit.store(polls > 0 ? polls : snd::kSpinLimit, std::memory_order_relaxed); }

@@ -74,6 +74,45 @@ __device__ __forceinline__ uint32_t ldraw_b(const f16_t *base, uint32_t off) { r
 __device__ __forceinline__ float raw_to_f32(const float *, uint32_t r) { return __builtin_bit_cast(float, r); }
 __device__ __forceinline__ float raw_to_f32(const bf16_t *, uint32_t r) { return __builtin_bit_cast(float, r << 16); }
 __device__ __forceinline__ float raw_to_f32(const f16_t *, uint32_t r) { return (float)__builtin_bit_cast(f16_t, (uint16_t)r); }
+// Four consecutive elements with one vector access (16 bytes of fp32, 8 bytes of 16-bit values), kept as raw bits
+// until they are needed.  The address must be aligned to the access (the launchers check the tensors for it).
+template <typename T> struct Raw4 { uint32_t w[sizeof(T)]; };           // 4 words, or 2 words of two 16-bit values each
+__device__ __forceinline__ void ldraw4_b(Raw4<float> &q, const float *base, uint32_t off) {
+    const uint4 v = *(const uint4 *)((const char *)base + off);
+    q.w[0] = v.x; q.w[1] = v.y; q.w[2] = v.z; q.w[3] = v.w;
+}
+__device__ __forceinline__ void ldraw4_b(Raw4<bf16_t> &q, const bf16_t *base, uint32_t off) {
+    const uint2 v = *(const uint2 *)((const char *)base + off);
+    q.w[0] = v.x; q.w[1] = v.y;
+}
+__device__ __forceinline__ void ldraw4_b(Raw4<f16_t> &q, const f16_t *base, uint32_t off) {
+    const uint2 v = *(const uint2 *)((const char *)base + off);
+    q.w[0] = v.x; q.w[1] = v.y;
+}
+__device__ __forceinline__ void raw4_to_f32(const Raw4<float> &q, float (&o)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = __builtin_bit_cast(float, q.w[e]);
+}
+__device__ __forceinline__ void raw4_to_f32(const Raw4<bf16_t> &q, float (&o)[4]) {
+    o[0] = __builtin_bit_cast(float, q.w[0] << 16); o[1] = __builtin_bit_cast(float, q.w[0] & 0xffff0000u);
+    o[2] = __builtin_bit_cast(float, q.w[1] << 16); o[3] = __builtin_bit_cast(float, q.w[1] & 0xffff0000u);
+}
+__device__ __forceinline__ void raw4_to_f32(const Raw4<f16_t> &q, float (&o)[4]) {
+    o[0] = (float)__builtin_bit_cast(f16_t, (uint16_t)q.w[0]); o[1] = (float)__builtin_bit_cast(f16_t, (uint16_t)(q.w[0] >> 16));
+    o[2] = (float)__builtin_bit_cast(f16_t, (uint16_t)q.w[1]); o[3] = (float)__builtin_bit_cast(f16_t, (uint16_t)(q.w[1] >> 16));
+}
+__device__ __forceinline__ void stg4_b(float *base, uint32_t off, const float (&v)[4]) {
+    *(float4 *)((char *)base + off) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void stg4_b(bf16_t *base, uint32_t off, const float (&v)[4]) {
+    *(uint2 *)((char *)base + off) = make_uint2((uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16),
+                                                (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16));
+}
+__device__ __forceinline__ void stg4_b(f16_t *base, uint32_t off, const float (&v)[4]) {
+    const uint32_t a = __builtin_bit_cast(uint16_t, (f16_t)v[0]), b = __builtin_bit_cast(uint16_t, (f16_t)v[1]);
+    const uint32_t c = __builtin_bit_cast(uint16_t, (f16_t)v[2]), d = __builtin_bit_cast(uint16_t, (f16_t)v[3]);
+    *(uint2 *)((char *)base + off) = make_uint2(a | (b << 16), c | (d << 16));
+}
 __device__ __forceinline__ void stg_b(float *base, uint32_t off, float v) { *(float *)((char *)base + off) = v; }
 __device__ __forceinline__ void stg_b(bf16_t *base, uint32_t off, float v) { ((bf16_t *)((char *)base + off))->v = f32_to_bf16(v); }
 __device__ __forceinline__ void stg_b(f16_t *base, uint32_t off, float v) { *(f16_t *)((char *)base + off) = (f16_t)v; }

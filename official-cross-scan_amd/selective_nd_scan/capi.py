@@ -77,7 +77,6 @@ def lib():
         _lib.snd_workspace_error.argtypes = [vp, vp]
         _lib.snd_debug_set_spin_limit.argtypes = [C.c_int]
         _lib.snd_debug_set_spin_limit.restype = None
-        _lib.snd_debug_issue_probe.argtypes = [C.c_int, C.c_int, C.c_int, vp, vp]
     return _lib
 
 

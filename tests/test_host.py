@@ -12,7 +12,7 @@ import capi
 def test_library_exports_every_declared_symbol():
     names = capi.declared_symbols()
     assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd", "snd_init",
-                          "snd_workspace_error", "snd_debug_set_spin_limit", "snd_debug_issue_probe", "snd_bwd_static",
+                          "snd_workspace_error", "snd_debug_set_spin_limit", "snd_bwd_static",
                           "snd_static_workspace_bytes"}
     lib = capi.lib()
     for n in names:
