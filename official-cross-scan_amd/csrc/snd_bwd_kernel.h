@@ -184,7 +184,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // fused CrossMerge: dout is the gradient of the merged output (one channel per feature, shared by the groups);
     // the channel's weight is applied where dout is staged, and every gradient, being linear in dout, follows
     const bool merge = f.merge != 0;
-    const float wm = merge && f.merge_weights ? f.merge_weights[cc] : 1.f;
+    // (times NaN if the saved state was written by the other kernel family: see kTagTile)
+    const float wm = (merge && f.merge_weights ? f.merge_weights[cc] : 1.f) * tag_poison(geo.tag, kTagTile);
     const uint32_t cDob = ((uint32_t)(merge ? cc - g * rg : cc) * (uint32_t)p.dout_d_stride) << sh_do;
     const uint32_t cGb = (uint32_t)cc * (uint32_t)(H * W) * ESZ;      // du, ddelta
     const int BhB = (int)f.B_h_stride * ESZ, ChB = (int)f.C_h_stride * ESZ, UhB = (int)f.u_h_stride * ESZ, DhB = (int)f.delta_h_stride * ESZ;
@@ -914,7 +915,8 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
 
 template <typename T, int NP>
 static int launch_bwd_np(const snd_bwd_params &p, hipStream_t stream) {
-    const Geo geo = make_geo(p.f.shape.nrows, p.f.shape.ncols);
+    Geo geo = make_geo(p.f.shape.nrows, p.f.shape.ncols);
+    geo.tag = state_tag(p.f.x_sd, p.f.shape);
     if (geo.te == 7) return launch_bwd_te<T, NP, 7, false>(p, geo, stream);
     return bwd_vec_ok(p) ? launch_bwd_te<T, NP, 8, true>(p, geo, stream) : launch_bwd_te<T, NP, 8, false>(p, geo, stream);
 }

@@ -14,10 +14,25 @@ constexpr int kTile = kRows * kCkX;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// The two kernel families lay the saved state out differently in tensors of the same shapes, so the forward leaves a
+// tag in a word of x_sd that neither layout uses (its last one) and the backward compares it with its own: a
+// backward of the other family would compute plausible-looking gradients from state it misreads; with the tag it
+// multiplies dout by NaN instead, and every gradient - all are linear in dout - comes out NaN.
+constexpr uint32_t kTagTile = 0x534E4431u, kTagWave = 0x534E4432u;
+__host__ inline float *state_tag(float *x_sd, const snd_shape &sh) {
+    if (x_sd == nullptr) return nullptr;
+    snd_plan plan;
+    return snd_make_plan(&sh, &plan) == SND_OK ? x_sd + plan.x_sd_elems - 1 : nullptr;
+}
+__device__ __forceinline__ float tag_poison(const float *tag, uint32_t mine) {
+    return (tag == nullptr || *(const volatile uint32_t *)tag == mine) ? 1.f : __builtin_nanf("");
+}
+
 // Geometry of the opaque saved state (see snd_plan in snd_scan.h).  A plane is walked in tiles of
 // te x te cells, te = 8 or 7: 7 where it leaves fewer padded cells (14, 28 and 7 are multiples of 7, not
 // of 8: 23 % less work at those sizes).  Storage keeps 8 slots per tile row / column either way.
 struct Geo {
+    float *tag;                    // the family tag's place in the saved state (state_tag), or null
     int nCX, nCY;                  // column tiles, row strips (of te)
     int Hp, Wp;                    // inner extents of the saved state: nCY*8, nCX*8
     int te;                        // tile extent
@@ -36,6 +51,7 @@ __host__ __device__ inline Geo make_geo(int H, int W) {
     g.nBands = 0;
     g.nQueues = 1;
     g.spinLimit = 1 << 21;
+    g.tag = nullptr;
     return g;
 }
 
@@ -483,6 +499,7 @@ __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, in
 // neighbours in the row come from wave_shr:1 / wave_shl:1; the state at a segment's last column goes to
 // the next wave through a few LDS words per row.
 struct WaveGeo {
+    float *tag;                    // the family tag's place in the saved state (state_tag), or null
     int nseg;                      // row segments (waves per plane): ceil(W / (64 * cpl))
     int R;                         // rows per band (wave_band_rows): row-checkpoint spacing = rows the backward holds in registers
     int nBands;                    // ceil(H / R)
@@ -526,6 +543,7 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     g.Hp = g.nBands * g.R;
     g.Wp = g.nseg * kSeg * g.cpl / wave_pack(g, W);   // (packed planes: a row checkpoint is the plane's own lanes wide)
     g.rg = g.rd = 1; g.gshift = 0; g.xcd = 0;
+    g.tag = nullptr;
     return g;
 }
 // Saved state of this family, per (batch, channel, state) plane, fp32 (S = 64 * cpl columns per segment):

@@ -71,6 +71,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     int *trace_ = nullptr, trace_wait_ = 0;
 #endif
     __shared__ int sDead;                           // (pipelined) a hand-over wait of this block has timed out
+    if (SAVE && blockIdx.x == 0 && threadIdx.x == 0 && geo.tag) *(uint32_t *)geo.tag = kTagTile;   // which family wrote this state
     if (PIPE) {
         if (threadIdx.x == 0) sDead = 0;            // ordered before its readers by the barrier in draw_job
         // A job is a band of consecutive strips (one strip each in the fully pipelined case), drawn
@@ -510,7 +511,8 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
 
 template <typename T, int NP>
 static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
-    const Geo geo = make_geo(p.shape.nrows, p.shape.ncols);
+    Geo geo = make_geo(p.shape.nrows, p.shape.ncols);
+    geo.tag = state_tag(p.x_sd, p.shape);
     return geo.te == 7 ? launch_fwd_te<T, NP, 7>(p, geo, stream) : launch_fwd_te<T, NP, 8>(p, geo, stream);
 }
 

@@ -337,6 +337,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         TORCH_CHECK(mode >= SND_SCHED_AUTO && mode <= SND_SCHED_WAVEFRONT, "schedule must be 0 (auto), 1 (plane), 2 (strips), 3 (bands) or 4 (row-segment wavefront)");
         g_schedule.store(mode);
     }, "Default block mapping of calls that pass no schedule: 0 auto, 1 one block per plane chunk, 2 pipelined row strips, 3 bands");
+    m.def("get_schedule", [] { return g_schedule.load(); }, "The default block mapping calls use when they name none (see set_schedule)");
     m.def("set_debug", [](bool on) { g_check_pipeline.store(on); },
           "Check the pipelined schedules' error word after every launch (a stream sync per call) and raise if a hand-over wait timed out");
     m.def("init", [](int device) { check_status(snd_init(device), "init"); },

@@ -141,7 +141,8 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const T *db = (const T *)f.delta + (int64_t)b * f.delta_batch_stride + (int64_t)(PK > 1 ? 0 : cd) * f.delta_d_stride;
     // fused CrossMerge: dout is the gradient of the merged output, shared by the groups and scaled by the channel's weight
     const bool merge = f.merge != 0;
-    const float wm = merge && f.merge_weights ? f.merge_weights[c] : 1.f;
+    // (times NaN if the saved state was written by the other kernel family: see kTagWave)
+    const float wm = (merge && f.merge_weights ? f.merge_weights[c] : 1.f) * tag_poison(wg.tag, kTagWave);
     const DoT *dob = (const DoT *)p.dout + (int64_t)b * p.dout_batch_stride + (int64_t)(merge ? chB : cB) * p.dout_d_stride;
     T *dub = (T *)p.du + ((int64_t)b * Dm + cB) * H * W;                // du, ddelta: dense [b, c, H, W]
     T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + cB) * H * W;
@@ -584,6 +585,7 @@ int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
     const int N = sh.dstate;
     WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
     wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
+    wg.tag = state_tag(p.f.x_sd, sh);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.dout_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned_b(f.u, e, 2 * e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&

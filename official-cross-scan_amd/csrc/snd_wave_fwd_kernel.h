@@ -113,6 +113,7 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
     const T *Cb = (const T *)p.C + (int64_t)b * p.C_batch_stride + (int64_t)g * p.C_group_stride;
     const T *ub = (const T *)p.u + (int64_t)b * p.u_batch_stride + (int64_t)(p.u_shared ? chB : cB) * p.u_d_stride;
     const T *db = (const T *)p.delta + (int64_t)b * p.delta_batch_stride + (int64_t)(PK > 1 ? 0 : cd) * p.delta_d_stride;
+    if (SAVE && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0 && wg.tag) *(uint32_t *)wg.tag = kTagWave;   // which family wrote this state
     // fused CrossMerge (fp32 out only): the channel adds weight * result to the feature channel it belongs to
     const bool merge = p.merge != 0;
     const float wm = merge && p.merge_weights ? p.merge_weights[c] : 1.f;
@@ -395,6 +396,7 @@ int launch_wave_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
     const int N = sh.dstate;
     WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
     wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
+    wg.tag = state_tag(p.x_sd, sh);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.out_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned(p.u, e, 2 * e, {p.u_batch_stride, p.u_d_stride, p.u_h_stride}) &&

@@ -45,9 +45,18 @@ def bwd(u, delta, A, B, C, D, delta_bias, dout, x, x_v, delta_softplus, A_decay,
 
 def set_schedule(mode):
     """Default block mapping of calls that name none: 0 = chosen by shape, 1 = one block per (batch,
-    group, 16-channel chunk) plane, 2 = one block per 8-row strip, strips pipelined, 3 = bands of strips.
-    Results do not depend on it (only the order of the atomic sums in dA, dB, dC, dD, ddelta_bias does)."""
+    group, 16-channel chunk) plane, 2 = one block per 8-row strip, strips pipelined, 3 = bands of strips,
+    4 = the row-segment wavefront kernels (1-4 states).
+    Results do not depend on it (only the order of the atomic sums in dA, dB, dC, dD, ddelta_bias does), but a
+    bwd must run the kernel family of the fwd whose saved state it is given (modes 1-3 are one family, 4 the other,
+    0 picks by shape): the autograd functions see to that themselves; a bwd on another family's state returns NaN
+    gradients, never plausible numbers."""
     ext().set_schedule(int(mode))
+
+
+def get_schedule():
+    """The default block mapping (see set_schedule)."""
+    return int(ext().get_schedule())
 
 
 def set_debug(on=True):
@@ -72,7 +81,10 @@ class SelectiveNdScanFn(torch.autograd.Function):
     def forward(ctx, u, delta, A, B, C, D=None, delta_bias=None, delta_softplus=False, out_float=True,
                 A_decay=None, directions=0):
         u, delta, B, C = map(_last_dim_contiguous, (u, delta, B, C))
-        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions)
+        # The block mapping is resolved once, here, and the backward is told the same one: the two kernel families keep
+        # different saved-state layouts, so a default changed between a forward and its backward must not reach it.
+        ctx.schedule = get_schedule()
+        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, out_float, A_decay, directions, ctx.schedule)
         ctx.delta_softplus = delta_softplus
         ctx.directions = directions
         ctx.has = (D is not None, delta_bias is not None, A_decay is not None)
@@ -85,7 +97,7 @@ class SelectiveNdScanFn(torch.autograd.Function):
         u, delta, A, B, C, D, delta_bias, A_decay, x, x_v, x_sd = ctx.saved_tensors
         dout = _last_dim_contiguous(dout)
         du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay = bwd(
-            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions)
+            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions, ctx.schedule)
         has_D, has_bias, has_decay = ctx.has
         return (du, ddelta, dA, dB, dC, dD if has_D else None, ddelta_bias if has_bias else None,
                 None, None, dA_decay if has_decay else None, None)
@@ -118,7 +130,8 @@ class SelectiveNdScanMergedFn(torch.autograd.Function):
         if merge_weights is not None:
             G = B.shape[1]
             w = merge_weights.detach().to(torch.float32).reshape(G, -1).expand(G, A.shape[0] // G).contiguous().view(-1)
-        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay, directions, -1, True, w)
+        ctx.schedule = get_schedule()               # (resolved once for the pair: see SelectiveNdScanFn.forward)
+        out, x, x_v, x_sd = fwd(u, delta, A, B, C, D, delta_bias, delta_softplus, True, A_decay, directions, ctx.schedule, True, w)
         ctx.delta_softplus = delta_softplus
         ctx.directions = directions
         ctx.has = (D is not None, delta_bias is not None, A_decay is not None)
@@ -137,7 +150,7 @@ class SelectiveNdScanMergedFn(torch.autograd.Function):
             floor = torch.full_like(w, _MERGE_WEIGHT_FLOOR)
             wb = torch.where(w.abs() < _MERGE_WEIGHT_FLOOR, floor, w)
         du, ddelta, dA, dB, dC, dD, ddelta_bias, dA_decay, wdw = bwd(
-            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions, -1,
+            u, delta, A, B, C, D, delta_bias, dout, x, x_v, ctx.delta_softplus, A_decay, x_sd, ctx.directions, ctx.schedule,
             True, wb)
         dw = None
         if w is not None and ctx.needs_input_grad[10]:

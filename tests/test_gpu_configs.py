@@ -49,6 +49,12 @@ def test_config_plane_sizes(gpu_device, name, Bt, Dm, H, W, N, K, dtype):
         tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
         assert relerr(a.float().cpu().numpy(), b_) <= tol, (nm, relerr(a.float().cpu().numpy(), b_))
     if half:
-        # headline tolerance for 16-bit inputs: within 1e-2 of the oracle fed the un-rounded fp32 inputs
+        # headline tolerance for 16-bit inputs: out and every gradient within 1e-2 of the oracle fed the UN-ROUNDED fp32
+        # inputs (max|x - ref| / max|ref| per tensor)
         ref32 = OC.fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], True, None, real="f64")
         assert relerr(out.cpu().numpy(), ref32) <= 1e-2
+        gref32 = OC.bwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["delta_bias"], d["dout"], True, None, real="f64")
+        for nm, a, b_ in zip(NAMES, g, gref32):
+            e = relerr(a.float().cpu().numpy(), b_)
+            print("  un-rounded", nm, "%.2e" % e, flush=True)
+            assert e <= 1e-2, (nm, e)
