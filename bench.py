@@ -10,15 +10,19 @@ Prints ONE JSON line.  `value` is the algorithmic HBM rate of the whole step:
 (compulsory tensor I/O only) divided by the mean step time.  `roofline` is the same figure for the
 dominant kernel alone (the backward), from one pair of HIP events on the launch stream around K back-to-back
 launches of it through the C ABI (after W untimed ones; defaults K = 50, W = 20: the clocks settle over the first
-10-15 steps after the host-side input generation), with
-a second leg beside it: vector-ALU wave-instructions per second against the published FP32 vector peak
-(157.3 TFLOP/s = 1228.9 G wave-wide multiply-adds per second: a SIMD retires one 64-lane FP32 instruction
-per two cycles), with the rate `--issue-probe` measures for a pure multiply-add stream on all CUs beside
-it (`valu.probe_peak`, from profiles/issue_probe_mi355x.txt).  The instruction count, the clock and the
-HBM traffic per launch are counter readings that a timed run cannot take; they come from the committed
-rocprofv3 summary of the same workload under profiles/ (named in `roofline.counters_from`), while every
-duration is measured live.  `roofline.bound` names the leg with the higher fraction.  `cpu_baseline` times the C restatement of the reference recurrence
-(oracle/) on the host cores on a bounded sample of the same workload.
+10-15 steps after the host-side input generation), with a second leg beside it: vector-ALU wave-instructions per
+second against the published FP32 vector peak (157.3 TFLOP/s = 1228.9 G wave-wide multiply-adds per second), with
+the rate a pure multiply-add stream reaches on all CUs beside it (`valu.probe_peak`, from
+profiles/issue_probe_mi355x.txt).  `roofline_fwd` is the same pair of figures for the forward kernel, plus the
+rate of its real memory traffic (checkpoints and re-reads included).  The instruction count, the clock and the
+traffic per launch are counter readings that a timed run cannot take; they come from the committed rocprofv3
+summary of the same workload under profiles/ (named in `counters_from`) and are used only if that summary was
+taken from the kernel sources of this tree (`kernel_source_sha`) and its kernel durations agree with the ones
+measured here within 5 % (`profile_vs_live`); otherwise they are left out (null) and `counters_stale` says why.
+Every duration is measured live.  `roofline.bound` names the leg with the higher fraction.
+`cpu_baseline` times the C restatement of the reference recurrence (oracle/) on the host cores on a bounded sample
+of the same workload; `cpu_baseline_torch` the line-for-line PyTorch transcription of the recurrence (forward, and
+autograd through it for the backward) on a smaller sample.
 """
 import argparse
 import json
@@ -33,7 +37,7 @@ for p in (ROOT, os.path.join(ROOT, "official-cross-scan_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-METRIC = "fwd+bwd 2D-scan ms/iter & HBM GB/s (% peak), B64 D192 56x56 N16 K4"
+METRIC = "fwd+bwd 2D-scan ms/iter & HBM GB/s (% peak), "     # + the workload: B64 D192 56x56 N16 K4 for c1
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published peak
 WORKLOADS = {                   # name: (B, D, H, W, N, K, input dtype)
     "c1": (64, 192, 56, 56, 16, 4, "float32"),
@@ -124,22 +128,72 @@ def probe_peak():
     return float(m.group(1)) * 1e9 if m else None
 
 
+def kernel_source_sha():
+    """sha256 (16 hex digits) over the kernel sources (csrc/*.h, *.hip, in name order): stored in every profile summary
+    under profiles/ and compared here, so that counters taken from other kernels than the ones that run are not used."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "official-cross-scan_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(csrc, "*.h")) + glob.glob(os.path.join(csrc, "*.hip"))):
+        h.update(os.path.basename(path).encode() + b"\0" + open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def profile_counters(workload):
-    """Counter readings of the dominant kernel (the backward) from the committed rocprofv3 summary of
-    this workload: kernel name, HBM bytes per launch, VALU wave-instructions per launch, shader clock
-    under this load.  A timed run cannot read counters; durations are always measured live."""
+    """Counter readings of the two kernels from the committed rocprofv3 summary of this workload: kernel names, memory
+    traffic per launch, VALU wave-instructions per launch, shader clock under this load, average durations, and the
+    hash of the kernel sources the summary was taken from.  A timed run cannot read counters; durations are always
+    measured live."""
     rel = os.path.join("profiles", "bwd_kernel_%s_pmc.txt" % workload)
     path = os.path.join(ROOT, rel)
     if not os.path.exists(path):
         return None
     text = open(path).read()
     out = {"file": rel}
-    for key in ("dominant_kernel", "avg_ns", "traffic_bytes_per_launch", "valu_insts_per_launch", "clock_ghz"):
+    for key in ("dominant_kernel", "avg_ns", "traffic_bytes_per_launch", "valu_insts_per_launch", "clock_ghz",
+                "fwd_kernel", "fwd_avg_ns", "fwd_traffic_bytes_per_launch", "fwd_valu_insts_per_launch", "fwd_clock_ghz",
+                "kernel_source_sha"):
         m = re.search(r"^%s:\s*(.+)$" % key, text, flags=re.M)
         if not m:
+            if key == "kernel_source_sha":
+                out[key] = None
+                continue
             return None
-        out[key] = m.group(1).strip() if key == "dominant_kernel" else float(m.group(1))
+        out[key] = m.group(1).strip() if key in ("dominant_kernel", "fwd_kernel", "kernel_source_sha") else float(m.group(1))
     return out
+
+
+def cpu_baseline_torch(workload, budget_s=12.0):
+    """The line-for-line PyTorch transcription of the reference recurrence (oracle/snd_torch_ref.py: a row loop over a
+    column loop of h = a*(h_left + h_up - 0.5*(a_up + a_left)*h_diag) + bu, vectorised over (batch, channel, state)),
+    forward and autograd backward, fp32, on the host cores, on a slice of the workload sized to a few seconds."""
+    import torch
+    from oracle import snd_oracle as O
+    from oracle.snd_torch_ref import selective_nd_scan_torch
+    Bt, Dm, H, W, N, K, dtn = WORKLOADS[workload]
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    cores = int(env) if env.isdigit() and int(env) > 0 else (os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    # the python loops cost about a millisecond per cell (forward + backward) whatever the slice holds, so the slice is
+    # 3072 (channel, state) planes wide (autograd keeps a dozen fp32 values per state-cell: ~150 KB per cell) and as
+    # many rows long as the budget allows: the first rows of the plane, all of them where they fit
+    rows = max(4, min(H, int(budget_s / 1e-3) // W))
+    sd = min(Dm, K * max(1, 3072 // (K * N)))
+    d = O.make_inputs(1, sd, rows, W, N=N, K=K, seed=0)
+    t = {k: torch.from_numpy(v) for k, v in d.items()}
+    leaves = [t[k].clone().requires_grad_(True) for k in ("u", "delta", "A", "B", "C", "D", "delta_bias")]
+    t0 = time.perf_counter()
+    out = selective_nd_scan_torch(*leaves, delta_softplus=True)
+    t1 = time.perf_counter()
+    out.backward(t["dout"])
+    t2 = time.perf_counter()
+    fb, bb = algorithmic_bytes(1, sd, rows, W, N, K, 4)
+    full = (t2 - t0) * (Bt * Dm * H) / (sd * rows)
+    return {"value": round((fb + bb) / (t2 - t0) / 1e9, 5), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "%s slice B=1 D=%d rows=%d of %d (fp32), forward %.2f s + autograd backward %.2f s, once"
+                      % (workload, sd, rows, H, t1 - t0, t2 - t1),
+            "ms_per_step_extrapolated": round(1e3 * full, 0)}
 
 
 def main():
@@ -207,30 +261,51 @@ def main():
     kb_ms = kernel_ms(bcall.launch_kernel_only)     # (the accumulated gradients are not cleared in between: timing only)
 
     value = (fb + bb) / (ms * 1e-3) / 1e9
-    achieved = bb / (kb_ms * 1e-3) / 1e9
     st, plan = capi.make_plan(capi.make_shape(u, delta, A, B))
     capi.check(st)
     used = sched if sched else plan.auto_schedule
-    kernel = "snd::wave_bwd_kernel" if used == capi.SCHED_WAVEFRONT else "snd::bwd_kernel"
-    roof = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_launch": bb,
-            "kernel_ms": round(kb_ms, 4)}
+    wave = used == capi.SCHED_WAVEFRONT
+    pp = probe_peak()
+
+    def leg(kernel, alg_bytes, k_ms):
+        ach = alg_bytes / (k_ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": kernel, "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                "kernel_ms": round(k_ms, 4)}
+
+    def add_counters(r, k_ms, file, traffic, insts, clock, prof_ns):
+        rate = insts / (k_ms * 1e-3)
+        r.update({"traffic": traffic, "traffic_GBs": round(traffic / (k_ms * 1e-3) / 1e9, 1), "counters_from": file,
+                  "profile_kernel_ms": round(prof_ns * 1e-6, 4), "profile_vs_live": round(prof_ns * 1e-6 / k_ms, 3),
+                  "valu": {"insts_per_launch": insts, "clock_ghz": clock, "achieved": round(rate / 1e9, 2),
+                           "peak": round(VALU_PEAK / 1e9, 2), "probe_peak": round(pp / 1e9, 2) if pp else None,
+                           "unit": "G wave-instructions/s"},
+                  "frac_valu": round(rate / VALU_PEAK, 4)})
+        if r["frac_valu"] > r["frac"]:
+            r["bound"] = "valu"
+
+    roof = leg("snd::wave_bwd_kernel" if wave else "snd::bwd_kernel", bb, kb_ms)
+    roof_fwd = leg("snd::wave_fwd_kernel" if wave else "snd::fwd_kernel", fb, kf_ms)
     pc = profile_counters(args.workload) if args.schedule == "auto" else None
-    if pc and pc["dominant_kernel"].startswith(kernel + "<"):
-        # counters from the committed profile of this workload; the rate uses the duration measured here
-        peak_valu = VALU_PEAK
-        rate_valu = pc["valu_insts_per_launch"] / (kb_ms * 1e-3)
-        pp = probe_peak()
-        roof.update({"traffic": pc["traffic_bytes_per_launch"], "counters_from": pc["file"],
-                     "profile_kernel_ms": round(pc["avg_ns"] * 1e-6, 4),
-                     "valu": {"insts_per_launch": pc["valu_insts_per_launch"], "clock_ghz": pc["clock_ghz"],
-                              "achieved": round(rate_valu / 1e9, 2), "peak": round(peak_valu / 1e9, 2),
-                              "probe_peak": round(pp / 1e9, 2) if pp else None, "unit": "G wave-instructions/s"},
-                     "frac_valu": round(rate_valu / peak_valu, 4)})
-        if roof["frac_valu"] > roof["frac"]:
-            roof["bound"] = "valu"
+    if pc:
+        # counters from the committed profile of this workload, if it is a profile of these kernels: same kernel,
+        # same sources, and durations that agree with the ones measured here
+        stale = None
+        if not pc["dominant_kernel"].startswith(roof["kernel"] + "<") or not pc["fwd_kernel"].startswith(roof_fwd["kernel"] + "<"):
+            stale = "the profile is of other kernels (%s)" % pc["dominant_kernel"].split("<")[0]
+        elif pc["kernel_source_sha"] != kernel_source_sha():
+            stale = "the profile was taken from other kernel sources (%s, here %s)" % (pc["kernel_source_sha"], kernel_source_sha())
+        elif not (0.95 <= pc["avg_ns"] * 1e-6 / kb_ms <= 1.05 and 0.95 <= pc["fwd_avg_ns"] * 1e-6 / kf_ms <= 1.05):
+            stale = "kernel durations differ from the profile's by more than 5 %% (bwd %.3f, fwd %.3f)" % (
+                pc["avg_ns"] * 1e-6 / kb_ms, pc["fwd_avg_ns"] * 1e-6 / kf_ms)
+        if stale is None:
+            add_counters(roof, kb_ms, pc["file"], pc["traffic_bytes_per_launch"], pc["valu_insts_per_launch"], pc["clock_ghz"], pc["avg_ns"])
+            add_counters(roof_fwd, kf_ms, pc["file"], pc["fwd_traffic_bytes_per_launch"], pc["fwd_valu_insts_per_launch"],
+                         pc["fwd_clock_ghz"], pc["fwd_avg_ns"])
+        else:
+            roof["counters_stale"] = roof_fwd["counters_stale"] = "%s: %s" % (pc["file"], stale)
     rec = {
-        "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "metric": METRIC + "B%d D%d %dx%d N%d K%d" % (Bt, Dm, H, W, N, K), "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         # arithmetic type of the recurrence and of every accumulation, whatever the I/O dtype of the workload
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -242,9 +317,11 @@ def main():
                    "kernel_ms": {"fwd": round(kf_ms, 4), "bwd": round(kb_ms, 4)},
                    "kernel_only_GBs": round((fb + bb) / ((kf_ms + kb_ms) * 1e-3) / 1e9, 2)},
         "roofline": roof,
+        "roofline_fwd": roof_fwd,
     }
     if not args.no_cpu:
         rec["cpu_baseline"] = cpu_baseline(args.workload)
+        rec["cpu_baseline_torch"] = cpu_baseline_torch(args.workload)
     print(json.dumps(rec))
 
 

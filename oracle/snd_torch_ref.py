@@ -25,6 +25,10 @@ def selective_nd_scan_torch(u, delta, A, B, C, D=None, delta_bias=None, delta_so
     Cc = C.repeat_interleave(Dm // G, dim=1)
     bu = Bc * (dl * u)[:, :, None]
     zero = torch.zeros(Bt, Dm, N, dtype=u.dtype)
+    # per-cell views taken once (unbind: its backward is one stack per row, where indexing a[..., i, j] cell by
+    # cell would scatter every cell's gradient into a zero tensor of the whole plane)
+    ac = [r.unbind(-1) for r in a.unbind(-2)]
+    buc = [r.unbind(-1) for r in bu.unbind(-2)]
     rows_h, rows_s = [], []
     for i in range(H):
         hrow, srow = [], []
@@ -32,13 +36,13 @@ def selective_nd_scan_torch(u, delta, A, B, C, D=None, delta_bias=None, delta_so
             left = hrow[j - 1] if j > 0 else zero
             up = rows_h[i - 1][j] if i > 0 else zero
             if i > 0 and j > 0:
-                corr = 0.5 * (a[..., i - 1, j] + a[..., i, j - 1]) * rows_h[i - 1][j - 1]
+                corr = 0.5 * (ac[i - 1][j] + ac[i][j - 1]) * rows_h[i - 1][j - 1]
             else:
                 corr = zero
-            hrow.append(a[..., i, j] * (left + up - corr) + bu[..., i, j])
+            hrow.append(ac[i][j] * (left + up - corr) + buc[i][j])
             if sd:
                 sl = srow[j - 1] if j > 0 else zero
-                srow.append(a[..., i, j] * sl + bu[..., i, j])
+                srow.append(ac[i][j] * sl + buc[i][j])
         rows_h.append(hrow)
         rows_s.append(srow)
     h = torch.stack([torch.stack(r, dim=-1) for r in rows_h], dim=-2)
