@@ -230,7 +230,8 @@ int snd_init(int device);
  * before; this call is how a host learns the reason: it copies word [1] back and WAITS for `stream`
  * (the only synchronising call of the library).  Returns SND_OK, SND_ERR_PIPELINE, or another error.
  * Meaningful only after a pipelined launch on that workspace (a whole-plane launch leaves the header
- * alone).  No counterpart in the reference, whose blocks never wait for each other. */
+ * alone).  workspace == NULL asks about the static scratch of snd_bwd_static on the current device.
+ * No counterpart in the reference, whose blocks never wait for each other. */
 int snd_workspace_error(const void *workspace, snd_stream_t stream);
 
 /* Test hook: poll limit of the hand-over waits for later launches (<= 0 restores the default 2^21).
@@ -243,7 +244,9 @@ void snd_debug_set_spin_limit(int polls);
  * torch::empty / torch::zeros inside every call (selective_scan_oflex.cpp:393-403).  Identical to
  * snd_bwd except that params->workspace / workspace_bytes are ignored: the scratch is a static device
  * array of snd_static_workspace_bytes() bytes (64 MiB per GPU, held until the process ends) that the
- * library owns.  Shapes whose plan.bwd_workspace_bytes exceeds it are refused with SND_ERR_TOO_LARGE.
+ * library owns.  Shapes whose plan.bwd_workspace_bytes exceeds it are refused with SND_ERR_TOO_LARGE (calls that
+ * run the row-segment kernels use no scratch and are never refused for size).  A timed-out hand-over is reported
+ * by snd_workspace_error(NULL, stream).
  * The caller still passes every input, output and saved-state buffer.  Allocates nothing, frees nothing.
  * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race;
  * calls on one stream are ordered.  The sync header is cleared by a fill kernel at the start of each

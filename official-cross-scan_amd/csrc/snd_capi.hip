@@ -322,7 +322,9 @@ int snd_bwd_static(const snd_bwd_params *params, snd_stream_t stream) {
     snd_plan plan;
     int st = snd_make_plan(&params->f.shape, &plan);
     if (st != SND_OK) return st;
-    if (plan.bwd_workspace_bytes > SND_STATIC_WORKSPACE_BYTES) return SND_ERR_TOO_LARGE;
+    // (the row-segment kernels use no scratch at all: no size limit for them)
+    const int wave = use_wavefront(params->f.shape, params->f.schedule);
+    if (wave == 0 && plan.bwd_workspace_bytes > SND_STATIC_WORKSPACE_BYTES) return SND_ERR_TOO_LARGE;
     st = snd::ensure_device_ready();                // no allocation: symbol lookup and kernel attributes, once per device
     if (st != SND_OK) return st;
     void *ws = snd::device_scratch();
@@ -334,7 +336,10 @@ int snd_bwd_static(const snd_bwd_params *params, snd_stream_t stream) {
 }
 
 int snd_workspace_error(const void *workspace, snd_stream_t stream) {
-    if (!workspace) return SND_ERR_NULL;
+    if (!workspace) {                               // the static scratch of snd_bwd_static on the current device
+        workspace = snd::device_scratch();
+        if (!workspace) return SND_ERR_NULL;        // (never set up: no launch has used it)
+    }
     int word = 0;
     if (hipMemcpyAsync(&word, (const int *)workspace + snd::kErrorWord, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
         return SND_ERR_LAUNCH;

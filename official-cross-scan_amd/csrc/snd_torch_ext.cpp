@@ -253,12 +253,15 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // so that a parameter gradient kept by the optimizer never pins the large buffer.
     const int64_t nA = (int64_t)dim * dstate, nBC = B.numel();
     auto round64 = [](int64_t v) { return (v + 63) / 64 * 64; };
-    // (dC a chosen distance past the 2 MiB-rounded end of dB, snd_plan.dC_skew_bytes: the two are accumulated at equal
-    // offsets at the same time and must not sit a multiple of 2 MiB apart)
-    const int64_t oC = (round_2mib(nBC * 4) + c.plan.dC_skew_bytes) / 4;
-    at::Tensor accBC = torch::zeros({oC + round64(nBC)}, f32);
+    // dB and dC are accumulated at equal offsets at the same time.  Where that matters (the row-segment kernels on
+    // tensors of 2 MiB and more) dC starts a chosen distance past the 2 MiB-rounded end of dB (snd_plan.dC_skew_bytes:
+    // not a multiple of 2 MiB apart); everywhere else it follows dB directly and nothing beyond the two is filled.
+    const bool spread = c.plan.auto_schedule == SND_SCHED_WAVEFRONT && nBC * 4 >= (int64_t)(2 << 20);
+    const int64_t oC = spread ? (round_2mib(nBC * 4) + c.plan.dC_skew_bytes) / 4 : round64(nBC);
+    at::Tensor accBC = spread ? torch::empty({oC + nBC}, f32) : torch::zeros({oC + nBC}, f32);
     at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
     at::Tensor dC = accBC.narrow(0, oC, nBC).view(C.sizes());
+    if (spread) { dB.zero_(); dC.zero_(); }         // (not the gap between them)
     const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim), oMerge = oDec + 64;
     at::Tensor accP = torch::zeros({oMerge + (merge ? round64(dim) : 0)}, f32);
     at::Tensor dA = accP.narrow(0, 0, nA).view({dim, dstate});
@@ -300,9 +303,14 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // (16-bit inputs: one cast kernel for the two tensors, which share a buffer)
     at::Tensor dBo = dB, dCo = dC;
     if (B.scalar_type() != at::ScalarType::Float) {
-        const at::Tensor cast = accBC.to(B.dtype());
-        dBo = cast.narrow(0, 0, nBC).view(B.sizes());
-        dCo = cast.narrow(0, oC, nBC).view(C.sizes());
+        if (spread) {                               // two casts of the live ranges, not one of the gap as well
+            dBo = dB.to(B.dtype());
+            dCo = dC.to(C.dtype());
+        } else {
+            const at::Tensor cast = accBC.to(B.dtype());
+            dBo = cast.narrow(0, 0, nBC).view(B.sizes());
+            dCo = cast.narrow(0, oC, nBC).view(C.sizes());
+        }
     }
     std::vector<at::Tensor> result = {du, ddelta, dA, dBo, dCo, dD, ddelta_bias, dA_decay};
     if (dim != c.delta_dim) {

@@ -60,3 +60,45 @@ def test_bwd_static_refuses_what_does_not_fit(gpu_device):
     q = capi.BwdParams.from_buffer_copy(b.params)
     q.f.shape = capi.Shape(64, 768, 56, 56, 16, 4, 768, capi.SND_F32)
     assert capi.lib().snd_bwd_static(capi.C.byref(q), torch.cuda.current_stream().cuda_stream) == -8
+    # the same size with one state runs the row-segment kernels, which use no scratch: never refused for size
+    # (null inputs: the call must get past the size check and stop at the pointer checks instead)
+    q.f.shape = capi.Shape(64, 768, 56, 56, 1, 4, 768, capi.SND_F32)
+    q.f.u = None
+    assert capi.lib().snd_bwd_static(capi.C.byref(q), torch.cuda.current_stream().cuda_stream) == -1
+
+
+def test_bwd_static_few_states_and_timeout_query(gpu_device):
+    """AUTO with one state (row-segment kernels) through the static entry point, and the error word of the static
+    scratch read back through snd_workspace_error(NULL, stream): clean after a clean pipelined call, set after one
+    whose hand-over waits were forced to give up (poll limit 1; every kernel still drains, the outputs are NaN)."""
+    lib = capi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    d, t, f, b = _case(gpu_device, 2, 16, 30, 70, 1, 4, capi.SCHED_AUTO, 5)
+    b.launch()
+    torch.cuda.synchronize()
+    want = _grads(b)
+    b.launch_static()
+    torch.cuda.synchronize()
+    got = _grads(b)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    for nm, a, w in zip(NAMES[2:], got[2:], want[2:]):
+        assert relerr(a.cpu().numpy(), w.cpu().numpy()) <= 1e-5, nm
+    d, t, f, b = _case(gpu_device, 1, 32, 160, 160, 16, 2, capi.SCHED_STRIPS, 13)
+    b.launch_static()
+    torch.cuda.synchronize()
+    assert lib.snd_workspace_error(None, stream) == 0 and not torch.isnan(b.du).any()
+    try:
+        lib.snd_debug_set_spin_limit(1)
+        b.launch_static()
+        torch.cuda.synchronize()
+        st = lib.snd_workspace_error(None, stream)
+        assert st in (0, -9)
+        if st == -9:
+            assert torch.isnan(b.du).any(), "a timed-out launch must poison its outputs"
+        else:                                         # every wait happened to be satisfied at once
+            assert not torch.isnan(b.du).any()
+    finally:
+        lib.snd_debug_set_spin_limit(0)
+    b.launch_static()
+    torch.cuda.synchronize()
+    assert lib.snd_workspace_error(None, stream) == 0 and not torch.isnan(b.du).any()
