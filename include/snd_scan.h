@@ -239,6 +239,12 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream);
  * kernel still runs to completion. */
 void snd_debug_set_spin_limit(int polls);
 
+/* Test hook: the number of block slots the backward's strip-pipeline model assumes when it decides whether to cut
+ * strips into column segments (0 restores the machine's own count); a negative value -n skips the model and cuts
+ * every pipelined strip into n segments (at least two tiles each).  Small test shapes then take the segmented
+ * path - plan sizes and launches alike - that only shapes with more strips than slots take otherwise. */
+void snd_debug_set_strip_slots(int slots);
+
 /* snd_bwd for callers that cannot allocate device memory (code under HIP-graph capture, serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference, which allocates its scratch with
  * torch::empty / torch::zeros inside every call (selective_scan_oflex.cpp:393-403).  Identical to

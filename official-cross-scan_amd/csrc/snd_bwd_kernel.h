@@ -68,9 +68,13 @@ __device__ __forceinline__ void rows_scatter4x2(float &b0, float &b1, float &b2,
 // 8-byte (16-bit) access per thread and tensor instead of one access per element - a quarter of the memory
 // instructions and of their address arithmetic.  Needs 8x8 tiles, a width that is a multiple of four and tensors
 // whose rows start on such boundaries (bwd_vec_ok); everything else takes the element-wise staging.
-template <typename T, int NP, bool PIPE, int TE, bool VEC>
+// SEG: (pipelined strips only) a job is a column segment of a strip; the carried column state goes from one
+// segment's block to the next through the workspace (strip_segments).  A variant of its own, because the few
+// registers it takes are registers the other variants do not have.
+template <typename T, int NP, bool PIPE, int TE, bool VEC, bool SEG = false>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD_WAVES, SND_BWD_WAVES))) void bwd_kernel(const snd_bwd_params p, const Geo geo) {
     static_assert(!VEC || TE == 8, "vector staging needs 8x8 tiles");
+    static_assert(!SEG || PIPE, "column segments belong to the strip pipeline");
     constexpr int WPB = NP / 4;                     // waves per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;
@@ -116,7 +120,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     const int nChunks = (rg + CB - 1) / CB;
     int pair, chunk;
     int I_hi = geo.nCY - 1, I_lo = 0;               // strips this block walks, bottom to top
-    int *sync = (int *)p.workspace, *progress = nullptr;
+    int J_hi = geo.nCX - 1, J_lo = 0, seg = 0;      // and the tiles of a strip, right to left (a column segment of a pipelined strip)
+    int *sync = (int *)p.workspace, *progress = nullptr, *segdone = nullptr;
+    float *colstate = nullptr;
     const int64_t nSync = sync_words((int64_t)sh.batch * G * nChunks, geo.nCY);
     bool dead = false;
     int seen = 0;                                   // last progress count read (strip pipeline)
@@ -131,15 +137,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         // bottom band first; band k from the bottom covers strips ceil(k*nCY/nBands) ..
         // ceil((k+1)*nCY/nBands)-1, counted from the bottom.
         int band;
-        if (!draw_job(sync, sh.batch * G, nChunks, geo.nBands, geo.nQueues, pair, chunk, band)) return;
+        if (!draw_job(sync, sh.batch * G, nChunks, geo.nBands, geo.nQueues, pair, chunk, band, SEG ? geo.nSeg : 1, geo.segTiles, &seg)) return;
         const int nPC = sh.batch * G * nChunks;
         const int pc = pair * nChunks + chunk;
         I_hi = geo.nCY - 1 - (band * geo.nCY + geo.nBands - 1) / geo.nBands;
         I_lo = geo.nCY - ((band + 1) * geo.nCY + geo.nBands - 1) / geo.nBands;
-        (void)nPC;
         progress = sync + kSyncHeader + pc * geo.nCY;
+        // (column-segmented strips: one strip per job) the segment's tiles, right to left; the carried column state
+        // of the strip goes from segment to segment through one slot of the workspace
+        if (SEG) {
+            J_hi = geo.nCX - 1 - seg * geo.segTiles;
+            J_lo = seg == geo.nSeg - 1 ? 0 : J_hi - geo.segTiles + 1;
+            segdone = progress + nPC * geo.nCY;
+            colstate = (float *)p.workspace + nSync + (int64_t)sh.batch * Dm * N * geo.Wp + ((int64_t)pc * geo.nCY + I_hi) * kColStateFloats;
+        }
 #ifdef SND_PIPE_TRACE
-        trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_hi);
+        trace_ = sync + kSyncHeader + 2 * nPC * geo.nCY + 4 * (pc * geo.nCY + I_hi);
         if (threadIdx.x == 0) trace_[0] = (int)wall_clock64();
 #endif
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;
@@ -455,8 +468,33 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
         float GRc = 0.f;                            // G[r0+8][j0+8]
 #pragma unroll
         for (int r = 0; r < kRows; ++r) { GR[r] = 0.f; GsR[r] = 0.f; aR[r] = 0.f; }
+        if (SEG && seg > 0) {
+            // a later column segment of the strip: G, Gs, a of the column right of it and the corner G come from the
+            // block that swept the segment before (written in full before its count moved: see strip_stores_done)
+            if (wave == 0) {
+                int seen_ = 0;
+                strip_wait(segdone + I, seg, seen_, sync, dead, geo.spinLimit SND_TRACE_PASS);
+                if (dead && tid == 0) sDead = 1;
+            }
+            __syncthreads();
+            const float *src = colstate + (tid << 1);
+            const bool bad = *(volatile int *)&sDead != 0;   // the wait timed out: poison everything downstream
+#pragma unroll
+            for (int r = 0; r < kRows; r += 2) {
+                ld2_coherent(src + (r >> 1) * 512, GR[r], GR[r + 1]);
+                ld2_coherent(src + (4 + (r >> 1)) * 512, GsR[r], GsR[r + 1]);
+                ld2_coherent(src + (8 + (r >> 1)) * 512, aR[r], aR[r + 1]);
+            }
+            float pad_;
+            ld2_coherent(src + 12 * 512, GRc, pad_);
+            if (bad) {
+                GRc = __builtin_nanf("");
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) GR[r] = GsR[r] = __builtin_nanf("");
+            }
+        }
 
-        for (int J = geo.nCX - 1; J >= 0; --J) {
+        for (int J = SEG ? J_hi : geo.nCX - 1; J >= (SEG ? J_lo : 0); --J) {
             const int j0 = J * TE;
             // ---- checkpoints and carried adjoints of this tile: requested first, so that they arrive
             // under the staging below instead of being waited for after the barrier
@@ -805,6 +843,21 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             }
             }
         }
+        if (SEG && seg + 1 < geo.nSeg) {
+            // hand the carried column state to the block of the strip's next segment: stores, each wave waits for its
+            // own to complete, block barrier, then one thread moves the strip's count of finished segments
+            float *dst = colstate + (tid << 1);
+#pragma unroll
+            for (int r = 0; r < kRows; r += 2) {
+                st2_coherent(dst + (r >> 1) * 512, GR[r], GR[r + 1]);
+                st2_coherent(dst + (4 + (r >> 1)) * 512, GsR[r], GsR[r + 1]);
+                st2_coherent(dst + (8 + (r >> 1)) * 512, aR[r], aR[r + 1]);
+            }
+            st2_coherent(dst + 12 * 512, GRc, 0.f);
+            strip_stores_done();
+            __syncthreads();
+            strip_signal(segdone + I);
+        }
     }
     if (pI >= 0) flush_bc(pI, pJ);
 #undef DL
@@ -851,6 +904,8 @@ template <int NP> constexpr size_t bwd_lds_bytes() {
 // done once per device at set-up and not inside the launch path.
 template <typename T, int NP, int TE, bool VEC> static bool configure_bwd_one() {
     const int lds = (int)bwd_lds_bytes<NP>();
+    if (NP == 16 && hipFuncSetAttribute((const void *)bwd_kernel<T, NP, true, TE, VEC, NP == 16>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return false;
     return hipFuncSetAttribute((const void *)bwd_kernel<T, NP, true, TE, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
            hipFuncSetAttribute((const void *)bwd_kernel<T, NP, false, TE, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess;
 }
@@ -905,7 +960,15 @@ static int launch_bwd_te(const snd_bwd_params &p, const Geo &geo, hipStream_t st
         gb.spinLimit = spin_limit();
         gb.nBands = bands;
         gb.nQueues = job_queues(sh.batch * sh.n_groups);
-        hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE, VEC>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);
+        // one strip per job and more strips than block slots: the strips may be cut into column segments (the plan
+        // has sized the workspace for their carried state)
+        if (bands == geo.nCY && NP == 16) gb.nSeg = strip_segments(nPC, geo.nCY, geo.nCX, bwd_slots(sh.dstate), gb.nQueues);
+        gb.segTiles = geo.nCX / gb.nSeg;
+        if (nPC * bands * gb.nSeg >= (int64_t)1 << 31) return SND_ERR_SHAPE;
+        if (NP == 16 && gb.nSeg > 1)
+            hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE, VEC, NP == 16>), dim3((int)(nPC * bands * gb.nSeg)), dim3(16 * NP), lds, stream, p, gb);
+        else
+            hipLaunchKernelGGL((bwd_kernel<T, NP, true, TE, VEC>), dim3((int)(nPC * bands)), dim3(16 * NP), lds, stream, p, gb);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
         hipLaunchKernelGGL((bwd_kernel<T, NP, false, TE, VEC>), dim3(grid), dim3(16 * NP), lds, stream, p, geo);

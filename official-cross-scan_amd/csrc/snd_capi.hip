@@ -1,8 +1,14 @@
 // C ABI of the gfx950 selective_nd_scan library: validation, planning and dispatch.
 // Mirrors the checks of the reference host binding
 // (kernels/selective_nd_scan/src/cusoflex/selective_scan_oflex.cpp:188-245,298-361) as status codes.
+#include <algorithm>
 #include <atomic>
+#include <functional>
+#include <map>
 #include <mutex>
+#include <queue>
+#include <tuple>
+#include <vector>
 
 #include "snd_device.h"
 
@@ -47,6 +53,63 @@ static void *g_scratch[kMaxDevices];                // device address of `scratc
 static std::atomic<int> g_spin_limit{kSpinLimit};
 
 int spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
+
+// Tile steps the strip pipeline takes: jobs (plane chunk, strip, segment) in ticket order, each taken by the first
+// free slot; a tile starts when its block has finished the tile before it, the same tile of the strip before it is
+// done and, for a segment's first tile, the segment before it is done.
+static double strip_pipeline_steps(int nPC, int nS, int nT, int slots, int nSeg) {
+    const int L = nT / nSeg;
+    std::vector<double> fin((size_t)nPC * nS * nT, 0.0);           // finish time of every tile
+    std::priority_queue<double, std::vector<double>, std::greater<double>> free;
+    for (int i = 0; i < slots; ++i) free.push(0.0);
+    double end = 0.0;
+    for (int key = 0; key < nS + (nSeg - 1) * L; ++key)
+        for (int g = 0; g < nSeg; ++g) {
+            const int s_ = key - g * L;
+            if (s_ < 0 || s_ >= nS) continue;
+            const int j0 = g * L, j1 = g == nSeg - 1 ? nT : j0 + L;
+            for (int pc = 0; pc < nPC; ++pc) {
+                double t = free.top();
+                free.pop();
+                double *row = &fin[((size_t)pc * nS + s_) * nT];
+                const double *prev = s_ > 0 ? row - nT : nullptr;
+                if (g > 0 && row[j0 - 1] > t) t = row[j0 - 1];
+                for (int j = j0; j < j1; ++j) {
+                    if (prev && prev[j] > t) t = prev[j];
+                    t += 1.0;
+                    row[j] = t;
+                }
+                free.push(t);
+                if (t > end) end = t;
+            }
+        }
+    return end;
+}
+static std::atomic<int> g_strip_slots{0};           // test hook: block slots the model assumes (0: the machine's)
+int strip_segments(int64_t nPlaneChunks, int nStrips, int nTilesX, int64_t slots, int nQueues) {
+    if (const int forced = g_strip_slots.load(std::memory_order_relaxed)) {
+        if (forced < 0) return nQueues == 1 && nStrips >= 2 ? std::max(1, std::min(-forced, nTilesX / 2)) : 1;   // that many segments
+        slots = forced;
+    }
+    if (nQueues != 1 || nStrips < 2 || nTilesX < 8 || nPlaneChunks * nStrips <= slots ||
+        nPlaneChunks * nStrips * nTilesX > ((int64_t)1 << 21))
+        return 1;
+    static std::mutex m;
+    static std::map<std::tuple<int64_t, int, int, int64_t>, int> cache;
+    const auto key = std::make_tuple(nPlaneChunks, nStrips, nTilesX, slots);
+    std::lock_guard<std::mutex> lock(m);
+    const auto it = cache.find(key);
+    if (it != cache.end()) return it->second;
+    int best = 1;
+    const double whole = strip_pipeline_steps((int)nPlaneChunks, nStrips, nTilesX, (int)slots, 1);
+    double best_cost = whole;
+    for (int nSeg = 2; nSeg <= 4 && nTilesX / nSeg >= 4; ++nSeg) {
+        const double cost = strip_pipeline_steps((int)nPlaneChunks, nStrips, nTilesX, (int)slots, nSeg) * (1.0 + 0.02 * (nSeg - 1));
+        if (cost < best_cost && cost < whole * 0.92) { best = nSeg; best_cost = cost; }
+    }
+    cache[key] = best;
+    return best;
+}
 
 // Set-up of the current device: done once, by whichever of snd_init() and the first launch comes first.
 int ensure_device_ready() {
@@ -212,6 +275,9 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);   // (tile layout: Wp = nCX * 8)
     plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
+    // and, where the backward's strips are cut into column segments, one carried column state per strip
+    if (snd::strip_segments(plane_chunks(*shape), g.nCY, g.nCX, snd::bwd_slots(shape->dstate), snd::job_queues(shape->batch * shape->n_groups)) > 1)
+        plan->bwd_workspace_bytes += plane_chunks(*shape) * g.nCY * (int64_t)snd::kColStateFloats * (int64_t)sizeof(float);
     const int fwd_jobs = snd::fwd_band_count(SND_SCHED_AUTO, (int64_t)shape->batch * shape->n_groups,
                                              (shape->dim / shape->n_groups + 15) / 16, g.nCY, plan, shape->dstate, g.nCX);
     plan->auto_schedule = fwd_jobs == 0 ? SND_SCHED_PLANE : fwd_jobs == g.nCY ? SND_SCHED_STRIPS : SND_SCHED_BANDS;
@@ -346,6 +412,8 @@ int snd_workspace_error(const void *workspace, snd_stream_t stream) {
     if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return SND_ERR_LAUNCH;
     return word != 0 ? SND_ERR_PIPELINE : SND_OK;
 }
+
+void snd_debug_set_strip_slots(int slots) { snd::g_strip_slots.store(slots, std::memory_order_relaxed); }
 
 void snd_debug_set_spin_limit(int polls) { snd::g_spin_limit.store(polls > 0 ? polls : snd::kSpinLimit, std::memory_order_relaxed); }
 

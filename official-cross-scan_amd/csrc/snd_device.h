@@ -39,6 +39,7 @@ struct Geo {
     int nBands;                    // pipelined schedules: jobs per plane chunk (set by the launcher)
     int nQueues;                   // and the number of job queues: 8 (one per XCD) or 1
     int spinLimit;                 // polls a hand-over wait makes before it gives up (set by the launcher)
+    int nSeg, segTiles;            // (backward, one strip per job) column segments per strip and tiles per segment
 };
 __host__ __device__ inline Geo make_geo(int H, int W) {
     const long long c8 = (long long)((H + 7) / 8) * ((W + 7) / 8) * 64, c7 = (long long)((H + 6) / 7) * ((W + 6) / 7) * 49;
@@ -51,6 +52,8 @@ __host__ __device__ inline Geo make_geo(int H, int W) {
     g.nBands = 0;
     g.nQueues = 1;
     g.spinLimit = 1 << 21;
+    g.nSeg = 1;
+    g.segTiles = g.nCX;
     g.tag = nullptr;
     return g;
 }
@@ -271,7 +274,8 @@ __host__ inline int xcd_grid(int nPairs, int nChunks) { return ((nPairs + 7) / 8
 // job waits for always holds an earlier ticket and is already running or finished.
 // Sync words (int32, zeroed before the launch): [1] error flag, [4..11] ticket counters (one per job
 // queue), [12 + plane chunk * strips + strip] count of tiles whose hand-over row the strip's block has
-// written.
+// written, and after those, in the same order, the count of column segments of the strip that are finished
+// (backward with column-segmented strips, see strip_segments).
 #ifndef SND_POLL_SLEEP
 #define SND_POLL_SLEEP 16                           // s_sleep units (64 cycles) between polls
 #endif
@@ -289,10 +293,11 @@ __host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips)
 #define SND_TILE_ABLATE 0
 #endif
 
+    // per (plane chunk, strip): tiles handed over, then column segments finished
 #ifdef SND_PIPE_TRACE   // timing study only: 4 extra words per job (start, end, time spent waiting, -)
-    return (kSyncHeader + 5 * nPlaneChunks * nStrips + 3) / 4 * 4;
+    return (kSyncHeader + 6 * nPlaneChunks * nStrips + 3) / 4 * 4;
 #else
-    return (kSyncHeader + nPlaneChunks * nStrips + 3) / 4 * 4;
+    return (kSyncHeader + 2 * nPlaneChunks * nStrips + 3) / 4 * 4;
 #endif
 }
 
@@ -372,25 +377,47 @@ __device__ __forceinline__ void strip_wait(const int *count, int need, int &seen
 // holding the pairs congruent to it, so that all chunks and bands of a pair - they stream the same B/C
 // planes - run on one XCD as in the whole-plane schedule; a block whose own queue is empty takes from
 // the next one.  Returns false when no job is left (every block makes at most nQueues draws).
+// With column segments (nSeg > 1; one strip per band, one queue) a job is (plane chunk, strip, segment) and the
+// tickets run in the order of the earliest step a job can start at, strip + segment * segTiles (strips and segments
+// counted in the order they are walked): both jobs a job waits for - the same segment of the strip before it and
+// the segment before it of its own strip - have a smaller key, hence an earlier ticket.
 __device__ __forceinline__ bool draw_job(int *sync, int nPairs, int nChunks, int nBands, int nQ, int &pair, int &chunk,
-                                         int &band) {
-    __shared__ int sJob[2];
+                                         int &band, int nSeg = 1, int segTiles = 0, int *seg = nullptr) {
+    __shared__ int sJob[3];
     if (threadIdx.x == 0) {
         int q = blockIdx.x & (nQ - 1), t = -1;
         for (int k = 0; k < nQ; ++k) {
-            const int jobs = ((nPairs - q + nQ - 1) / nQ) * nChunks * nBands;
+            const int jobs = ((nPairs - q + nQ - 1) / nQ) * nChunks * nBands * nSeg;
             if (jobs > 0) {
                 const int got = __hip_atomic_fetch_add(sync + kTicketWord + q, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (got < jobs) { t = got; break; }
             }
             q = (q + 1) & (nQ - 1);
         }
+        int sg = 0;
+        if (nSeg > 1 && t >= 0) {                   // ticket -> (key, segment, plane chunk); the band follows from the key
+            const int per = ((nPairs - q + nQ - 1) / nQ) * nChunks;
+            int rem = t, key = 0;
+            for (;; ++key) {
+                int cnt = 0;
+                for (int g = 0; g < nSeg; ++g) cnt += (key - g * segTiles >= 0 && key - g * segTiles < nBands);
+                if (rem < cnt * per) break;
+                rem -= cnt * per;
+            }
+            int gi = rem / per;
+            rem -= gi * per;
+            for (sg = 0; sg < nSeg; ++sg)
+                if (key - sg * segTiles >= 0 && key - sg * segTiles < nBands && gi-- == 0) break;
+            t = (key - sg * segTiles) * per + rem;  // the ticket this (band, plane chunk) has without segments
+        }
         sJob[0] = t;
         sJob[1] = q;
+        sJob[2] = sg;
     }
     __syncthreads();
     const int t = sJob[0], q = sJob[1];
     if (t < 0) return false;
+    if (seg) *seg = sJob[2];
     const int per_band = ((nPairs - q + nQ - 1) / nQ) * nChunks;
     band = t / per_band;
     const int r = t - band * per_band;
@@ -399,6 +426,17 @@ __device__ __forceinline__ bool draw_job(int *sync, int nPairs, int nChunks, int
     return true;
 }
 __host__ inline int job_queues(int nPairs) { return nPairs >= 16 ? 8 : 1; }
+// Column segments per strip of the backward's strip pipeline (1 = whole strips).  A block that has drawn a strip
+// holds its slot while it waits for the strip before it, so with more strip jobs than block slots the last strips of
+// every plane start late (2 x 192 channels of 200 x 336: 600 strips of 42 tiles on 512 slots take 87 tile steps where
+// the work is 49 and the chain of one plane 66).  Cut into segments of fewer tiles - the carried column state goes
+// from one segment's block to the next through the workspace - the same jobs pack into 70 steps.  Decided by running
+// the ticket order through a list-scheduling model (unit tile time, `slots` blocks at once; cached per shape):
+// segments are taken where the model gains at least 8 %.  (256 channels of 512 x 512: 159 steps either way.)
+int strip_segments(int64_t nPlaneChunks, int nStrips, int nTilesX, int64_t slots, int nQueues);
+// floats of one strip's carried column state in the workspace (G, Gs, a of eight rows and the corner G per lane of a
+// 256-thread block, as 8-byte words of all lanes one after the other)
+constexpr int kColStateFloats = 13 * 2 * 256;
 // Enqueue a fill kernel that zeroes n int32 words (defined with the C entry points).
 int zero_words(int *p, int64_t n, hipStream_t stream);
 // Per-device set-up (kernel attributes, the address of the static scratch array), done by snd_init() or

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
         (void)nPC;
         progress = sync + kSyncHeader + pc * geo.nCY;
 #ifdef SND_PIPE_TRACE
-        trace_ = sync + kSyncHeader + nPC * geo.nCY + 4 * (pc * geo.nCY + I_begin);
+        trace_ = sync + kSyncHeader + 2 * nPC * geo.nCY + 4 * (pc * geo.nCY + I_begin);
         if (threadIdx.x == 0) trace_[0] = (int)wall_clock64();
 #endif
     } else if (!xcd_job(blockIdx.x, sh.batch * G, nChunks, pair, chunk)) return;

@@ -77,6 +77,8 @@ def lib():
         _lib.snd_workspace_error.argtypes = [vp, vp]
         _lib.snd_debug_set_spin_limit.argtypes = [C.c_int]
         _lib.snd_debug_set_spin_limit.restype = None
+        _lib.snd_debug_set_strip_slots.argtypes = [C.c_int]
+        _lib.snd_debug_set_strip_slots.restype = None
     return _lib
 
 

@@ -99,3 +99,51 @@ def test_strips_need_workspace(gpu_device):
     assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -6
     f.params.workspace, f.params.workspace_bytes = f.ws.data_ptr(), 8
     assert capi.lib().snd_fwd(capi.C.byref(f.params), torch.cuda.current_stream().cuda_stream) == -6
+
+
+@pytest.mark.parametrize("Bt,Dm,H,W,N,K,dtype,slots", [
+    (1, 32, 100, 70, 16, 4, torch.float32, -2),       # 4 plane chunks x 13 strips x 9 tiles, two segments (4 + 5 tiles)
+    (2, 48, 61, 131, 16, 2, torch.float32, -3),       # ragged strips and tiles, partial channel chunks (24 = 16 + 8), 17 tiles in three segments
+    (1, 16, 200, 96, 12, 1, torch.bfloat16, -4),      # one plane chunk, 25 strips x 12 tiles, vector staging of 16-bit inputs
+    (1, 64, 90, 133, 16, 4, torch.float16, -2),       # unaligned rows (element-wise staging)
+    (1, 8, 40, 21, 16, 2, torch.float32, -8),         # 7x7 tiles, three tiles: one segment of two tiles is all that fits
+])
+def test_column_segmented_strips(gpu_device, Bt, Dm, H, W, N, K, dtype, slots):
+    """The backward's strips cut into column segments (taken where there are more strip jobs than block slots; here
+    forced through the test hook): bit-identical du / ddelta to whole strips and to whole planes, sums to
+    rounding, everything against the float64 oracle."""
+    print("column segments", Bt, Dm, H, W, N, K, dtype, slots, flush=True)
+    lib = capi.lib()
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=21)
+    t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+    for k in ("u", "delta", "B", "C"):
+        t[k] = t[k].to(dtype)
+    args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+    f = capi.FwdCall(*args, True, True, None, True, capi.SCHED_PLANE)
+    f.launch()
+    res = {}
+    try:
+        for name, sched, sl in (("plane", capi.SCHED_PLANE, 0), ("strips", capi.SCHED_STRIPS, 0), ("segments", capi.SCHED_STRIPS, slots)):
+            lib.snd_debug_set_strip_slots(sl)
+            b = capi.BwdCall(*args, t["dout"], f.x, f.x_v, True, None, f.x_sd, sched)
+            if name == "segments":
+                st, plan = capi.make_plan(capi.make_shape(t["u"], t["delta"], t["A"], t["B"]))
+                assert (plan.bwd_workspace_bytes > plan.fwd_workspace_bytes) == (plan.n_chunks_x >= 4), "this shape was meant to take column segments"
+            b.ws.view(torch.int32)[:16] = 0x7fffffff
+            b.launch()
+            torch.cuda.synchronize()
+            if sched != capi.SCHED_PLANE:
+                assert sync_error(b.ws) == 0, "a wait ran into its poll limit"
+            res[name] = [b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias]
+    finally:
+        lib.snd_debug_set_strip_slots(0)
+    for name in ("strips", "segments"):
+        assert torch.equal(res["plane"][0], res[name][0]) and torch.equal(res["plane"][1], res[name][1]), name
+        for nm, a, b_ in zip(NAMES[2:], res["plane"][2:], res[name][2:]):
+            assert relerr(a.float().cpu().numpy(), b_.float().cpu().numpy()) <= 1e-5, (name, nm)
+    r = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    gref = OC.bwd(r["u"], r["delta"], d["A"], r["B"], r["C"], d["D"], d["delta_bias"], d["dout"], True, None, real="f64")
+    half = dtype != torch.float32
+    for nm, a, b_ in zip(NAMES, res["segments"], gref):
+        tol = 1e-2 if (half and nm in ("du", "ddelta", "dB", "dC")) else 1e-4
+        assert relerr(a.float().cpu().numpy(), b_) <= tol, (nm, relerr(a.float().cpu().numpy(), b_))

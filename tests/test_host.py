@@ -12,7 +12,7 @@ import capi
 def test_library_exports_every_declared_symbol():
     names = capi.declared_symbols()
     assert set(names) >= {"snd_version", "snd_status_string", "snd_make_plan", "snd_fwd", "snd_bwd", "snd_init",
-                          "snd_workspace_error", "snd_debug_set_spin_limit", "snd_bwd_static",
+                          "snd_workspace_error", "snd_debug_set_spin_limit", "snd_debug_set_strip_slots", "snd_bwd_static",
                           "snd_static_workspace_bytes"}
     lib = capi.lib()
     for n in names:
@@ -73,10 +73,10 @@ def test_plan_geometry(H, W, ncx, ncy):
     planes = 2 * 8 * 16
     assert plan.x_elems == planes * ncx * plan.x_inner == plan.x_sd_elems
     assert plan.x_v_elems == planes * ncy * plan.xv_inner
-    sync_words = (12 + 2 * 4 * 1 * ncy + 3) // 4 * 4        # header + (batch * groups * chunks) * strips
+    sync_words = (12 + 2 * (2 * 4 * 1 * ncy) + 3) // 4 * 4   # header + two counters per (batch * groups * chunks) * strips
     assert plan.fwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
     assert plan.auto_schedule == (capi.SCHED_STRIPS if ncy > 1 else capi.SCHED_PLANE)   # 8 plane chunks only
-    assert plan.bwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
+    assert plan.bwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4      # (8 plane chunks: no column segments)
 
 
 @pytest.mark.parametrize("shape,code", [
@@ -312,3 +312,16 @@ def test_packaging_names_match_the_reference():
     `selective_nd_scan_cuda_oflex` (:80)."""
     text = open(os.path.join(capi.ROOT, "setup.py")).read()
     assert 'name="selective_nd_scan"' in text and '"selective_nd_scan_cuda_oflex"' in text
+
+
+def test_plan_sizes_the_backward_workspace_for_column_segments():
+    """More strip jobs than the backward's block slots: the strips are cut into column segments, whose carried column
+    state (one slot of 13 x 2 x 256 floats per strip) the plan adds to the backward's workspace."""
+    st, plan = capi.make_plan(capi.Shape(2, 192, 200, 336, 16, 4, 192, capi.SND_F32))     # 24 plane chunks x 25 strips on 512 slots
+    assert st == 0 and plan.auto_schedule == capi.SCHED_STRIPS
+    planes, chunks = 2 * 192 * 16, 24
+    sync_words = (12 + 2 * chunks * 25 + 3) // 4 * 4
+    assert plan.fwd_workspace_bytes == sync_words * 4 + planes * plan.xv_inner * 4
+    assert plan.bwd_workspace_bytes == plan.fwd_workspace_bytes + chunks * 25 * 13 * 2 * 256 * 4
+    st, plan = capi.make_plan(capi.Shape(1, 256, 512, 512, 16, 4, 256, capi.SND_BF16))    # 1024 strips of 64 tiles: nothing to gain
+    assert st == 0 and plan.bwd_workspace_bytes == plan.fwd_workspace_bytes
