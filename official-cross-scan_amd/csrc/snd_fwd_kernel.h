@@ -26,12 +26,18 @@
 //   * a block either walks a whole plane or (PIPE) one strip of it, the strips of a plane running
 //     as a pipeline of blocks one tile apart (few, large planes).
 #pragma once
+#include <initializer_list>
 #include "snd_device.h"
 
 namespace snd {
 
-template <typename T, int NP, bool SAVE, bool PIPE, int TE>
+// VEC: the tile's inputs are staged four columns at a time, one 16-byte (fp32) or 8-byte (16-bit) load per thread and
+// tensor instead of one load per element: a quarter of the memory instructions and of their address arithmetic.
+// Needs 8x8 tiles, a width that is a multiple of four and tensors whose rows start on such boundaries (fwd_vec_ok).
+template <typename T, int NP, bool SAVE, bool PIPE, int TE, bool VEC = false>
 __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8 ? 3 : 2, 4))) void fwd_kernel(const snd_fwd_params p, const Geo geo) {
+    static_assert(!VEC || TE == 8, "vector staging needs 8x8 tiles");
+    constexpr int NCH = VEC ? kTile / 4 / NP : 1;   // (VEC) four-column chunks of a channel's tile per thread
     constexpr int WPB = NP / 4, NT = 16 * NP;      // waves / threads per block
     constexpr int CB = 16;                          // channels per block
     constexpr int NSTR = kTile + 4;                 // per-state pitch: lane n hits banks 4n..4n+3
@@ -50,13 +56,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     // The bu/4 term of the output, sum_n C*B*delta'*u/4, is delta'*u times a per-pixel sum that all
     // channels share: S/4 = sum_n B*C / 4 is built once per tile (per-wave partial sums at staging, added
     // up by one wave) instead of one multiply-add per state cell.
-    __shared__ float sSp[(NP / 4) * kTile], sS[kTile];
+    __shared__ __align__(16) float sSp[(NP / 4) * kTile], sS[kTile];
     // out of up to four consecutive tiles of a strip (two in the 8-state kernels, whose blocks have
     // less LDS each), flushed together: a 32-byte run per tile row is a partial line write (measured:
     // 13 % of the kernel for the 154 MB of out at B=64, D=192, 56x56), four tiles make whole lines
     constexpr int QT = NP == 16 ? 4 : 2, QC = QT * kCkX;
     constexpr int OROW = NP == 16 ? QC + 8 : QC, OCH = kRows * OROW + (NP == 16 ? 16 : 8);   // padded against bank conflicts
-    __shared__ float sOut[CB * OCH];
+    __shared__ __align__(16) float sOut[CB * OCH];
 
     const snd_shape &sh = p.shape;
     const int H = sh.nrows, W = sh.ncols, N = sh.dstate, Dm = sh.dim, G = sh.n_groups;
@@ -155,7 +161,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     // (Only where it pays and fits: the 16-state whole-plane kernels, which are bandwidth-bound.)
     constexpr bool PAIR = NP == 16;
     constexpr int NHL = (kCkX + NP - 1) / NP;       // halo-row elements per thread (1; 2 with four lanes per channel)
-    struct Stage { uint32_t qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; };   // raw: masked and converted at commit
+    struct StageE { uint32_t qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; };   // raw: masked and converted at commit
+    struct StageV { Raw4<T> vb, vc, vdl[NCH], vu[NCH]; uint32_t qhalo[NHL]; };       // (VEC) one chunk of B and C, NCH of delta and u
+    typedef typename std::conditional<VEC, StageV, StageE>::type Stage;
     Stage st0, st1;                                 // tile J uses st0 when J is even (or always), st1 when odd
     float qxv[kCkX], qcorner = 0.f;                 // h of the row above the next tile (from x_v)
     auto load_tile = [&](Stage &q, int I, int J) {
@@ -164,7 +172,24 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
         // they are a few integer ops per tile instead of dozens of registers kept live across the tile.
         SND_THREAD_MAPS(NP);
         // loads are always in bounds (clamped coordinates); commit() zeroes what lies outside the plane
-        {
+        if constexpr (VEC) {
+            // chunk c of a tile = row c / 2, columns 4 * (c % 2) .. + 3; under a mirrored column order the same four
+            // memory columns in reverse (the chunk then starts at the memory column of its last scan column)
+            auto chunk_off = [&](int c, int hB) {
+                const int row = min(r0 + (c >> 1), H - 1), col = min(j0 + (c & 1) * 4, W - 4);
+                return (uint32_t)mad24(mrow(row), hB, mcol(col + (fh ? 3 : 0)) * ESZ);
+            };
+            {
+                const int sn = min(t_ >> 4, N - 1), c = t_ & 15;
+                ldraw4_b(q.vb, (const T *)((const char *)Bb + sn * BsB), chunk_off(c, BhB));
+                ldraw4_b(q.vc, (const T *)((const char *)Cb + sn * CsB), chunk_off(c, ChB));
+            }
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                ldraw4_b(q.vdl[k], db, cDb + chunk_off(n + NP * k, DhB));
+                ldraw4_b(q.vu[k], ub, cUb + chunk_off(n + NP * k, UhB));
+            }
+        } else {
             const int row = r0 + pr, col = j0 + pj;
             const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
             const uint32_t ob = mad24(mr, BhB, mcB), oc = mad24(mr, ChB, mcB);
@@ -174,14 +199,14 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 q.qb[k] = ldraw_b((const T *)((const char *)Bb + sc * BsB), ob);
                 q.qc[k] = ldraw_b((const T *)((const char *)Cb + sc * CsB), oc);
             }
-        }
 #pragma unroll
-        for (int k = 0; k < NPX; ++k) {
-            const int pp = n + NP * k;
-            const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
-            const int mr = mrow(min(row, H - 1)), mcB = mcol(min(col, W - 1)) * ESZ;
-            q.qdl[k] = ldraw_b(db, cDb + mad24(mr, DhB, mcB));
-            q.qu[k] = ldraw_b(ub, cUb + mad24(mr, UhB, mcB));
+            for (int k = 0; k < NPX; ++k) {
+                const int pp = n + NP * k;
+                const int row_ = r0 + (pp >> 3), col_ = j0 + (pp & 7);
+                const int mr_ = mrow(min(row_, H - 1)), mcB_ = mcol(min(col_, W - 1)) * ESZ;
+                q.qdl[k] = ldraw_b(db, cDb + mad24(mr_, DhB, mcB_));
+                q.qu[k] = ldraw_b(ub, cUb + mad24(mr_, UhB, mcB_));
+            }
         }
 #pragma unroll
         for (int k = 0; k < NHL; ++k) {     // halo row r0-1 (needed for a[i-1,j] of the strip's first row)
@@ -225,9 +250,44 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     float dukeep[NPX];   // D*u of this thread's pixels, for the output phase
     auto commit = [&](const Stage &qr, int I, int J) {
         SND_THREAD_MAPS(NP);
-        struct { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX], qhalo[NHL]; } q;
+        const int r0 = I * TE, j0 = J * TE;
+        float dsp;
+        if constexpr (VEC) {
+            auto flip4 = [&](float (&v)[4]) {                     // memory order -> scan order under a mirrored column order
+                if (fh) { const float a0 = v[0], a1 = v[1]; v[0] = v[3]; v[1] = v[2]; v[2] = a1; v[3] = a0; }
+            };
+            {
+                const int sn = t_ >> 4, c = t_ & 15;
+                const bool ok = sn < N && r0 + (c >> 1) < H && j0 + (c & 1) * 4 < W;
+                float b4[4], c4[4];
+                raw4_to_f32(qr.vb, b4); raw4_to_f32(qr.vc, c4);
+                flip4(b4); flip4(c4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { b4[e] = ok ? b4[e] : 0.f; c4[e] = ok ? c4[e] : 0.f; }
+                *(float4 *)(sB + sn * NSTR + c * 4) = make_float4(b4[0], b4[1], b4[2], b4[3]);
+                *(float4 *)(sC + sn * NSTR + c * 4) = make_float4(c4[0], c4[1], c4[2], c4[3]);
+            }
+#pragma unroll
+            for (int k = 0; k < NCH; ++k) {
+                const int c = n + NP * k;
+                const bool ok = cvalid && r0 + (c >> 1) < H && j0 + (c & 1) * 4 < W;
+                float d4[4], u4[4], du4[4];
+                raw4_to_f32(qr.vdl[k], d4); raw4_to_f32(qr.vu[k], u4);
+                flip4(d4); flip4(u4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float raw = (ok ? d4[e] : 0.f) + bias;
+                    d4[e] = softplus ? softplus20(raw, dsp) : raw;
+                    u4[e] = ok ? u4[e] : 0.f;
+                    du4[e] = d4[e] * u4[e];
+                    dukeep[4 * k + e] = Dv * u4[e];
+                }
+                *(float4 *)(sDl + cl * DLP + kCkX + c * 4) = make_float4(d4[0], d4[1], d4[2], d4[3]);
+                *(float4 *)(sDu + cl * PCH + c * 4) = make_float4(du4[0], du4[1], du4[2], du4[3]);
+            }
+        } else {
+        struct { float qb[NBC], qc[NBC], qdl[NPX], qu[NPX]; } q;
         {   // to fp32; zero outside the plane, the tile (7 x 7 tiles) and the state / channel ranges
-            const int r0 = I * TE, j0 = J * TE;
             const bool in = pr < TE && pj < TE && r0 + pr < H && j0 + pj < W;
 #pragma unroll
             for (int k = 0; k < NBC; ++k) {
@@ -242,11 +302,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 q.qdl[k] = ok ? raw_to_f32((const T *)nullptr, qr.qdl[k]) : 0.f;
                 q.qu[k] = ok ? raw_to_f32((const T *)nullptr, qr.qu[k]) : 0.f;
             }
-#pragma unroll
-            for (int k = 0; k < NHL; ++k) {
-                const int hj = n + NP * k;
-                q.qhalo[k] = (hj < TE && cvalid && r0 > 0 && j0 + hj < W) ? raw_to_f32((const T *)nullptr, qr.qhalo[k]) : 0.f;
-            }
         }
 #pragma unroll
         for (int k = 0; k < NBC; ++k) {
@@ -260,7 +315,6 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             for (int k = 0; k < NBC; ++k) part = fmaf(q.qb[k], q.qc[k], part);
             sSp[wave * kTile + px] = part;
         }
-        float dsp;
 #pragma unroll
         for (int k = 0; k < NPX; ++k) {
             const int pp = n + NP * k;
@@ -270,11 +324,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             sDu[cl * PCH + pp] = dl * q.qu[k];
             dukeep[k] = Dv * q.qu[k];
         }
+        }
 #pragma unroll
         for (int k = 0; k < NHL; ++k) {
             const int hj = n + NP * k;
             if (hj < kCkX) {
-                const float raw = q.qhalo[k] + bias;
+                const float hv = (hj < TE && cvalid && r0 > 0 && j0 + hj < W) ? raw_to_f32((const T *)nullptr, qr.qhalo[k]) : 0.f;
+                const float raw = hv + bias;
                 sDl[cl * DLP + hj] = softplus ? softplus20(raw, dsp) : raw;
             }
         }
@@ -302,8 +358,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             __syncthreads();
             if (wave == 0) {                        // read by the output phase, behind the next barrier
                 float t = 0.f;
+                if (VEC) {                          // from the committed tile: sum_n B*C of the pixel
 #pragma unroll
-                for (int w = 0; w < WPB; ++w) t += sSp[w * kTile + (tid & 63)];
+                    for (int k = 0; k < NP; ++k) t = fmaf(sB[k * NSTR + (tid & 63)], sC[k * NSTR + (tid & 63)], t);
+                } else {
+#pragma unroll
+                    for (int w = 0; w < WPB; ++w) t += sSp[w * kTile + (tid & 63)];
+                }
                 sS[tid & 63] = 0.25f * t;
             }
             // row above this tile: fetched one tile ahead (taken before the next prefetch reuses the
@@ -427,7 +488,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 const uint32_t cOb = (uint32_t)(cc - mshift) * (uint32_t)p.out_d_stride * esz_out;
 #pragma unroll
                 for (int k = 0; k < NPX; ++k) {
-                    const int pp = n + NP * k;
+                    const int pp = VEC ? 4 * (n + NP * (k >> 2)) + (k & 3) : n + NP * k;
                     const int row = r0 + (pp >> 3), col = j0 + (pp & 7);
                     if (cvalid && (pp >> 3) < TE && (pp & 7) < TE && row < H && col < W && !(SND_TILE_ABLATE & 1)) {
                         const float v = fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
@@ -438,11 +499,22 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 }
                 return;
             }
+            if constexpr (VEC) {
+#pragma unroll
+                for (int k = 0; k < NCH; ++k) {
+                    const int pp = 4 * (n + NP * k);
+                    const float4 du4 = *(const float4 *)(sDu + cl * PCH + pp), s4 = *(const float4 *)(sS + pp), y4 = *(const float4 *)(sY + cl * PCH + pp);
+                    *(float4 *)(sOut + cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)) =
+                        make_float4(wm * fmaf(du4.x, s4.x, y4.x + dukeep[4 * k]), wm * fmaf(du4.y, s4.y, y4.y + dukeep[4 * k + 1]),
+                                    wm * fmaf(du4.z, s4.z, y4.z + dukeep[4 * k + 2]), wm * fmaf(du4.w, s4.w, y4.w + dukeep[4 * k + 3]));
+                }
+            } else {
 #pragma unroll
             for (int k = 0; k < NPX; ++k) {
                 const int pp = n + NP * k;
                 if ((pp >> 3) < TE && (pp & 7) < TE)
                     sOut[cl * OCH + (pp >> 3) * OROW + jq * TE + (pp & 7)] = wm * fmaf(sDu[cl * PCH + pp], sS[pp], sY[cl * PCH + pp] + dukeep[k]);
+            }
             }
             // the next commit() does not touch sY; its barrier orders these sY reads against the
             // next tile's sY writes, and the barrier above ordered this tile's LDS reads against it
@@ -480,7 +552,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
 #endif
 }
 
-template <typename T, int NP, int TE>
+template <typename T, int NP, int TE, bool VEC>
 static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int rg = sh.dim / sh.n_groups;
@@ -496,24 +568,47 @@ static int launch_fwd_te(const snd_fwd_params &p, const Geo &geo, hipStream_t st
         gs.nBands = bands;
         gs.nQueues = job_queues(sh.batch * sh.n_groups);
         if (p.x != nullptr)
-            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, true, TE, VEC>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
         else
-            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, true, TE, VEC>), dim3(grid), dim3(16 * NP), 0, stream, p, gs);
     } else {
         const int grid = xcd_grid(sh.batch * sh.n_groups, nChunks);
         if (p.x != nullptr)
-            hipLaunchKernelGGL((fwd_kernel<T, NP, true, false, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, true, false, TE, VEC>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
         else
-            hipLaunchKernelGGL((fwd_kernel<T, NP, false, false, TE>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
+            hipLaunchKernelGGL((fwd_kernel<T, NP, false, false, TE, VEC>), dim3(grid), dim3(16 * NP), 0, stream, p, geo);
     }
     return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
+// Whether a call can stage four columns per load (fwd_kernel's VEC): every row of u, delta, B and C must start on a
+// four-element boundary (16 bytes of fp32, 8 bytes of 16-bit values); a state's plane of B / C must lie within 2^31
+// bytes of the first (the state offset is per lane there).
+inline bool fwd_vec_ok(const snd_fwd_params &f) {
+    const snd_shape &sh = f.shape;
+    const int e = sh.in_dtype == SND_F32 ? 4 : 2;
+    if (sh.ncols % 4 != 0) return false;
+    auto ok = [&](const void *ptr, std::initializer_list<int64_t> strides) {
+        if (((uintptr_t)ptr & (uintptr_t)(4 * e - 1)) != 0) return false;
+        for (int64_t s : strides)
+            if (s % 4 != 0) return false;
+        return true;
+    };
+    const int64_t span = (int64_t)(sh.dstate - 1) * e;
+    if (span * f.B_dstate_stride + (int64_t)sh.nrows * f.B_h_stride * e >= ((int64_t)1 << 31) ||
+        span * f.C_dstate_stride + (int64_t)sh.nrows * f.C_h_stride * e >= ((int64_t)1 << 31))
+        return false;
+    return ok(f.u, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) && ok(f.delta, {f.delta_batch_stride, f.delta_d_stride, f.delta_h_stride}) &&
+           ok(f.B, {f.B_batch_stride, f.B_group_stride, f.B_dstate_stride, f.B_h_stride}) &&
+           ok(f.C, {f.C_batch_stride, f.C_group_stride, f.C_dstate_stride, f.C_h_stride});
 }
 
 template <typename T, int NP>
 static int launch_fwd_np(const snd_fwd_params &p, hipStream_t stream) {
     Geo geo = make_geo(p.shape.nrows, p.shape.ncols);
     geo.tag = state_tag(p.x_sd, p.shape);
-    return geo.te == 7 ? launch_fwd_te<T, NP, 7>(p, geo, stream) : launch_fwd_te<T, NP, 8>(p, geo, stream);
+    if (geo.te == 7) return launch_fwd_te<T, NP, 7, false>(p, geo, stream);
+    return fwd_vec_ok(p) ? launch_fwd_te<T, NP, 8, true>(p, geo, stream) : launch_fwd_te<T, NP, 8, false>(p, geo, stream);
 }
 
 // One instantiation per input dtype, each in its own translation unit.
