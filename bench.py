@@ -204,6 +204,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default=None, metavar="B,D,H,W,N,K,dtype",
+                    help="time another shape than the named workloads (same value distributions), e.g. 64,192,56,56,5,4,float32; "
+                         "no committed counters exist for such a shape, so the roofline objects carry the timed legs only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
                     help="kernel family and block mapping: chosen by shape (default), one block per plane chunk, "
@@ -221,6 +224,10 @@ def main():
 
     sched = {"auto": 0, "plane": 1, "strips": 2, "bands": 3, "wavefront": 4}[args.schedule]
     snd.set_schedule(sched)
+    if args.shape:
+        f_ = args.shape.split(",")
+        WORKLOADS["custom"] = tuple(int(v) for v in f_[:6]) + (f_[6],)
+        args.workload = "custom"
     Bt, Dm, H, W, N, K, dtn = WORKLOADS[args.workload]
     dtype = getattr(torch, dtn)
     u, delta, A, B, C, D, bias, dout = make_inputs(torch, Bt, Dm, H, W, N, K, dtype, dev)
@@ -286,7 +293,7 @@ def main():
 
     roof = leg("snd::wave_bwd_kernel" if wave else "snd::bwd_kernel", bb, kb_ms)
     roof_fwd = leg("snd::wave_fwd_kernel" if wave else "snd::fwd_kernel", fb, kf_ms)
-    pc = profile_counters(args.workload) if args.schedule == "auto" else None
+    pc = profile_counters(args.workload) if args.schedule == "auto" and not args.shape else None
     if pc:
         # counters from the committed profile of this workload, if it is a profile of these kernels: same kernel,
         # same sources, and durations that agree with the ones measured here
