@@ -90,6 +90,12 @@ typedef struct snd_plan {
      * measured at).  Results do not depend on placement, and no other pair of buffers shows the effect
      * (timed with dC moved step by step inside one large allocation). */
     int64_t dC_skew_bytes;
+    int32_t wavefront_workspace;               /* 1 if WAVEFRONT takes this shape's planes in column groups (rows of more
+                                                  than 512 columns; with one state and an even width, more than 1024):
+                                                  the groups hand over through memory - bwd then needs its workspace
+                                                  (bwd_workspace_bytes covers it), and a fwd that saves no state
+                                                  (x == NULL) needs fwd_workspace_bytes, or AUTO runs the tile kernels */
+    int32_t reserved_;
 } snd_plan;
 
 /* How a launch maps work to blocks.  The reference has one fixed mapping (one block per
@@ -101,9 +107,10 @@ typedef struct snd_plan {
  *           only at band ends.  For more plane chunks than the chip holds blocks at once (backward at B=64, D=192, 56x56, N=16:
  *           768 chunks, 512 slots), where whole-plane blocks leave the last round half empty.  Needs
  *           the workspace.
- *   WAVEFRONT  the second kernel family, for 1-4 states per channel and planes up to 512 columns wide: a
- *           block per (batch, channel), a wave per 64-column row segment, the segments of a plane advancing
- *           as an anti-diagonal wavefront (what AUTO picks whenever it applies).  Its saved state has a
+ *   WAVEFRONT  the second kernel family, for 1-4 states per channel: a block per (batch, channel), a wave
+ *           per 64-column row segment, the segments of a plane advancing as an anti-diagonal wavefront
+ *           (what AUTO picks whenever its timing model prefers it).  Planes of more than eight segments
+ *           are taken in column groups of eight, one launch per group (snd_plan.wavefront_workspace).  Its saved state has a
  *           layout of its own: fwd and bwd of one call pair must both run WAVEFRONT or both run one of the
  *           three tile schedules above (AUTO decides by shape alone, so AUTO on both sides always agrees). */
 typedef enum snd_schedule { SND_SCHED_AUTO = 0, SND_SCHED_PLANE = 1, SND_SCHED_STRIPS = 2, SND_SCHED_BANDS = 3, SND_SCHED_WAVEFRONT = 4 } snd_schedule;

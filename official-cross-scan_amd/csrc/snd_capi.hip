@@ -19,12 +19,12 @@ int launch_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
 int launch_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
 int launch_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
-int launch_wave_fwd_f32(const snd_fwd_params &p, hipStream_t stream);
-int launch_wave_fwd_bf16(const snd_fwd_params &p, hipStream_t stream);
-int launch_wave_fwd_f16(const snd_fwd_params &p, hipStream_t stream);
-int launch_wave_bwd_f32(const snd_bwd_params &p, hipStream_t stream);
-int launch_wave_bwd_bf16(const snd_bwd_params &p, hipStream_t stream);
-int launch_wave_bwd_f16(const snd_bwd_params &p, hipStream_t stream);
+int launch_wave_fwd_f32(const snd_fwd_params &p, float *group_ws, hipStream_t stream);
+int launch_wave_fwd_bf16(const snd_fwd_params &p, float *group_ws, hipStream_t stream);
+int launch_wave_fwd_f16(const snd_fwd_params &p, float *group_ws, hipStream_t stream);
+int launch_wave_bwd_f32(const snd_bwd_params &p, float *group_ws, hipStream_t stream);
+int launch_wave_bwd_bf16(const snd_bwd_params &p, float *group_ws, hipStream_t stream);
+int launch_wave_bwd_f16(const snd_bwd_params &p, float *group_ws, hipStream_t stream);
 int configure_bwd_f32();
 int configure_bwd_bf16();
 int configure_bwd_f16();
@@ -138,6 +138,12 @@ int64_t plane_chunks(const snd_shape &s) {
     return (int64_t)s.batch * s.n_groups * ((s.dim / s.n_groups + 15) / 16);
 }
 
+// Where the column groups of a wide plane (row-segment kernels) hand over inside a workspace: behind the sync words
+int64_t group_ws_offset(const snd_shape &s) {
+    const snd::Geo g = snd::make_geo(s.nrows, s.ncols);
+    return (snd::sync_words(plane_chunks(s), g.nCY) * (int64_t)sizeof(int) + 255) / 256 * 256;
+}
+
 int check_shape(const snd_shape &s) {
     if (s.batch <= 0 || s.dim <= 0 || s.nrows <= 0 || s.ncols <= 0 || s.dstate <= 0 || s.n_groups <= 0 ||
         s.delta_dim <= 0)
@@ -174,7 +180,8 @@ bool wave_family_pays(const snd_shape &s) {
     const bool shared = wg.nseg == 1 && waves >= 512;        // (wave_bwd_share() of the backward's launcher)
     const double t_row = pk == 8 ? (s.dstate <= 1 ? 0.75 : s.dstate == 2 ? 1.15 : 2.2) : pk > 1 ? (s.dstate <= 1 ? 0.65 : s.dstate == 2 ? 1.05 : 2.05)
                        : shared ? (s.dstate <= 1 ? 0.7 : s.dstate == 2 ? 1.15 : 2.4) : (s.dstate <= 1 ? 0.85 : s.dstate == 2 ? 1.5 : 2.95);
-    const double t_wave = (double)((waves + 2047) / 2048) * (wg.Hp + (wg.nseg - 1) * wg.R) * t_row;
+    // (a wide plane: one launch per column group of eight segments, one after the other)
+    const double t_wave = (double)snd::wave_groups(wg.nsegAll) * (double)((waves + 2047) / 2048) * (wg.Hp + (wg.nseg - 1) * wg.R) * t_row;
     const int64_t blocks = plane_chunks(s);
     const double t_plane = (double)((blocks + 1023) / 1024) * g.nCX * g.nCY * 18.5;
     const int64_t rounds = (blocks * g.nCY + 1023) / 1024;
@@ -185,7 +192,7 @@ bool wave_family_pays(const snd_shape &s) {
 }
 
 // Which kernel family a call runs: the row-segment wavefront when asked for, or under AUTO when the shape
-// qualifies (1-4 states, at most 512 columns) and the model above prefers it; the tile kernels otherwise.
+// qualifies (1-4 states) and the model above prefers it; the tile kernels otherwise.
 // -1: WAVEFRONT asked for a shape it does not cover.
 int use_wavefront(const snd_shape &s, int schedule) {
     const bool fits = snd::wave_family_fits(s.ncols, s.dstate);
@@ -275,6 +282,18 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     const int64_t row_bytes = planes * (int64_t)g.Wp * (int64_t)sizeof(float);   // (tile layout: Wp = nCX * 8)
     plan->fwd_workspace_bytes = sync_bytes + row_bytes;      // the strip schedule's hand-over row of h
     plan->bwd_workspace_bytes = sync_bytes + row_bytes;      // the adjoint row G = a*g
+    plan->wavefront_workspace = 0;
+    plan->reserved_ = 0;
+    if (wave && snd::wave_wide(shape->ncols, shape->dstate)) {
+        plan->wavefront_workspace = 1;
+        // wide planes under the row-segment kernels: what column groups hand over (behind the sync words, which stay
+        // the tile kernels'): forward without saved state, a stand-in for x and x_sd; backward, G, Gs, a per boundary
+        const snd::WaveGeo wg = snd::make_wave_geo(shape->nrows, shape->ncols, shape->dstate);
+        const int64_t off = group_ws_offset(*shape);
+        const int64_t fw = off + 2 * planes * snd::wave_x_plane(wg) * (int64_t)sizeof(float), bw = off + planes * snd::wave_bcol_plane(wg) * (int64_t)sizeof(float);
+        if (fw > plan->fwd_workspace_bytes) plan->fwd_workspace_bytes = fw;
+        if (bw > plan->bwd_workspace_bytes) plan->bwd_workspace_bytes = bw;
+    }
     // and, where the backward's strips are cut into column segments, one carried column state per strip
     if (snd::strip_segments(plane_chunks(*shape), g.nCY, g.nCX, snd::bwd_slots(shape->dstate), snd::job_queues(shape->batch * shape->n_groups)) > 1)
         plan->bwd_workspace_bytes += plane_chunks(*shape) * g.nCY * (int64_t)snd::kColStateFloats * (int64_t)sizeof(float);
@@ -309,13 +328,26 @@ int snd_fwd(const snd_fwd_params *params, snd_stream_t stream) {
         return SND_ERR_STRIDE;
     if (params->schedule < SND_SCHED_AUTO || params->schedule > SND_SCHED_WAVEFRONT) return SND_ERR_SHAPE;
     if (params->directions != SND_DIR_TOPLEFT && params->directions != SND_DIR_CORNERS) return SND_ERR_SHAPE;
-    const int wave = use_wavefront(params->shape, params->schedule);
+    int wave = use_wavefront(params->shape, params->schedule);
     if (wave < 0) return SND_ERR_SHAPE;
-    if (wave) {                                     // needs no workspace
+    float *group_ws = nullptr;
+    if (wave && snd::wave_wide(params->shape.ncols, params->shape.dstate)) {
+        // a wide plane's column groups hand over through the saved state, or without one through the workspace
+        snd_plan plan;
+        snd_make_plan(&params->shape, &plan);
+        if (params->workspace && params->workspace_bytes >= plan.fwd_workspace_bytes) {
+            if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+            group_ws = (float *)((char *)params->workspace + group_ws_offset(params->shape));
+        } else if (!params->x) {
+            if (params->schedule == SND_SCHED_WAVEFRONT) return SND_ERR_WORKSPACE;
+            wave = 0;                               // (AUTO: the tile kernels need neither)
+        }
+    }
+    if (wave) {                                     // (other planes need no workspace)
         switch (params->shape.in_dtype) {
-            case SND_F32: return snd::launch_wave_fwd_f32(*params, (hipStream_t)stream);
-            case SND_BF16: return snd::launch_wave_fwd_bf16(*params, (hipStream_t)stream);
-            default: return snd::launch_wave_fwd_f16(*params, (hipStream_t)stream);
+            case SND_F32: return snd::launch_wave_fwd_f32(*params, group_ws, (hipStream_t)stream);
+            case SND_BF16: return snd::launch_wave_fwd_bf16(*params, group_ws, (hipStream_t)stream);
+            default: return snd::launch_wave_fwd_f16(*params, group_ws, (hipStream_t)stream);
         }
     }
     if (params->workspace) {
@@ -354,11 +386,17 @@ static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
         return SND_ERR_STRIDE;
     const int wave = use_wavefront(params->f.shape, params->f.schedule);
     if (wave < 0) return SND_ERR_SHAPE;
-    if (wave) {                                     // needs no workspace
+    float *group_ws = nullptr;
+    if (wave && snd::wave_wide(params->f.shape.ncols, params->f.shape.dstate)) {   // a wide plane's column groups hand over here
+        if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
+        if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+        group_ws = (float *)((char *)params->workspace + group_ws_offset(params->f.shape));
+    }
+    if (wave) {                                     // (other planes need no workspace)
         switch (params->f.shape.in_dtype) {
-            case SND_F32: return snd::launch_wave_bwd_f32(*params, (hipStream_t)stream);
-            case SND_BF16: return snd::launch_wave_bwd_bf16(*params, (hipStream_t)stream);
-            default: return snd::launch_wave_bwd_f16(*params, (hipStream_t)stream);
+            case SND_F32: return snd::launch_wave_bwd_f32(*params, group_ws, (hipStream_t)stream);
+            case SND_BF16: return snd::launch_wave_bwd_bf16(*params, group_ws, (hipStream_t)stream);
+            default: return snd::launch_wave_bwd_f16(*params, group_ws, (hipStream_t)stream);
         }
     }
     if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
@@ -388,9 +426,10 @@ int snd_bwd_static(const snd_bwd_params *params, snd_stream_t stream) {
     snd_plan plan;
     int st = snd_make_plan(&params->f.shape, &plan);
     if (st != SND_OK) return st;
-    // (the row-segment kernels use no scratch at all: no size limit for them)
+    // (the row-segment kernels use no scratch at all, wide planes aside: no size limit for them)
     const int wave = use_wavefront(params->f.shape, params->f.schedule);
-    if (wave == 0 && plan.bwd_workspace_bytes > SND_STATIC_WORKSPACE_BYTES) return SND_ERR_TOO_LARGE;
+    const bool scratch = wave == 0 || snd::wave_wide(params->f.shape.ncols, params->f.shape.dstate);
+    if (scratch && plan.bwd_workspace_bytes > SND_STATIC_WORKSPACE_BYTES) return SND_ERR_TOO_LARGE;
     st = snd::ensure_device_ready();                // no allocation: symbol lookup and kernel attributes, once per device
     if (st != SND_OK) return st;
     void *ws = snd::device_scratch();

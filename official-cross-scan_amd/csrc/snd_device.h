@@ -538,7 +538,14 @@ __host__ inline int fwd_band_count(int schedule, int64_t nPairs, int nChunks, in
 // the next wave through a few LDS words per row.
 struct WaveGeo {
     float *tag;                    // the family tag's place in the saved state (state_tag), or null
-    int nseg;                      // row segments (waves per plane): ceil(W / (64 * cpl))
+    int nseg;                      // row segments a block of this launch works on (its waves per plane)
+    int nsegAll;                   // row segments of a plane: ceil(W / (64 * cpl)); more than kMaxSeg: a wide plane, whose
+                                   // segments are taken in column groups of at most kMaxSeg, one launch per group
+    int seg0;                      // first segment of this launch's column group
+    int extL, extR;                // whether a column group lies to the left / right of this launch's
+    float *colh, *cols;            // (wide planes, forward) where column groups hand over h, a and s: the saved state
+                                   // x, x_sd themselves, or a workspace of the same layout when no state is saved
+    float *bcol;                   // (wide planes, backward) G, Gs, a at the first column of every column group
     int R;                         // rows per band (wave_band_rows): row-checkpoint spacing = rows the backward holds in registers
     int nBands;                    // ceil(H / R)
     int Hp, Wp;                    // nBands * R, nseg * 64 * cpl / planes per wave
@@ -565,21 +572,31 @@ __host__ __device__ constexpr int wave_fwd_rows(int N) { return N <= 2 ? 4 : 2; 
 // cover a row.  Narrower rows keep one column per lane - measured at 256 planes of 512 x 512: the same forward
 // time and a 1.5 x slower backward with two, whose doubled per-lane state leaves one wave per SIMD.  Decided by
 // the shape alone, because the saved state's segment boundaries follow from it.
-__host__ __device__ inline int wave_cpl(int W, int N) { return (N <= 1 && W > kSeg * kMaxSeg && W % 2 == 0) ? 2 : 1; }
-__host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4 && W <= kSeg * kMaxSeg * wave_cpl(W, N); }
+// Rows wider still (wide planes) keep one column per lane: their segments are taken in column groups anyway.
+__host__ __device__ inline int wave_cpl(int W, int N) { return (N <= 1 && W > kSeg * kMaxSeg && W <= 2 * kSeg * kMaxSeg && W % 2 == 0) ? 2 : 1; }
+__host__ __device__ inline bool wave_family_fits(int W, int N) { return N <= 4; }
+// A wide plane: more row segments than a block has waves.  Its segments are taken in column groups of kMaxSeg, left to
+// right in the forward and right to left in the backward, one launch per group (the stream orders them); what crosses a
+// group boundary - h, s, a of the column on its left (forward), G, Gs, a of the column on its right (backward), per row
+// and state - goes through global memory instead of LDS.
+__host__ __device__ inline bool wave_wide(int W, int N) { return (W + kSeg * wave_cpl(W, N) - 1) / (kSeg * wave_cpl(W, N)) > kMaxSeg; }
+__host__ __device__ inline int wave_groups(int nsegAll) { return (nsegAll + kMaxSeg - 1) / kMaxSeg; }
 // Planes per wave: narrow planes (one segment, at most 32 / 16 / 7 columns) are packed two / four / eight to a wave,
 // plane q of a wave in lanes q*32.. / q*16.. / q*8.. (both kernels of a pair pack alike: the row checkpoints are as
 // wide as a plane's lanes).  With eight planes the first lane of a plane is a barrier lane (wave_scan3_pk) and its
 // columns are in lanes 1..7.
-__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nseg == 1 ? (W <= 7 ? 8 : W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
+__host__ __device__ inline int wave_pack(const WaveGeo &g, int W) { return g.cpl == 1 && g.nsegAll == 1 ? (W <= 7 ? 8 : W <= 16 ? 4 : W <= 32 ? 2 : 1) : 1; }
 __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     WaveGeo g;
     g.cpl = wave_cpl(W, N);
-    g.nseg = (W + kSeg * g.cpl - 1) / (kSeg * g.cpl);
+    g.nsegAll = (W + kSeg * g.cpl - 1) / (kSeg * g.cpl);
+    g.nseg = g.nsegAll < kMaxSeg ? g.nsegAll : kMaxSeg;
+    g.seg0 = 0; g.extL = g.extR = 0;
+    g.colh = g.cols = g.bcol = nullptr;
     g.R = wave_band_rows(N);
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
-    g.Wp = g.nseg * kSeg * g.cpl / wave_pack(g, W);   // (packed planes: a row checkpoint is the plane's own lanes wide)
+    g.Wp = g.nsegAll * kSeg * g.cpl / wave_pack(g, W);   // (packed planes: a row checkpoint is the plane's own lanes wide)
     g.rg = g.rd = 1; g.gshift = 0; g.xcd = 0;
     g.tag = nullptr;
     return g;
@@ -589,7 +606,10 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
 //   x_sd [segment w][2][Hp]   s at the same places (second half unused)
 //   x_v  [band][Wp]           h on the last row of every band (the backward recomputes a of that row from delta)
 typedef float wave_f2 __attribute__((ext_vector_type(2)));
-__host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nseg * 2 * g.Hp; }
+__host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int64_t)g.nsegAll * 2 * g.Hp; }
+// (wide planes, backward) the hand-over between column groups, per (batch, channel, state) plane:
+//   bcol [group q][3][Hp]   G, Gs, a at the first column of group q on every row (written by group q, read by group q-1)
+__host__ __device__ inline int64_t wave_bcol_plane(const WaveGeo &g) { return (int64_t)wave_groups(g.nsegAll) * 3 * g.Hp; }
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all

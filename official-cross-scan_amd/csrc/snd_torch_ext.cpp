@@ -272,8 +272,8 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     at::Tensor dmerge;                              // weight * d(weight) per channel (the caller divides)
     if (merge) dmerge = accP.narrow(0, oMerge, dim);
     const int sched = resolve_schedule(schedule);
-    at::Tensor ws;                                  // the wavefront kernels need none
-    if (!wavefront(sched, c.plan)) ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
+    at::Tensor ws;                                  // the wavefront kernels need none, except for planes taken in column groups
+    if (!wavefront(sched, c.plan) || c.plan.wavefront_workspace) ws = torch::empty({(c.plan.bwd_workspace_bytes + 3) / 4}, f32);
 
     snd_bwd_params p;
     memset(&p, 0, sizeof(p));

@@ -55,9 +55,15 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 // then holds CHB * PK channels, and the planes of a wave are added up with the waves of the block.
 //
 // XW: the most waves a block may have, 8 or (two channels of five to eight segments) 16.
-template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW>
+//
+// EXT: the launch works on one column group of a wide plane (wave_wide() in snd_device.h), segments seg0 .. seg0+nseg-1;
+// the groups are launched right to left.  The group's last wave takes G, Gs, a of the column on its right from global
+// memory (with the band's loads, three values per state and row spread over the lanes of one register), where the
+// first wave of the group on the right left them.
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW, bool EXT = false>
 __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = wave_band_rows(NS);            // rows per band
+    static_assert(!EXT || (CHB == 1 && PK == 1 && CPL == 1 && !EVEN), "column groups: one channel per block, one column per lane");
     static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
     static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
     constexpr int S = 64 / PK;                       // lanes per plane
@@ -84,6 +90,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const int lane = threadIdx.x & 63, wi = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int kc = CHB > 1 ? wi / nseg : 0, w = PK > 1 ? 0 : wi - kc * nseg;     // channel of the block, segment of the channel
     const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
+    const int sg = EXT ? wg.seg0 + w : w;            // this wave's segment of the plane
     int pair, chunk;
     if (!wave_job2(wg, sh.batch * G, pair, chunk)) return;
     chunk = (chunk * CHB + kc) * PK + (PK > 1 ? lane / S : 0);       // (packed: a lane's own from here on)
@@ -106,11 +113,11 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     // Mirrored order: this lane owns scan columns jm0 .. jm0+CPL-1 and walks them downwards (its local index t is
     // scan column jm0 + CPL-1-t); in natural order (row checkpoints, recomputation) lane l owns columns jn0 ...
     const bool bar = PK == 8 && sl == 0;             // (eight planes per wave) the plane's barrier lane: mirrored column 7
-    const int jm0 = PK > 1 ? S - 1 - sl : (w * kSeg + 63 - lane) * CPL;
+    const int jm0 = PK > 1 ? S - 1 - sl : (sg * kSeg + 63 - lane) * CPL;
     const bool jin = EVEN || jm0 < W;
     const int jc = jin ? jm0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
-    const int jn0 = PK == 8 ? max(sl - 1, 0) : (w * kSeg + sl) * CPL;
+    const int jn0 = PK == 8 ? max(sl - 1, 0) : (sg * kSeg + sl) * CPL;
     // the mirror lane inside the plane (eight planes: lanes 1..7 among themselves, the barrier lane stays)
     const int rev_addr = PK == 8 ? ((lane - sl) + (sl == 0 ? 0 : 8 - sl)) * 4 : PK > 1 ? ((lane - sl) + S - 1 - sl) * 4 : (63 - lane) * 4;
     auto mirror = [&](float v) {
@@ -161,8 +168,15 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     // saved state of this plane set (layouts in snd_device.h)
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
     const float *xv = f.x_v + plane0 * wave_xv_plane(wg) + jn0;
-    const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
-    const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp;
+    const float *xh = f.x + plane0 * wave_x_plane(wg) + (int64_t)sg * 2 * wg.Hp;
+    const float *xs = f.x_sd + plane0 * wave_x_plane(wg) + (int64_t)sg * 2 * wg.Hp;
+    // (column groups) lane (q*NS + n)*R + r fetches G (q = 0), Gs (1), a (2) of the group on the right: row r of a band, state n
+    constexpr int kExtLanes = 3 * NS * R;
+    const int el = lane < kExtLanes ? lane : 0, eq = el / (NS * R), er = el % R, gq = EXT ? wg.seg0 / kMaxSeg : 0;
+    const float *ebase = EXT ? wg.bcol + (plane0 + (el / R) % NS) * wave_bcol_plane(wg)
+                               + (int64_t)min(gq + 1, wave_groups(wg.nsegAll) - 1) * 3 * wg.Hp + eq * wg.Hp : nullptr;
+    float *eout = EXT ? wg.bcol + plane0 * wave_bcol_plane(wg) + (int64_t)gq * 3 * wg.Hp : nullptr;
+    const bool ext_in = EXT && wg.extR && w == nseg - 1, ext_out = EXT && wg.extL && w == 0;
 
     // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
     // last columns (always in bounds) and only their dout is masked to zero where it is used, which makes every
@@ -171,7 +185,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     // the segment from the left on rows i0-1 .. i0+R-1, one row per lane.
     typedef WaveRaw<T, CPL, VEC> Raw;
     typedef WaveRaw<DoT, CPL, VEC> RawO;
-    struct In { Raw u[R], d[R], b[R][NS], c[R][NS]; RawO o[R]; Raw dtop; float h0[NS][CPL], ch[NS], cs[NS], ca[NS]; };
+    struct In { Raw u[R], d[R], b[R][NS], c[R][NS]; RawO o[R]; Raw dtop; float h0[NS][CPL], ch[NS], cs[NS], ca[NS], e; };
     // Every band issues the same loads on every path (the wait counters the compiler derives for the prefetch
     // need that): rows past the end of a ragged last band read the last row again and are never used.
     auto load_band = [&](In &q, int band) {
@@ -213,7 +227,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                     for (int k = 0; k < CPL; ++k)
                         if (PK == 8) q.h0[n][k] = bar ? 0.f : q.h0[n][k];
                 }
-                if (w > 0 && lane <= R && row >= 0) {
+                if (sg > 0 && lane <= R && row >= 0) {
                     const int64_t o = (int64_t)n * wave_x_plane(wg) + row;
                     q.ch[n] = xh[o];
                     q.ca[n] = xh[o + wg.Hp];
@@ -221,6 +235,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                 }
             }
         }
+        if (EXT) q.e = ebase[i0 + er];               // (by every wave, like the other loads; only the group's last wave uses it)
     };
     // the lane's CPL values in its walking order t (element e of the raw bits is t = CPL-1-e, or t = e when fh)
     auto unpack = [&](const auto &q, float (&v)[CPL]) {
@@ -371,7 +386,8 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
-                    const float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
+                    float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
+                    if (EXT && ext_in) in = make_float4(bcast(cur.e, n * R + r), bcast(cur.e, (NS + n) * R + r), bcast(cur.e, (2 * NS + n) * R + r), 0.f);
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
                     unpack(cur.b[r][n], Bv);
@@ -429,6 +445,12 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) { Gd[n][t] = Gt[t]; ad[n][t] = a[t]; }
                     if (hands_over && lane == 63) sHO[step & 1][kc][w][r][n] = make_float4(Gt[CPL - 1], Gst[CPL - 1], a[CPL - 1], 0.f);
+                    if (EXT && ext_out && lane == 63) {   // for the column group on the left
+                        float *d = eout + (int64_t)n * wave_bcol_plane(wg) + i0 + r;
+                        d[0] = Gt[CPL - 1];
+                        d[wg.Hp] = Gst[CPL - 1];
+                        d[2 * wg.Hp] = a[CPL - 1];
+                    }
                 }
                 if (jin) {
                     float duv[CPL], ddl[CPL];
@@ -578,14 +600,39 @@ static int launch_wave_bwd_v(const snd_bwd_params &p, const WaveGeo &wg, hipStre
     return launch_wave_bwd_c<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
 }
 
+// One launch per column group of a wide plane, right to left (the stream orders them).
+template <typename T, int NS>
+static int launch_wave_bwd_wide(const snd_bwd_params &p, WaveGeo wg, float *group_ws, hipStream_t stream) {
+    const snd_shape &sh = p.f.shape;
+    constexpr bool F32 = std::is_same<T, float>::value;
+    if (!group_ws) return SND_ERR_WORKSPACE;
+    wg.bcol = group_ws;
+    const dim3 grid = wave_grid2(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    const int groups = wave_groups(wg.nsegAll);
+    for (int q = groups - 1; q >= 0; --q) {
+        wg.seg0 = q * kMaxSeg;
+        wg.nseg = min(kMaxSeg, wg.nsegAll - wg.seg0);
+        wg.extL = q > 0;
+        wg.extR = q + 1 < groups;
+        const dim3 block(64 * wg.nseg);
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, NS, 1, true, true, false, 1, 1, kMaxSeg, true>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, NS, 1, true, F32, false, 1, 1, kMaxSeg, true>), grid, block, 0, stream, p, wg);
+        if (hipGetLastError() != hipSuccess) return SND_ERR_LAUNCH;
+    }
+    return SND_OK;
+}
+
 template <typename T>
-int launch_wave_bwd_t(const snd_bwd_params &p, hipStream_t stream) {
+int launch_wave_bwd_t(const snd_bwd_params &p, float *group_ws, hipStream_t stream) {
     const snd_fwd_params &f = p.f;
     const snd_shape &sh = f.shape;
     const int N = sh.dstate;
     WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
     wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
     wg.tag = state_tag(p.f.x_sd, sh);
+    if (wg.nsegAll > kMaxSeg)
+        return N == 1 ? launch_wave_bwd_wide<T, 1>(p, wg, group_ws, stream) : N == 2 ? launch_wave_bwd_wide<T, 2>(p, wg, group_ws, stream)
+             : N == 3 ? launch_wave_bwd_wide<T, 3>(p, wg, group_ws, stream) : launch_wave_bwd_wide<T, 4>(p, wg, group_ws, stream);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.dout_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned_b(f.u, e, 2 * e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&

@@ -45,9 +45,15 @@ namespace snd {
 // block is kOneWaves independent waves, each with a channel (PK channels) of its own, a quarter of the blocks to hand
 // out (measured against blocks of one wave, bf16, one state: 64 x 1536 x 14x14 0.055 -> 0.049 ms, 64 x 768 x 14x14
 // 0.035 -> 0.031, 64 x 3072 x 7x7 unchanged at 0.051).
-template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU, bool ONE>
+// EXT: the launch works on one column group of a wide plane (wave_wide() in snd_device.h): segments seg0 .. seg0+nseg-1.
+// The group's first wave takes what enters it on every row - h, s, a of the column on its left - from global memory,
+// where the launch of the group on the left put them (a band's values come with the band's loads, three per state and
+// row spread over the lanes of one register), and the group's last wave leaves the same for the group on its right.
+// The places are those of the column checkpoints the backward reads anyway (x, x_sd of segment seg0 and seg0+nseg).
+template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU, bool ONE, bool EXT = false>
 __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
     static_assert(ONE || PK == 1, "packed planes are one segment wide");
+    static_assert(!EXT || (!ONE && PK == 1 && CPL == 1), "column groups: whole segments, one column per lane");
     constexpr int R = wave_fwd_rows(NS);             // rows per band of this kernel = rows per load group
     constexpr int RC = wave_band_rows(NS);           // spacing of the row checkpoints (the backward's bands)
     static_assert(R % RC == 0, "a band ends on a checkpoint row");
@@ -93,7 +99,8 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
     const bool fv = p.directions == SND_DIR_CORNERS && (g & 2), fh = p.directions == SND_DIR_CORNERS && (g & 1);
     const int r0m = fv ? H - 1 : 0, rs = fv ? -1 : 1;
     const bool bar = PK == 8 && sl == 0;             // (eight planes per wave) the plane's barrier lane
-    const int j0 = PK == 8 ? max(sl - 1, 0) : (w * kSeg + sl) * CPL;   // this lane's first scan column
+    const int sg = EXT ? wg.seg0 + w : w;            // this wave's segment of the plane
+    const int j0 = PK == 8 ? max(sl - 1, 0) : (sg * kSeg + sl) * CPL;   // this lane's first scan column
     const bool jin = j0 < W && !bar;                 // (W is a multiple of CPL: a lane is inside or outside as a whole)
     const int jc = jin ? j0 : W - CPL;
     const int mc = fh ? W - CPL - jc : jc;           // memory column of the lane's lowest address
@@ -130,13 +137,21 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
     // saved state of this plane set
     const int64_t plane0 = ((int64_t)b * Dm + c) * N;
     float *xv = p.x_v + plane0 * wave_xv_plane(wg) + j0;
-    float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
-    float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)w * 2 * wg.Hp : nullptr;
+    float *xh = SAVE ? p.x + plane0 * wave_x_plane(wg) + (int64_t)sg * 2 * wg.Hp : nullptr;
+    float *xs = SAVE ? p.x_sd + plane0 * wave_x_plane(wg) + (int64_t)sg * 2 * wg.Hp : nullptr;
+    // (column groups) lane (q*NS + n)*R + r fetches h (q = 0), s (1), a (2) entering segment sg on row r of a band, state n
+    constexpr int kExtLanes = 3 * NS * wave_fwd_rows(NS);
+    const int el = lane < kExtLanes ? lane : 0, eq = el / (NS * wave_fwd_rows(NS)), er = el % wave_fwd_rows(NS);
+    const float *ebase = EXT ? (eq == 1 ? wg.cols : wg.colh) + (plane0 + (el / wave_fwd_rows(NS)) % NS) * wave_x_plane(wg)
+                               + (int64_t)sg * 2 * wg.Hp + (eq == 2 ? wg.Hp : 0) : nullptr;
+    const bool ext_in = EXT && wg.extL && w == 0, ext_out = EXT && wg.extR && w == wg.nseg - 1;
+    float *eoh = EXT ? wg.colh + plane0 * wave_x_plane(wg) + (int64_t)(sg + 1) * 2 * wg.Hp : nullptr;
+    float *eos = EXT ? wg.cols + plane0 * wave_x_plane(wg) + (int64_t)(sg + 1) * 2 * wg.Hp : nullptr;
 
     // Raw bits of a band's rows.  Lanes beyond the last column read the last columns (always in bounds): what they
     // compute only feeds cells further right and is never stored.
     typedef WaveRaw<T, CPL, VEC> Raw;
-    struct Stage { Raw u[R], d[R], b[R][NS], c[R][NS]; };
+    struct Stage { Raw u[R], d[R], b[R][NS], c[R][NS]; float e; };
     // Byte offsets advance by one row step per load (one vector add each).  Every band issues the same loads on
     // every path - the wait counters the compiler derives for the prefetch need that - so rows past the end of a
     // ragged last band read the last row again (their step is zero) and are never used.
@@ -157,6 +172,10 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
             const bool more = i0 + r + 1 < H;
             ou += more ? UhB : 0; od += more ? DhB : 0; ob += more ? BhB : 0; oc += more ? ChB : 0;
         }
+        if (EXT) q.e = ebase[min(i0 + er, wg.Hp - 1)];   // (by every wave, like the other loads; only the group's first wave uses it)
+    };
+    auto bcast = [](float v, int src_lane) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
     };
     // the lane's CPL values in scan order (element e of the raw bits is scan column CPL-1-e when fh)
     auto unpack = [&](const Raw &q, float (&v)[CPL]) {
@@ -205,7 +224,10 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
 #pragma unroll
                 for (int q = 0; q < RD; ++q)
 #pragma unroll
-                    for (int n = 0; n < NS; ++n) inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
+                    for (int n = 0; n < NS; ++n) {
+                        inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
+                        if (EXT && ext_in) inb[HOIST_IN ? q : 0][n] = make_float4(bcast(cur.e, n * R + r + q), bcast(cur.e, (NS + n) * R + r + q), bcast(cur.e, (2 * NS + n) * R + r + q), 0.f);
+                    }
             }
             if (r % RD == 0) wr = writer ? &sHO[step & 1][w + 1][0][0] : dump;   // this step's slot (or the lane's own word)
             if (r % RD == 0) {
@@ -234,8 +256,9 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column S*w-1
-                    const float4 in = ((SND_WAVE_ABLATE & 32) || ONE) ? make_float4(0.f, 0.f, 0.f, 0.f)
-                                      : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
+                    float4 in = ((SND_WAVE_ABLATE & 32) || ONE) ? make_float4(0.f, 0.f, 0.f, 0.f)
+                                : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
+                    if (EXT && !HOIST_IN && ext_in) in = make_float4(bcast(cur.e, n * R + r), bcast(cur.e, (NS + n) * R + r), bcast(cur.e, (2 * NS + n) * R + r), 0.f);
                     float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
                     unpack(cur.b[r][n], bu);
                     unpack(cur.c[r][n], cv);
@@ -268,6 +291,12 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
                     hdiag[n] = in.x;
                     if (!ONE && !(SND_WAVE_ABLATE & 32)) {
                         wr[(r % RD) * NS + n] = make_float4(h[CPL - 1], s[CPL - 1], a[CPL - 1], 0.f);
+                    }
+                    if (EXT && ext_out && lane == 63) {   // what enters the column group on the right
+                        const int64_t o = (int64_t)n * wave_x_plane(wg) + i0 + r;
+                        eoh[o] = h[CPL - 1];
+                        eoh[o + wg.Hp] = a[CPL - 1];
+                        eos[o] = s[CPL - 1];
                     }
                     if (SAVE) {                     // lane r keeps what entered the segment on row r (selects, no branch)
                         const bool mine = lane == r;
@@ -390,13 +419,42 @@ static int launch_wave_fwd_v(const snd_fwd_params &p, const WaveGeo &wg, hipStre
     return launch_wave_fwd_p<T, NS, CPL, VEC, 1, 1>(p, wg, stream);
 }
 
+// One launch per column group of a wide plane, left to right (the stream orders them).
+template <typename T, int NS>
+static int launch_wave_fwd_wide(const snd_fwd_params &p, WaveGeo wg, float *group_ws, hipStream_t stream) {
+    const snd_shape &sh = p.shape;
+    const bool save = p.x != nullptr, out32 = p.out_dtype == SND_F32;
+    constexpr bool F = std::is_same<T, float>::value;
+    if (!save && !group_ws) return SND_ERR_WORKSPACE;
+    wg.colh = save ? p.x : group_ws;
+    wg.cols = save ? p.x_sd : group_ws + (int64_t)sh.batch * sh.dim * sh.dstate * wave_x_plane(wg);
+    const dim3 grid = wave_grid2(sh.batch * sh.n_groups, sh.dim / sh.n_groups);
+    const int groups = wave_groups(wg.nsegAll);
+    for (int q = 0; q < groups; ++q) {
+        wg.seg0 = q * kMaxSeg;
+        wg.nseg = min(kMaxSeg, wg.nsegAll - wg.seg0);
+        wg.extL = q > 0;
+        wg.extR = q + 1 < groups;
+        const dim3 block(64 * wg.nseg);
+        if (save && out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, 1, true, true, true, 1, 1, false, true>), grid, block, 0, stream, p, wg);
+        else if (save) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, 1, true, true, F, 1, 1, false, true>), grid, block, 0, stream, p, wg);
+        else if (out32) hipLaunchKernelGGL((wave_fwd_kernel<T, NS, 1, true, false, true, 1, 1, false, true>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_fwd_kernel<T, NS, 1, true, false, F, 1, 1, false, true>), grid, block, 0, stream, p, wg);
+        if (hipGetLastError() != hipSuccess) return SND_ERR_LAUNCH;
+    }
+    return SND_OK;
+}
+
 template <typename T>
-int launch_wave_fwd_t(const snd_fwd_params &p, hipStream_t stream) {
+int launch_wave_fwd_t(const snd_fwd_params &p, float *group_ws, hipStream_t stream) {
     const snd_shape &sh = p.shape;
     const int N = sh.dstate;
     WaveGeo wg = make_wave_geo(sh.nrows, sh.ncols, N);
     wave_geo_channels(wg, sh.batch, sh.dim, sh.n_groups, sh.delta_dim);
     wg.tag = state_tag(p.x_sd, sh);
+    if (wg.nsegAll > kMaxSeg)
+        return N == 1 ? launch_wave_fwd_wide<T, 1>(p, wg, group_ws, stream) : N == 2 ? launch_wave_fwd_wide<T, 2>(p, wg, group_ws, stream)
+             : N == 3 ? launch_wave_fwd_wide<T, 3>(p, wg, group_ws, stream) : launch_wave_fwd_wide<T, 4>(p, wg, group_ws, stream);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.out_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned(p.u, e, 2 * e, {p.u_batch_stride, p.u_d_stride, p.u_h_stride}) &&

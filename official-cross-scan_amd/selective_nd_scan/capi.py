@@ -27,7 +27,7 @@ class Plan(C.Structure):
     _fields_ = [("n_chunks_x", i32), ("n_chunks_y", i32), ("x_inner", i32), ("xv_inner", i32),
                 ("x_elems", i64), ("x_sd_elems", i64), ("x_v_elems", i64), ("bwd_workspace_bytes", i64),
                 ("fwd_workspace_bytes", i64), ("auto_schedule", i32), ("auto_bwd_jobs", i32),
-                ("dC_skew_bytes", i64)]
+                ("dC_skew_bytes", i64), ("wavefront_workspace", i32), ("reserved_", i32)]
 
 
 class FwdParams(C.Structure):

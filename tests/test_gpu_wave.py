@@ -1,4 +1,4 @@
-"""The row-segment wavefront kernels (1-4 states per channel, planes up to 512 columns wide) against the
+"""The row-segment wavefront kernels (1-4 states per channel, planes of at most eight row segments) against the
 float64 oracle and against the tile kernels on the same inputs, through the C ABI."""
 import numpy as np
 import pytest
@@ -175,7 +175,7 @@ def test_wavefront_shared_u_and_second_backward(gpu_device):
 
 
 def test_wavefront_refuses_what_it_does_not_cover(gpu_device):
-    d = O.make_inputs(1, 4, 8, 601, N=1, K=1, seed=1)       # odd width above 512: one column per lane, nine segments
+    d = O.make_inputs(1, 4, 8, 60, N=5, K=1, seed=1)        # five states
     t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
     f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], None, None, False, True, None, True, capi.SCHED_WAVEFRONT)
     assert f.plan.auto_schedule != capi.SCHED_WAVEFRONT

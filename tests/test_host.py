@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header_sizes():
     # field-by-field mirror of include/snd_scan.h: natural alignment, no packing
     assert C.sizeof(capi.Shape) == 32
-    assert C.sizeof(capi.Plan) == 72
+    assert C.sizeof(capi.Plan) == 80
     assert C.sizeof(capi.FwdParams) == 32 + 8 + 12 * 8 + 19 * 8 + 8 + 8 + 4 * 4 + 8
     assert C.sizeof(capi.BwdParams) == C.sizeof(capi.FwdParams) + 8 + 8 + 3 * 8 + 9 * 8 + 8 + 8
 
@@ -31,7 +31,7 @@ def test_struct_layouts_match_header_sizes():
 def test_struct_layouts_match_the_c_compiler(tmp_path):
     """sizeof / offsetof of the header's structs as gcc sees them against the ctypes mirror."""
     import subprocess
-    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs", "dC_skew_bytes"]),
+    probes = [("snd_plan", capi.Plan, ["fwd_workspace_bytes", "bwd_workspace_bytes", "auto_schedule", "auto_bwd_jobs", "dC_skew_bytes", "wavefront_workspace"]),
               ("snd_fwd_params", capi.FwdParams, ["out", "x_sd", "u_batch_stride", "out_h_stride", "workspace", "schedule", "directions", "u_shared", "merge", "merge_weights"]),
               ("snd_bwd_params", capi.BwdParams, ["dout", "dout_dtype", "dout_batch_stride", "du", "workspace", "workspace_bytes", "dmerge"])]
     src = ["#include <stdio.h>", "#include <stddef.h>", '#include "snd_scan.h"', "int main(void) {"]
@@ -243,7 +243,29 @@ def test_kernel_family_choice():
     assert family(4, 192, 56, 56, 4) == "wave"            # 48 blocks: the strip pipeline's ramp costs more than the rows
     assert family(64, 192, 56, 56, 2) == "wave"
     assert family(64, 192, 56, 56, 16) == "tile"
-    assert family(1, 8, 9, 1500, 4, K=2) == "tile"         # wider than the wavefront kernels cover
+    assert family(1, 8, 9, 1500, 4, K=2) == "wave"         # a wide plane: 24 row segments in three column groups
+    assert family(2, 64, 256, 1024, 2) == "wave"
+    assert family(1, 8, 9, 1500, 5, K=2) == "tile"
+
+
+def test_wide_plane_plan():
+    """More than eight row segments: the row-segment kernels take the plane in column groups that hand over through
+    memory - the plan says so and sizes both workspaces for it; narrower planes need none."""
+    def plan_of(H, W, N, Bt=1, Dm=8):
+        st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, N, 2, Dm, capi.SND_F32))
+        assert st == 0
+        return plan
+    assert plan_of(9, 512, 2).wavefront_workspace == 0
+    assert plan_of(9, 1024, 1).wavefront_workspace == 0     # one state, even width: two columns per lane, eight segments
+    assert plan_of(9, 1023, 1).wavefront_workspace == 1     # odd: one column per lane, 16 segments
+    assert plan_of(9, 513, 2).wavefront_workspace == 1
+    assert plan_of(9, 2048, 16).wavefront_workspace == 0    # (5-16 states: the tile kernels)
+    p = plan_of(10, 1500, 2)
+    planes, Hp, nseg, groups = 8 * 2, 10, 24, 3
+    assert p.wavefront_workspace == 1
+    assert p.x_elems >= planes * nseg * 2 * Hp              # column checkpoints of all 24 segments
+    assert p.bwd_workspace_bytes >= planes * groups * 3 * Hp * 4
+    assert p.fwd_workspace_bytes >= 2 * planes * nseg * 2 * Hp * 4
 
 
 def test_tile_extent_choice():
