@@ -211,6 +211,9 @@ def main():
     ap.add_argument("--schedule", default="auto", choices=["auto", "plane", "strips", "bands", "wavefront"],
                     help="kernel family and block mapping: chosen by shape (default), one block per plane chunk, "
                          "pipelined row strips / bands, or the row-segment wavefront kernels (1-4 states)")
+    ap.add_argument("--strip-segments", type=int, default=0, metavar="N",
+                    help="timing studies: force the column segments per strip of the pipelined 16-state backward "
+                         "(1 = whole strips; 0 = the library's own choice)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this operator is measured on ONE GPU (every (batch, channel, state) plane is an "
@@ -224,6 +227,8 @@ def main():
 
     sched = {"auto": 0, "plane": 1, "strips": 2, "bands": 3, "wavefront": 4}[args.schedule]
     snd.set_schedule(sched)
+    if args.strip_segments:
+        capi.lib().snd_debug_set_strip_slots(-args.strip_segments)
     if args.shape:
         f_ = args.shape.split(",")
         WORKLOADS["custom"] = tuple(int(v) for v in f_[:6]) + (f_[6],)

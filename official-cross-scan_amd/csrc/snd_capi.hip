@@ -310,8 +310,11 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
     // backward is fastest half a row apart when a row is 2 KiB or more (512 x 512: 0.46 ms at 1 KiB + k * 2 KiB,
     // 0.55 at k * 2 KiB), and with narrower rows at 16 KiB (0 .. 9 KiB cost some shapes 10 % and gain others as much);
     // the tile kernels are indifferent.
+    // With three or four states and rows of 2 KiB or more no distance beat none at all (2 x 64 x 256x512, four states:
+    // 0.69 ms at 0, 0.77 half a row apart; 256x1024: 1.81 against 2.17).
     const int64_t row = (int64_t)shape->ncols * 4;
-    plan->dC_skew_bytes = plan->auto_schedule != SND_SCHED_WAVEFRONT ? 5 * 1024 : row >= 2048 ? (row / 2 + 255) / 256 * 256 : 16 * 1024;
+    plan->dC_skew_bytes = plan->auto_schedule != SND_SCHED_WAVEFRONT ? 5 * 1024
+                        : row < 2048 ? 16 * 1024 : shape->dstate >= 3 ? 0 : (row / 2 + 255) / 256 * 256;
     return SND_OK;
 }
 

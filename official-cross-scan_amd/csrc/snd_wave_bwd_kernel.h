@@ -28,7 +28,8 @@
 #include <type_traits>
 #include "snd_device.h"
 
-// Timing studies only (-DSND_WAVE_ABLATE=<bits>, results wrong): 64 no dB / dC atomics, 128 no du / ddelta stores.
+// Timing studies only (-DSND_WAVE_ABLATE=<bits>, results wrong): 64 no dB / dC atomics, 128 no du / ddelta stores,
+// 256 (column groups) nothing left for the group on the left, 512 nothing taken from the group on the right.
 #ifndef SND_WAVE_ABLATE
 #define SND_WAVE_ABLATE 0
 #endif
@@ -59,7 +60,7 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 // EXT: the launch works on one column group of a wide plane (wave_wide() in snd_device.h), segments seg0 .. seg0+nseg-1;
 // the groups are launched right to left.  The group's last wave takes G, Gs, a of the column on its right from global
 // memory (with the band's loads, three values per state and row spread over the lanes of one register), where the
-// first wave of the group on the right left them.
+// first wave of the group on the right left them, and puts them into the LDS slot a neighbouring wave would have filled.
 template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW, bool EXT = false>
 __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = wave_band_rows(NS);            // rows per band
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const float *ebase = EXT ? wg.bcol + (plane0 + (el / R) % NS) * wave_bcol_plane(wg)
                                + (int64_t)min(gq + 1, wave_groups(wg.nsegAll) - 1) * 3 * wg.Hp + eq * wg.Hp : nullptr;
     float *eout = EXT ? wg.bcol + plane0 * wave_bcol_plane(wg) + (int64_t)gq * 3 * wg.Hp : nullptr;
-    const bool ext_in = EXT && wg.extR && w == nseg - 1, ext_out = EXT && wg.extL && w == 0;
+    const bool ext_in = EXT && wg.extR && w == nseg - 1 && !(SND_WAVE_ABLATE & 512), ext_out = EXT && wg.extL && w == 0 && !(SND_WAVE_ABLATE & 256);
 
     // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
     // last columns (always in bounds) and only their dout is masked to zero where it is used, which makes every
@@ -368,6 +369,9 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         if (PF) load_band(nxt, max(band - 1, 0));
 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
+        // (column groups) what the group on the right left for this band goes where a wave on the right would have put
+        // it: the group's last wave fills its own neighbour slot, one word per lane, and the rows below read it as ever
+        if (EXT && ext_in && lane < kExtLanes) ((float *)&sHO[(step + 1) & 1][0][nseg][er][(el / R) % NS])[eq] = cur.e;
         const int rows = EVEN ? R : min(R, H - i0);  // rows of this band inside the plane
         const int mlast = mad24(i0 + rows - 1, rs, r0m);
         uint32_t og = mad24(mlast, WB * rs, colG), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
@@ -386,8 +390,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
-                    float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
-                    if (EXT && ext_in) in = make_float4(bcast(cur.e, n * R + r), bcast(cur.e, (NS + n) * R + r), bcast(cur.e, (2 * NS + n) * R + r), 0.f);
+                    const float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
                     const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
                     unpack(cur.b[r][n], Bv);

@@ -48,7 +48,8 @@ namespace snd {
 // EXT: the launch works on one column group of a wide plane (wave_wide() in snd_device.h): segments seg0 .. seg0+nseg-1.
 // The group's first wave takes what enters it on every row - h, s, a of the column on its left - from global memory,
 // where the launch of the group on the left put them (a band's values come with the band's loads, three per state and
-// row spread over the lanes of one register), and the group's last wave leaves the same for the group on its right.
+// row spread over the lanes of one register) and puts them into the LDS slot a wave on its left would have filled;
+// the group's last wave leaves the same for the group on its right.
 // The places are those of the column checkpoints the backward reads anyway (x, x_sd of segment seg0 and seg0+nseg).
 template <typename T, int NS, int CPL, bool VEC, bool SAVE, bool OUT32, int PK, int EU, bool ONE, bool EXT = false>
 __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__((amdgpu_waves_per_eu(EU))) void wave_fwd_kernel(const snd_fwd_params p, const WaveGeo wg) {
@@ -174,9 +175,6 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
         }
         if (EXT) q.e = ebase[min(i0 + er, wg.Hp - 1)];   // (by every wave, like the other loads; only the group's first wave uses it)
     };
-    auto bcast = [](float v, int src_lane) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src_lane));
-    };
     // the lane's CPL values in scan order (element e of the raw bits is scan column CPL-1-e when fh)
     auto unpack = [&](const Raw &q, float (&v)[CPL]) {
 #pragma unroll
@@ -220,14 +218,15 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
         float4 *wr = dump;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            // (column groups) what the group on the left left for this step's rows goes where a wave on the left would have
+            // put it: the group's first wave fills its own slot, one word per lane, and the rows read it as ever
+            if (EXT && r % RD == 0 && ext_in && lane < kExtLanes && er / RD == r / RD)
+                ((float *)&sHO[(step + 1) & 1][0][er % RD][(el / wave_fwd_rows(NS)) % NS])[eq] = cur.e;
             if (r % RD == 0 && HOIST_IN && !ONE && !(SND_WAVE_ABLATE & 32)) {
 #pragma unroll
                 for (int q = 0; q < RD; ++q)
 #pragma unroll
-                    for (int n = 0; n < NS; ++n) {
-                        inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
-                        if (EXT && ext_in) inb[HOIST_IN ? q : 0][n] = make_float4(bcast(cur.e, n * R + r + q), bcast(cur.e, (NS + n) * R + r + q), bcast(cur.e, (2 * NS + n) * R + r + q), 0.f);
-                    }
+                    for (int n = 0; n < NS; ++n) inb[HOIST_IN ? q : 0][n] = sHO[(step + 1) & 1][w][q][n];
             }
             if (r % RD == 0) wr = writer ? &sHO[step & 1][w + 1][0][0] : dump;   // this step's slot (or the lane's own word)
             if (r % RD == 0) {
@@ -256,9 +255,8 @@ __global__ __launch_bounds__(ONE ? 64 * kOneWaves : 64 * kMaxSeg) __attribute__(
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the left left for this row: h, s, a at column S*w-1
-                    float4 in = ((SND_WAVE_ABLATE & 32) || ONE) ? make_float4(0.f, 0.f, 0.f, 0.f)
-                                : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
-                    if (EXT && !HOIST_IN && ext_in) in = make_float4(bcast(cur.e, n * R + r), bcast(cur.e, (NS + n) * R + r), bcast(cur.e, (2 * NS + n) * R + r), 0.f);
+                    const float4 in = ((SND_WAVE_ABLATE & 32) || ONE) ? make_float4(0.f, 0.f, 0.f, 0.f)
+                                      : HOIST_IN ? inb[HOIST_IN ? r % RD : 0][n] : sHO[(step + 1) & 1][w][r % RD][n];
                     float a[CPL], bu[CPL], cv[CPL], y[CPL], h[CPL], s[CPL];
                     unpack(cur.b[r][n], bu);
                     unpack(cur.c[r][n], cv);

@@ -1,6 +1,8 @@
-"""Wide planes under the row-segment wavefront kernels (1-4 states, more than eight 64-column segments per row): the
+"""Wide planes.  Under the row-segment wavefront kernels (1-4 states, more than eight 64-column segments per row) the
 segments are taken in column groups of eight, one launch per group, and what crosses a group boundary goes through
-memory.  Against the float64 oracle on the same inputs, through the C ABI and through the autograd function."""
+memory.  Under the tile kernels planes wider than 1024 columns are the reference's nChunksX > 1 path
+(selective_scan_oflex.cpp:249): many column tiles per strip, the out gather over groups of tiles, hand-over rows at
+hundreds of tiles.  Against the float64 oracle on the same inputs, through the C ABI and through the autograd function."""
 import numpy as np
 import pytest
 import torch
@@ -33,6 +35,16 @@ def test_wide_planes_match_oracle(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, kw)
     d, t, f, b = run(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, capi.SCHED_WAVEFRONT, **kw)
     assert f.plan.wavefront_workspace == 1
     check_against_oracle(d, t, f, b, Dd=Dd, **kw)
+
+
+@pytest.mark.parametrize("N,dtype,sched", [(16, torch.float32, capi.SCHED_PLANE), (16, torch.float32, capi.SCHED_STRIPS),
+                                           (4, torch.float32, capi.SCHED_STRIPS), (16, torch.bfloat16, capi.SCHED_STRIPS),
+                                           (1, torch.float32, capi.SCHED_PLANE), (12, torch.float32, capi.SCHED_AUTO)])
+def test_wide_plane_tile_kernels(gpu_device, N, dtype, sched):
+    print("wide plane, tile kernels", N, dtype, sched, flush=True)
+    d, t, f, b = run(gpu_device, 1, 8, 9, 1500, N, 2, None, dtype, sched, seed=31)
+    assert f.plan.wavefront_workspace == (1 if N <= 4 else 0)
+    check_against_oracle(d, t, f, b)
 
 
 def test_wide_forward_without_saved_state_and_static_backward(gpu_device):
