@@ -313,6 +313,38 @@ def test_wavefront_packed_planes(gpu_device, Bt, Dm, H, W, N, K, Dd, dtype, kw):
     check_against_oracle(d, t, f, b, Dd=Dd, **kw)   # and the float64 oracle under the same options
 
 
+def test_packed_planes_keep_a_diverged_channel_inside_its_group(gpu_device):
+    """Eight 7-column planes share a wave, separated by barrier lanes that stop the scan by a multiplication with
+    zero: a channel that has run off to inf can therefore take the channel next to it in the wave along (inf * 0).
+    All planes of a wave belong to one (batch, group) pair, whose dB / dC a diverged channel spoils in any case;
+    pinned here: every other group comes out exactly as without the diverged channel."""
+    Bt, Dm, H, W, N, K = 1, 16, 7, 7, 1, 2
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=21)
+    res = {}
+    for poisoned in (False, True):
+        t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
+        if poisoned:
+            t["u"][0, 3, 2, 2] = float("inf")          # channel 3 of group 0 (channels 0-7)
+        args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
+        f = capi.FwdCall(*args, True, True, None, True, capi.SCHED_WAVEFRONT)
+        f.launch()
+        b = capi.BwdCall(*args, t["dout"], f.x, f.x_v, True, None, f.x_sd, capi.SCHED_WAVEFRONT)
+        b.launch()
+        torch.cuda.synchronize()
+        res[poisoned] = [x.clone() for x in (f.out, b.du, b.ddelta, b.dA, b.dB, b.dC, b.dD, b.dbias)]
+    assert not torch.isfinite(res[True][0][0, 3]).all()            # the inf did reach channel 3's result
+    rg = Dm // K
+    for nm, clean, got in zip(["out"] + NAMES, res[False], res[True]):
+        if nm in ("dB", "dC"):
+            clean, got = clean[:, 1], got[:, 1]                     # [batch, group, ...]
+        elif nm in ("out", "du", "ddelta"):
+            clean, got = clean[:, rg:], got[:, rg:]
+        else:
+            clean, got = clean[rg:], got[rg:]
+        assert torch.isfinite(got).all(), nm
+        assert relerr(got.cpu().numpy(), clean.cpu().numpy()) <= 1e-6, nm
+
+
 def _draw_large(seed):
     r = np.random.RandomState(7000 + seed)
     K = int(r.choice([2, 4]))
