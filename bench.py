@@ -119,8 +119,8 @@ VALU_PEAK = 157.3e12 / 128.0    # published FP32 vector peak in wave-wide multip
 
 
 def probe_peak():
-    """Wave-instructions per second of a pure v_fma_f32 stream on all CUs, as `bench.py --issue-probe` measured it
-    (committed summary), or None."""
+    """Wave-instructions per second of a pure v_fma_f32 stream on all CUs, from the committed summary of the
+    instruction-issue micro-benchmark, or None."""
     path = os.path.join(ROOT, "profiles", "issue_probe_mi355x.txt")
     if not os.path.exists(path):
         return None
