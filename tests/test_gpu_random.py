@@ -29,6 +29,15 @@ def draw(seed):
     c["Dd"] = c["Dm"] // 2 if (c["share_delta"] and c["Dm"] % 2 == 0) else c["Dm"]
     if c["N"] <= 4 and seed % 2 == 1:
         c["sched"] = capi.SCHED_WAVEFRONT                  # half of the small-state cases name the wavefront kernels (AUTO picks them too)
+    c["segments"] = 0
+    if c["N"] <= 4 and seed % 8 == 5:
+        # a wide plane: 9 to 24 row segments, taken by the wavefront kernels in column groups (few rows: the oracle's time)
+        c.update(W=int(r.randint(513, 1501)), H=int(r.randint(1, 13)), Bt=int(r.randint(1, 3)), Dm=K * min(rg, 4),
+                 sched=int(r.choice([capi.SCHED_AUTO, capi.SCHED_WAVEFRONT])))
+        c["Dd"] = c["Dm"] // 2 if (c["share_delta"] and c["Dm"] % 2 == 0) else c["Dm"]
+    if c["N"] >= 9 and seed % 4 == 3:
+        # the 16-lane backward with its strips cut into column segments (forced: the model only cuts large launches)
+        c.update(sched=capi.SCHED_STRIPS, segments=int(r.choice([2, 3, 4])), W=max(c["W"], 20))
     return c
 
 
@@ -56,9 +65,13 @@ def test_random_case(gpu_device, seed):
     f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, c["softplus"], c["out_float"], dec, True,
                      c["sched"], c["dirs"])
     f.launch()
-    g = capi.bwd(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, dout, f.x, f.x_v, c["softplus"], dec, f.x_sd,
-                 None, c["sched"], c["dirs"])
-    torch.cuda.synchronize()
+    capi.lib().snd_debug_set_strip_slots(-c["segments"])    # (0: the library's own choice)
+    try:
+        g = capi.bwd(t["u"], t["delta"], t["A"], t["B"], t["C"], D, bias, dout, f.x, f.x_v, c["softplus"], dec, f.x_sd,
+                     None, c["sched"], c["dirs"])
+        torch.cuda.synchronize()
+    finally:
+        capi.lib().snd_debug_set_strip_slots(0)
     strips = c["sched"] in (capi.SCHED_STRIPS, capi.SCHED_BANDS) or (c["sched"] == capi.SCHED_AUTO and f.plan.auto_schedule in (capi.SCHED_STRIPS, capi.SCHED_BANDS))
     if strips and f.plan.n_chunks_y > 1:                   # a single strip always runs as a whole plane
         assert int(f.ws.view(torch.int32)[1]) == 0         # no strip wait gave up
