@@ -76,10 +76,11 @@ typedef struct snd_plan {
                                                   (16-byte aligned, uninitialised; one row per plane) */
     int32_t auto_schedule;                     /* what SND_SCHED_AUTO resolves to in the forward for this shape
                                                   (PLANE, STRIPS, BANDS or WAVEFRONT): a caller may skip the fwd
-                                                  workspace for PLANE and WAVEFRONT */
+                                                  workspace for PLANE and WAVEFRONT (see wavefront_workspace) */
     int32_t auto_bwd_jobs;                     /* jobs per plane chunk SND_SCHED_AUTO gives the backward: 0 = one
                                                   block per plane chunk (also when auto_schedule is WAVEFRONT: then
-                                                  the backward runs WAVEFRONT too and needs no workspace),
+                                                  the backward runs WAVEFRONT too and needs no workspace unless
+                                                  wavefront_workspace is 1),
                                                   n_chunks_y = one per strip, 2-4 = bands */
     /* Placement advice for callers that allocate the buffers (no counterpart in the reference, which leaves
      * placement to torch::empty).  The backward accumulates dB and dC at equal offsets at the same time.

@@ -46,6 +46,9 @@ def _case(gpu_device, Bt, Dm, H, W, N, K, dtype, seed, shared_u):
     (2, 24, 14, 14, 1, 4, torch.float32, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, True, True),  # four planes per wave, 6 channels per group
     (2, 28, 9, 30, 2, 4, torch.bfloat16, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, False, True), # two planes per wave, 7 channels per group
     (2, 40, 7, 7, 1, 4, torch.float32, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, True, True),    # eight planes per wave, 10 channels per group
+    (1, 8, 9, 1100, 2, 4, torch.float32, capi.SCHED_AUTO, capi.DIR_CORNERS, True, True),       # a wide plane: three column groups
+    (1, 8, 6, 700, 1, 4, torch.bfloat16, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, False, True), # odd-free width 700 > 512 with one state: two columns per lane, six segments
+    (1, 8, 6, 701, 1, 4, torch.float32, capi.SCHED_WAVEFRONT, capi.DIR_CORNERS, True, False),  # odd width: one column per lane, eleven segments in two groups
 ])
 def test_fused_merge_matches_two_steps(gpu_device, Bt, Dm, H, W, N, K, dtype, sched, dirs, shared_u, weighted):
     print("merge", Bt, Dm, H, W, N, K, dtype, sched, dirs, shared_u, weighted, flush=True)
