@@ -396,6 +396,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             }
 
             // ---- per-lane tile walk
+            // The tile walk runs at the default wave priority and everything around it (stores, epilogue, the next tile's
+            // commit and load requests) at a raised one: of a SIMD's three waves the ones with memory instructions to issue
+            // go first.  Measured (same box, forward ms): c1 0.497 -> 0.490, c2 0.115 -> 0.109, c3 0.615 -> 0.602,
+            // c4 1.177 -> 1.153; the reverse assignment gains half as much.
+            __builtin_amdgcn_s_setprio(0);
 #pragma unroll
             for (int j = 0; j < kCkX; ++j) aup[j] = (I > 0 && j < TE) ? fast_exp2(fmaf(myDl[j], A2, ld)) : 0.f;
 
@@ -445,6 +450,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                     }
                 }
             }
+            __builtin_amdgcn_s_setprio(3);
             if (geo.nCX == 1 && I + 1 < I_end) {    // the next strip's row above is this tile's last row
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) qxv[j] = hup[j];

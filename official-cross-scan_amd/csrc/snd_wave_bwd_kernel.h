@@ -261,6 +261,10 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     auto do_band = [&](In &cur, In &nxt, int band) {
         if (!PF) load_band(cur, band);
         const int i0 = band * R;
+        // (the recomputation at a raised wave priority, the sweep with its stores and atomics at the default one: the
+        // waves sharing a SIMD then interleave the two phases.  2 x 192 x 200x336, two states: 0.419 -> 0.400 ms, four
+        // states at 56x56 0.662 -> 0.647, the one-state workloads unchanged)
+        __builtin_amdgcn_s_setprio(3);
 
         // ---- recompute h, s on the band's rows (with the columns); results back in mirrored order.
         // Index t of the mirrored order is natural column index CPL-1-t of the lane that holds the same columns.
@@ -367,6 +371,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         // here they have had the whole recomputation to complete.  Unconditionally (band 0 once more): a skipped
         // load would leave two paths with different numbers of loads in flight, and the waits follow the smaller.
         if (PF) load_band(nxt, max(band - 1, 0));
+        __builtin_amdgcn_s_setprio(0);
 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
         // (column groups) what the group on the right left for this band goes where a wave on the right would have put
