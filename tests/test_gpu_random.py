@@ -116,6 +116,11 @@ def test_random_case(gpu_device, seed):
             # (2 x 8 planes of 22 x 10, N = 2) measures 1.0e-4 to 1.2e-4 depending on the order the atomics
             # land in.  Every other gradient keeps 1e-4.
             tol = 5e-4
+        if nm == "dA" and c["H"] == 1:
+            # likewise dA of a single row is identically zero, a sum of terms that cancel: what comes back is the fp32
+            # rounding noise of that sum on relerr's absolute scale of 1e-2, and it grows with the row (seed 1805:
+            # 1.4e-6 over 2 x 891 cells of four states with A_decay)
+            tol = 5e-3
         if nm == "dA_decay" and c["H"] == 1:
             # a single row makes h = s, so out does not depend on a: the reference is zero and relerr
             # measures the fp32 rounding noise of a sum over every cell of every plane on its absolute
