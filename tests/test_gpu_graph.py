@@ -14,9 +14,24 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("sched,dims", [(capi.SCHED_PLANE, (2, 16, 40, 24, 16)), (capi.SCHED_STRIPS, (2, 16, 40, 24, 16)),
                                         (capi.SCHED_BANDS, (2, 16, 40, 24, 16)),
                                         # the row-segment kernels: packed planes in four-wave blocks; three segments
-                                        (capi.SCHED_WAVEFRONT, (4, 160, 14, 14, 1)), (capi.SCHED_WAVEFRONT, (2, 16, 40, 150, 2))])
+                                        (capi.SCHED_WAVEFRONT, (4, 160, 14, 14, 1)), (capi.SCHED_WAVEFRONT, (2, 16, 40, 150, 2)),
+                                        # a wide plane: three launches per kernel (column groups) handing over through memory
+                                        (capi.SCHED_WAVEFRONT, (1, 8, 12, 1300, 2)),
+                                        # strips of the 16-lane backward cut into three column segments (forced)
+                                        (-3, (2, 16, 40, 100, 16))])
 def test_graph_replays_match_eager(gpu_device, sched, dims):
     print("graph", sched, dims, flush=True)
+    segments = 0
+    if sched < 0:
+        segments, sched = -sched, capi.SCHED_STRIPS
+    capi.lib().snd_debug_set_strip_slots(-segments)
+    try:
+        _graph_replays(gpu_device, sched, dims)
+    finally:
+        capi.lib().snd_debug_set_strip_slots(0)
+
+
+def _graph_replays(gpu_device, sched, dims):
     d = O.make_inputs(*dims[:4], N=dims[4], K=4, seed=13)
     t = {k: torch.from_numpy(v).to(gpu_device) for k, v in d.items()}
     args = (t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"])
