@@ -91,11 +91,15 @@ typedef struct snd_plan {
      * measured at).  Results do not depend on placement, and no other pair of buffers shows the effect
      * (timed with dC moved step by step inside one large allocation). */
     int64_t dC_skew_bytes;
-    int32_t wavefront_workspace;               /* 1 if WAVEFRONT takes this shape's planes in column groups (rows of more
-                                                  than 512 columns; with one state and an even width, more than 1024):
-                                                  the groups hand over through memory - bwd then needs its workspace
-                                                  (bwd_workspace_bytes covers it), and a fwd that saves no state
-                                                  (x == NULL) needs fwd_workspace_bytes, or AUTO runs the tile kernels */
+    int32_t wavefront_workspace;               /* 1 if WAVEFRONT uses the workspace for this shape.  Planes taken in
+                                                  column groups (rows of more than 512 columns; with one state and an
+                                                  even width, more than 1024) hand over through memory: bwd then needs
+                                                  its workspace (bwd_workspace_bytes covers it), and a fwd that saves
+                                                  no state (x == NULL) needs fwd_workspace_bytes, or AUTO runs the tile
+                                                  kernels.  Few planes of 449-512 columns with one or two
+                                                  states (at most 256 planes, e.g. 256 of 512x512): bwd cuts each plane
+                                                  in two halves that run side by side if it is given its workspace
+                                                  (about a fifth faster), and runs whole planes without one */
     int32_t reserved_;
 } snd_plan;
 

@@ -294,6 +294,13 @@ int snd_make_plan(const snd_shape *shape, snd_plan *plan) {
         if (fw > plan->fwd_workspace_bytes) plan->fwd_workspace_bytes = fw;
         if (bw > plan->bwd_workspace_bytes) plan->bwd_workspace_bytes = bw;
     }
+    if (wave && snd::wave_bwd_split(shape->batch, shape->dim, shape->ncols, shape->dstate)) {
+        // split planes (backward of the row-segment kernels): the tagged words the two halves of a plane hand over through
+        plan->wavefront_workspace = 1;
+        const snd::WaveGeo wg = snd::make_wave_geo(shape->nrows, shape->ncols, shape->dstate);
+        const int64_t bw = group_ws_offset(*shape) + planes * snd::wave_split_words(wg) * (int64_t)sizeof(float);
+        if (bw > plan->bwd_workspace_bytes) plan->bwd_workspace_bytes = bw;
+    }
     // and, where the backward's strips are cut into column segments, one carried column state per strip
     if (snd::strip_segments(plane_chunks(*shape), g.nCY, g.nCX, snd::bwd_slots(shape->dstate), snd::job_queues(shape->batch * shape->n_groups)) > 1)
         plan->bwd_workspace_bytes += plane_chunks(*shape) * g.nCY * (int64_t)snd::kColStateFloats * (int64_t)sizeof(float);
@@ -393,6 +400,10 @@ static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
     if (wave && snd::wave_wide(params->f.shape.ncols, params->f.shape.dstate)) {   // a wide plane's column groups hand over here
         if (!params->workspace || params->workspace_bytes < plan.bwd_workspace_bytes) return SND_ERR_WORKSPACE;
         if (!aligned16(params->workspace)) return SND_ERR_ALIGN;
+        group_ws = (float *)((char *)params->workspace + group_ws_offset(params->f.shape));
+    } else if (wave && snd::wave_bwd_split(params->f.shape.batch, params->f.shape.dim, params->f.shape.ncols, params->f.shape.dstate) &&
+               params->workspace && params->workspace_bytes >= plan.bwd_workspace_bytes && aligned16(params->workspace)) {
+        // split planes: the faster backward where the caller brought the workspace for it, whole planes otherwise
         group_ws = (float *)((char *)params->workspace + group_ws_offset(params->f.shape));
     }
     if (wave) {                                     // (other planes need no workspace)

@@ -545,7 +545,10 @@ struct WaveGeo {
     int extL, extR;                // whether a column group lies to the left / right of this launch's
     float *colh, *cols;            // (wide planes, forward) where column groups hand over h, a and s: the saved state
                                    // x, x_sd themselves, or a workspace of the same layout when no state is saved
-    float *bcol;                   // (wide planes, backward) G, Gs, a at the first column of every column group
+    float *bcol;                   // (wide planes, backward) G, Gs, a at the first column of every column group;
+                                   // (split planes, backward) the same as tagged words, see wave_bwd_split()
+    int *sync;                     // (split planes) the workspace's sync words (error word) and the bound of a wait
+    int spinLimit;
     int R;                         // rows per band (wave_band_rows): row-checkpoint spacing = rows the backward holds in registers
     int nBands;                    // ceil(H / R)
     int Hp, Wp;                    // nBands * R, nseg * 64 * cpl / planes per wave
@@ -593,6 +596,7 @@ __host__ __device__ inline WaveGeo make_wave_geo(int H, int W, int N) {
     g.nseg = g.nsegAll < kMaxSeg ? g.nsegAll : kMaxSeg;
     g.seg0 = 0; g.extL = g.extR = 0;
     g.colh = g.cols = g.bcol = nullptr;
+    g.sync = nullptr; g.spinLimit = 0;
     g.R = wave_band_rows(N);
     g.nBands = (H + g.R - 1) / g.R;
     g.Hp = g.nBands * g.R;
@@ -610,6 +614,22 @@ __host__ __device__ inline int64_t wave_x_plane(const WaveGeo &g) { return (int6
 // (wide planes, backward) the hand-over between column groups, per (batch, channel, state) plane:
 //   bcol [group q][3][Hp]   G, Gs, a at the first column of group q on every row (written by group q, read by group q-1)
 __host__ __device__ inline int64_t wave_bcol_plane(const WaveGeo &g) { return (int64_t)wave_groups(g.nsegAll) * 3 * g.Hp; }
+// Split planes (backward).  Few planes of eight segments with one or two states - 256 planes of 512 x 512 are
+// one block of eight waves per CU - leave no room for two channels in a block, which is what halves the dB / dC
+// atomics the kernel is bound by there.  Such a plane is cut in two halves of four segments: a block is two
+// channels x one half, the two blocks of a channel pair run side by side in one launch, and the left half takes G, Gs,
+// a of the right half's first column, band by band, through memory: 8-byte words {value, band + 1} that the right
+// half's edge wave stores as it goes (no count, no wait for the stores) and an extra wave of the left half's block
+// loads a band ahead and checks (all tags must be the band's; otherwise it loads again, a bounded number of times).
+// The words are zeroed by a fill kernel before the launch.  Per (batch, channel, state) plane: [band][3][R] words.
+__host__ __device__ inline bool wave_bwd_split(int batch, int dim, int W, int N) {
+    const int cpl = wave_cpl(W, N), nseg = (W + kSeg * cpl - 1) / (kSeg * cpl);
+    const int64_t planes = (int64_t)batch * dim;
+    // (eight segments only: with six - two halves of three - the split measured 8-11 % slower than whole planes at
+    // 1 x 192 x 300x384, two states, and 1 x 200 x 300x360; with eight 7-15 % faster, ragged widths included)
+    return cpl == 1 && N <= 2 && nseg == 8 && planes <= 256 && planes * nseg >= 1024;
+}
+__host__ __device__ inline int64_t wave_split_words(const WaveGeo &g) { return (int64_t)g.nBands * 3 * g.R * 2; }   // floats per plane
 __host__ __device__ inline int64_t wave_xv_plane(const WaveGeo &g) { return (int64_t)g.nBands * g.Wp; }
 
 // Block of the wavefront kernels -> (batch, group) pair and channel inside the group.  With many pairs all

@@ -61,10 +61,15 @@ __device__ __forceinline__ void wave_glb_add(float *p, float v) {
 // the groups are launched right to left.  The group's last wave takes G, Gs, a of the column on its right from global
 // memory (with the band's loads, three values per state and row spread over the lanes of one register), where the
 // first wave of the group on the right left them, and puts them into the LDS slot a neighbouring wave would have filled.
-template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW, bool EXT = false>
-__global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
+//
+// SPL (with EXT): a split plane (wave_bwd_split() in snd_device.h): the block works on one half of the segments of two
+// channels, the two halves of a channel pair are blocks of the same launch, and the hand-over goes through tagged
+// words that the left half's edge wave checks.
+template <typename T, int NS, int CPL, bool VEC, bool DO32, bool EVEN, int CHB, int PK, int XW, bool EXT = false, bool SPL = false>
+__global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(const snd_bwd_params p, const WaveGeo wg) {
     constexpr int R = wave_band_rows(NS);            // rows per band
-    static_assert(!EXT || (CHB == 1 && PK == 1 && CPL == 1 && !EVEN), "column groups: one channel per block, one column per lane");
+    static_assert(!EXT || (CHB == (SPL ? 2 : 1) && PK == 1 && CPL == 1 && (!EVEN || SPL)), "column groups: one channel per block, one column per lane");
+    static_assert(!SPL || EXT, "a split plane hands over like a column group");
     static_assert(CHB == 1 || CPL == 1, "shared atomics: one column per lane");
     static_assert(PK == 1 || (CHB > 1 && !EVEN), "packed planes share their atomics");
     constexpr int S = 64 / PK;                       // lanes per plane
@@ -91,9 +96,59 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const int lane = threadIdx.x & 63, wi = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int kc = CHB > 1 ? wi / nseg : 0, w = PK > 1 ? 0 : wi - kc * nseg;     // channel of the block, segment of the channel
     const int sl = PK > 1 ? lane % S : lane;         // the lane inside its plane
-    const int sg = EXT ? wg.seg0 + w : w;            // this wave's segment of the plane
-    int pair, chunk;
-    if (!wave_job2(wg, sh.batch * G, pair, chunk)) return;
+    int pair, chunk, half = 0;
+    if (SPL) {
+        // Blocks are dealt to the XCDs in turn (block i to XCD i % 8); the two halves of a channel pair take consecutive
+        // places of one XCD, the right half - which never waits - first: what it hands over then passes through the L2
+        // the left half reads from.
+        const int id = blockIdx.x, slot = id >> 3, unit = (slot >> 1) * 8 + (id & 7), nCP = (rg + 1) >> 1;
+        half = slot & 1;
+        if (unit >= sh.batch * G * nCP) return;
+        pair = unit / nCP;
+        chunk = unit - pair * nCP;
+    } else if (!wave_job2(wg, sh.batch * G, pair, chunk)) {
+        return;
+    }
+    if (SPL && wi == CHB * nseg) {
+        // The block's extra wave.  In a left half it fetches what the right half has left for the coming band - the tagged
+        // words of both channels, one word per lane, loaded again until every tag is the band's (a bounded number of
+        // times) - and puts the values where a wave on the right of the half's last segment would have put them, one
+        // step ahead of the wave that reads them.  Loads that pass the L2 by take several microseconds behind the
+        // kernel's dB / dC atomics, and a wave's memory instructions complete in order: issued by the half's last wave
+        // itself, one such load per band held up its whole queue (0.46 instead of 0.36 ms at 256 planes of 512x512).
+        // This wave has no other loads.  It joins every barrier of the block; in a right half that is all it does.
+        constexpr int kWords = 3 * NS * R;           // (at most 12)
+        const int hk = lane >> 4, hl = lane & 15, hq = hl / (NS * R), hn = (hl / R) % NS, hr = hl % R;
+        int b_, g_;
+        wave_pair_split(wg, pair, G, b_, g_);
+        const int64_t plane = ((int64_t)b_ * Dm + g_ * rg + min(chunk * CHB + hk, rg - 1)) * N + hn;
+        const bool fetch = half == 1 && hk < CHB && hl < kWords;
+        const uint64_t *src = (const uint64_t *)(wg.bcol + (fetch ? plane : 0) * wave_split_words(wg) + 2 * (hq * R + hr));
+        bool dead = false;
+        lds_barrier();                               // the zeroed slots
+        for (int s = 0; s < wg.nBands + nseg; ++s) {
+            if (half == 1 && s < wg.nBands) {
+                const int band = wg.nBands - 1 - s;
+                const bool mine = fetch && band * R + hr < H;   // (rows past the plane's last are never swept: no words for them)
+                const uint32_t want = (uint32_t)band + 1u;
+                uint64_t word = 0;
+                for (int polls = 0;; ++polls) {
+                    if (mine) word = __hip_atomic_load(src + (int64_t)band * (3 * R), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (dead || __builtin_amdgcn_ballot_w64(mine && (uint32_t)(word >> 32) != want) == 0) break;
+                    if (polls >= wg.spinLimit) {
+                        dead = true;
+                        __hip_atomic_store(wg.sync + kErrorWord, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(SND_POLL_SLEEP);
+                }
+                if (fetch) ((float *)&sHO[(s + 1) & 1][hk < CHB ? hk : 0][nseg][hr][hn])[hq] = dead ? __builtin_nanf("") : __builtin_bit_cast(float, (uint32_t)word);   // (never plausible numbers)
+            }
+            lds_barrier();
+        }
+        return;
+    }
+    const int sg = EXT ? (SPL ? (half ? 0 : wg.seg0) : wg.seg0) + w : w;   // this wave's segment of the plane
     chunk = (chunk * CHB + kc) * PK + (PK > 1 ? lane / S : 0);       // (packed: a lane's own from here on)
     // A wave (a plane of a wave) past the last channel of its group repeats that channel (identical du / ddelta
     // stores) and adds nothing.
@@ -177,7 +232,10 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     const float *ebase = EXT ? wg.bcol + (plane0 + (el / R) % NS) * wave_bcol_plane(wg)
                                + (int64_t)min(gq + 1, wave_groups(wg.nsegAll) - 1) * 3 * wg.Hp + eq * wg.Hp : nullptr;
     float *eout = EXT ? wg.bcol + plane0 * wave_bcol_plane(wg) + (int64_t)gq * 3 * wg.Hp : nullptr;
-    const bool ext_in = EXT && wg.extR && w == nseg - 1 && !(SND_WAVE_ABLATE & 512), ext_out = EXT && wg.extL && w == 0 && !(SND_WAVE_ABLATE & 256);
+    const bool ext_in = EXT && (SPL ? half == 1 : wg.extR != 0) && w == nseg - 1 && !(SND_WAVE_ABLATE & 512),
+               ext_out = EXT && (SPL ? half == 0 : wg.extL != 0) && w == 0 && !(SND_WAVE_ABLATE & 256);
+    // (split planes) the tagged words of the plane's first state
+    float *eouttag = SPL ? wg.bcol + plane0 * wave_split_words(wg) : nullptr;
 
     // Inputs of one band.  Rows wait as raw bits in mirrored lane order; lanes beyond the last column read the
     // last columns (always in bounds) and only their dout is masked to zero where it is used, which makes every
@@ -236,7 +294,9 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
                 }
             }
         }
-        if (EXT) q.e = ebase[i0 + er];               // (by every wave, like the other loads; only the group's last wave uses it)
+        if (EXT && !SPL) q.e = ebase[i0 + er];       // (by every wave, like the other loads; only the group's last wave uses it)
+        // (split planes: by the left half's edge wave alone - the load passes the L2 by, takes that much longer, and every
+        // load behind it in a wave's queue waits for it: issued by all waves it cost 256 planes of 512x512 0.07 of 0.44 ms)
     };
     // the lane's CPL values in its walking order t (element e of the raw bits is t = CPL-1-e, or t = e when fh)
     auto unpack = [&](const auto &q, float (&v)[CPL]) {
@@ -376,7 +436,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
         // ---- adjoint sweep over the band's rows, bottom-up (against the columns: local index t walks downwards)
         // (column groups) what the group on the right left for this band goes where a wave on the right would have put
         // it: the group's last wave fills its own neighbour slot, one word per lane, and the rows below read it as ever
-        if (EXT && ext_in && lane < kExtLanes) ((float *)&sHO[(step + 1) & 1][0][nseg][er][(el / R) % NS])[eq] = cur.e;
+        if (EXT && !SPL && ext_in && lane < kExtLanes) ((float *)&sHO[(step + 1) & 1][kc][nseg][er][(el / R) % NS])[eq] = cur.e;
         const int rows = EVEN ? R : min(R, H - i0);  // rows of this band inside the plane
         const int mlast = mad24(i0 + rows - 1, rs, r0m);
         uint32_t og = mad24(mlast, WB * rs, colG), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
@@ -453,11 +513,18 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) { Gd[n][t] = Gt[t]; ad[n][t] = a[t]; }
                     if (hands_over && lane == 63) sHO[step & 1][kc][w][r][n] = make_float4(Gt[CPL - 1], Gst[CPL - 1], a[CPL - 1], 0.f);
-                    if (EXT && ext_out && lane == 63) {   // for the column group on the left
+                    if (EXT && !SPL && ext_out && lane == 63) {   // for the column group on the left
                         float *d = eout + (int64_t)n * wave_bcol_plane(wg) + i0 + r;
                         d[0] = Gt[CPL - 1];
                         d[wg.Hp] = Gst[CPL - 1];
                         d[2 * wg.Hp] = a[CPL - 1];
+                    }
+                    if (SPL && ext_out && lane == 63) {           // for the left half: tagged with the band
+                        float *d = eouttag + (int64_t)n * wave_split_words(wg) + (int64_t)band * (6 * R) + 2 * r;
+                        const float tg = __builtin_bit_cast(float, (uint32_t)band + 1u);
+                        st2_coherent(d, Gt[CPL - 1], tg);
+                        st2_coherent(d + 2 * R, Gst[CPL - 1], tg);
+                        st2_coherent(d + 4 * R, a[CPL - 1], tg);
                     }
                 }
                 if (jin) {
@@ -509,6 +576,7 @@ __global__ __launch_bounds__(64 * XW) void wave_bwd_kernel(const snd_bwd_params 
     // (nothing in flight on the way into the band loop: its first waits then follow the loop's own path as well)
     if (PF && EVEN) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     lds_barrier();                                   // the zeroed slot
+    if (SPL) lds_barrier();                          // (and what the block's extra wave has fetched for the first band)
     if (multi)
         for (int e = 0; e < (nseg - 1 - w) * (CHB > 1 && kXBuf == 1 ? 2 : 1); ++e) lds_barrier();
     if (PF) {
@@ -630,6 +698,35 @@ static int launch_wave_bwd_wide(const snd_bwd_params &p, WaveGeo wg, float *grou
     return SND_OK;
 }
 
+// A split plane: one launch, two blocks (right half, left half) per pair of channels; the tagged words are zeroed first.
+template <typename T, int NS>
+static int launch_wave_bwd_split(const snd_bwd_params &p, WaveGeo wg, float *group_ws, hipStream_t stream) {
+    const snd_shape &sh = p.f.shape;
+    constexpr bool F32 = std::is_same<T, float>::value;
+    constexpr bool K = NS <= 2;                      // (the kernel exists for one and two states)
+    const int64_t words = (int64_t)((char *)group_ws - (char *)p.workspace) / 4 + (int64_t)sh.batch * sh.dim * sh.dstate * wave_split_words(wg);
+    if (zero_words((int *)p.workspace, words, stream) != SND_OK) return SND_ERR_LAUNCH;
+    wg.bcol = group_ws;
+    wg.sync = (int *)p.workspace;
+    wg.spinLimit = spin_limit();
+    wg.nseg = wg.nsegAll / 2;
+    wg.seg0 = wg.nseg;                               // (of the right halves; left halves start at segment 0)
+    const int rg = sh.dim / sh.n_groups;
+    const int units = sh.batch * sh.n_groups * ((rg + 1) / 2);          // channel pairs
+    const dim3 grid(2 * 8 * ((units + 7) / 8)), block(64 * (wg.nseg * 2 + 1));   // (two blocks per pair, see the kernel's block mapping; a block's
+                                                                              // last wave only fetches what the other half left)
+    // (whole bands and whole segments: the instantiation without a branch around a row or a lane, as for whole planes)
+    const bool even = sh.nrows % wave_band_rows(NS) == 0 && sh.ncols % kSeg == 0;
+    if (even) {
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, K ? NS : 1, 1, true, true, true, 2, 1, kMaxSeg, true, true>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, K ? NS : 1, 1, true, F32, true, 2, 1, kMaxSeg, true, true>), grid, block, 0, stream, p, wg);
+    } else {
+        if (p.dout_dtype == SND_F32) hipLaunchKernelGGL((wave_bwd_kernel<T, K ? NS : 1, 1, true, true, false, 2, 1, kMaxSeg, true, true>), grid, block, 0, stream, p, wg);
+        else hipLaunchKernelGGL((wave_bwd_kernel<T, K ? NS : 1, 1, true, F32, false, 2, 1, kMaxSeg, true, true>), grid, block, 0, stream, p, wg);
+    }
+    return hipGetLastError() == hipSuccess ? SND_OK : SND_ERR_LAUNCH;
+}
+
 template <typename T>
 int launch_wave_bwd_t(const snd_bwd_params &p, float *group_ws, hipStream_t stream) {
     const snd_fwd_params &f = p.f;
@@ -641,6 +738,8 @@ int launch_wave_bwd_t(const snd_bwd_params &p, float *group_ws, hipStream_t stre
     if (wg.nsegAll > kMaxSeg)
         return N == 1 ? launch_wave_bwd_wide<T, 1>(p, wg, group_ws, stream) : N == 2 ? launch_wave_bwd_wide<T, 2>(p, wg, group_ws, stream)
              : N == 3 ? launch_wave_bwd_wide<T, 3>(p, wg, group_ws, stream) : launch_wave_bwd_wide<T, 4>(p, wg, group_ws, stream);
+    if (group_ws && wave_bwd_split(sh.batch, sh.dim, sh.ncols, N))   // (without a workspace: whole planes, one channel per block)
+        return N == 1 ? launch_wave_bwd_split<T, 1>(p, wg, group_ws, stream) : launch_wave_bwd_split<T, 2>(p, wg, group_ws, stream);
     if (wg.cpl == 2) {                               // (N = 1 only)
         const int e = (int)sizeof(T), oe = p.dout_dtype == SND_F32 ? 4 : e;
         const bool vec = wave_aligned_b(f.u, e, 2 * e, {f.u_batch_stride, f.u_d_stride, f.u_h_stride}) &&

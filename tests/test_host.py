@@ -268,6 +268,23 @@ def test_wide_plane_plan():
     assert p.fwd_workspace_bytes >= 2 * planes * nseg * 2 * Hp * 4
 
 
+def test_split_plane_plan():
+    """Few planes of eight row segments with one or two states: the backward may cut them in two halves that hand over
+    through tagged words in the workspace - the plan says so and sizes the backward's workspace for the words."""
+    def plan_of(Bt, Dm, H, W, N):
+        st, plan = capi.make_plan(capi.Shape(Bt, Dm, H, W, N, 4, Dm, capi.SND_BF16))
+        assert st == 0
+        return plan
+    p = plan_of(1, 256, 512, 512, 1)                        # 256 planes x 8 segments
+    assert p.auto_schedule == capi.SCHED_WAVEFRONT and p.wavefront_workspace == 1
+    assert p.bwd_workspace_bytes >= 256 * (512 // 4) * 3 * 4 * 8     # planes x bands x (G, Gs, a) x rows per band x 8 bytes
+    assert plan_of(1, 256, 512, 512, 2).wavefront_workspace == 1
+    assert plan_of(1, 256, 512, 512, 4).wavefront_workspace == 0    # three and four states: whole planes
+    assert plan_of(1, 256, 512, 384, 1).wavefront_workspace == 0    # six segments: whole planes
+    assert plan_of(2, 256, 512, 512, 1).wavefront_workspace == 0    # 512 planes: two channels share a block of 16 waves
+    assert plan_of(1, 64, 512, 512, 1).wavefront_workspace == 0     # 512 waves: too few to be worth the pairing
+
+
 def test_tile_extent_choice():
     """7x7 tiles where they leave clearly fewer padded cells (the 14 / 28 / 7 stage sizes), else 8x8."""
     def tiles(H, W):
