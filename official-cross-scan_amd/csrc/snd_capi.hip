@@ -407,6 +407,11 @@ static int bwd_checked(const snd_bwd_params *params, snd_stream_t stream) {
         group_ws = (float *)((char *)params->workspace + group_ws_offset(params->f.shape));
     }
     if (wave) {                                     // (other planes need no workspace)
+        // the row-segment backward addresses a batch image of du / ddelta and a (batch, group)'s dB / dC planes through
+        // buffer descriptors: unsigned 32-bit byte offsets that must stay below the out-of-range marker
+        const snd_shape &ws = params->f.shape;
+        if ((int64_t)ws.dim * ws.nrows * ws.ncols * 4 >= (int64_t)snd::kBufOOB || (int64_t)ws.dstate * ws.nrows * ws.ncols * 4 >= (int64_t)snd::kBufOOB)
+            return SND_ERR_STRIDE;
         switch (params->f.shape.in_dtype) {
             case SND_F32: return snd::launch_wave_bwd_f32(*params, group_ws, (hipStream_t)stream);
             case SND_BF16: return snd::launch_wave_bwd_bf16(*params, group_ws, (hipStream_t)stream);

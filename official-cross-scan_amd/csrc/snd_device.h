@@ -726,6 +726,38 @@ __device__ __forceinline__ void wave_st(T *base, uint32_t off, const float (&v)[
         for (int e = 0; e < CPL; ++e) stg_b(base, off + e * (uint32_t)sizeof(T), v[e]);
     }
 }
+// Stores and float atomics that take their own out-of-range lanes out: buffer instructions check a lane's offset against
+// the descriptor's size in hardware and drop the lane if it is beyond, so a lane that is to do nothing is given the
+// offset kBufOOB instead of a branch or an exec mask around the instruction.  The wave kernels' backward uses them for
+// planes that are not whole bands x whole segments: with a branch around a store on some paths the waits the compiler
+// derives for the prefetched loads have to assume the store was not issued (one counter, decremented in issue order),
+// which cost such planes 12-38 % (64 x 192 x 56x63 against 56x64, one state; 2 x 256 x 512x250 against 512x256).
+// The descriptor spans [base, base + kBufOOB); the scalar offset (a state's plane) is not part of the check.
+constexpr uint32_t kBufOOB = 0xFFFFFFF0u;
+typedef uint32_t buf_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buf_rsrc(void *base) { return __builtin_amdgcn_make_buffer_rsrc(base, 0, kBufOOB, 0x00020000); }
+__device__ __forceinline__ void buf_add_f32(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t soff, float v) {
+    __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, r, off, soff, 0);
+}
+__device__ __forceinline__ uint16_t bits16(const bf16_t *, float v) { return (uint16_t)f32_to_bf16(v); }
+__device__ __forceinline__ uint16_t bits16(const f16_t *, float v) { return __builtin_bit_cast(uint16_t, (f16_t)v); }
+__device__ __forceinline__ uint16_t bits16(const float *, float) { return 0; }
+// CPL values to consecutive elements in memory order (wave_st through a buffer descriptor)
+template <typename T, int CPL, bool VEC>
+__device__ __forceinline__ void wave_st_buf(__amdgpu_buffer_rsrc_t r, uint32_t off, const float (&v)[CPL]) {
+    const T *const tp = nullptr;
+    if (CPL == 2 && VEC && sizeof(T) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b64((buf_u2){__builtin_bit_cast(uint32_t, v[0]), __builtin_bit_cast(uint32_t, v[CPL - 1])}, r, off, 0, 0);
+    } else if (CPL == 2 && VEC) {
+        __builtin_amdgcn_raw_buffer_store_b32((uint32_t)bits16(tp, v[0]) | ((uint32_t)bits16(tp, v[CPL - 1]) << 16), r, off, 0, 0);
+    } else {
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) {
+            if (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v[e]), r, off + e * 4u, 0, 0);
+            else __builtin_amdgcn_raw_buffer_store_b16(bits16(tp, v[e]), r, off + e * 2u, 0, 0);
+        }
+    }
+}
 // Block barrier for hand-overs through LDS only: waits for this wave's LDS traffic, not for its global loads
 // and stores (the prefetched rows and the row just written stay in flight across it; __syncthreads would
 // drain them at every step).

@@ -211,6 +211,9 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
     T *ddb = (T *)p.ddelta + ((int64_t)b * Dm + cB) * H * W;
     float *dBg = p.dB + ((int64_t)b * G + g) * N * H * W;               // dense [b, g, N, H, W]
     float *dCg = p.dC + ((int64_t)b * G + g) * N * H * W;
+    // (stores and atomics go through buffer descriptors: lanes and rows outside the plane are dropped by the hardware's
+    // range check instead of a branch, see buf_rsrc() in snd_device.h)
+    const __amdgpu_buffer_rsrc_t rdu = buf_rsrc(dub), rdd = buf_rsrc(ddb), rdB = buf_rsrc(dBg), rdC = buf_rsrc(dCg);
     // byte steps from one scan row to the next (negative when the group scans bottom-up) and column offsets
     const int UhB = (int)f.u_h_stride * ESZ * rs, DhB = (int)f.delta_h_stride * ESZ * rs, BhB = (int)f.B_h_stride * ESZ * rs,
               ChB = (int)f.C_h_stride * ESZ * rs, DohB = (int)p.dout_h_stride * DSZ * rs, WB = W * ESZ * rs, W4 = W * 4 * rs;
@@ -383,13 +386,17 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                     for (int t = 0; t < CPL; ++t) bn_[r][n][CPL - 1 - t] = mirror(bm[t]);
                 }
             }
+            // (every row of the band, also those past the plane's last row in a ragged last band: they read the last row's
+            // inputs again, their dout is taken as zero below, and nothing of them is stored)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                if (EVEN || i0 + r < H) {
+                {
                     const float (&dln)[CPL] = dln_[r], (&dlun)[CPL] = dlun_[r];
 #pragma unroll
                     for (int n = 0; n < NS; ++n) {
-                        const float hin = bcast(cur.ch[n], r + 1), sin_ = bcast(cur.cs[n], r + 1), ain = bcast(cur.ca[n], r + 1);
+                        // (rows past the plane's last have no column checkpoint: zeros, so that what is computed there is finite)
+                        const bool rin = EVEN || i0 + r < H;
+                        const float hin = rin ? bcast(cur.ch[n], r + 1) : 0.f, sin_ = rin ? bcast(cur.cs[n], r + 1) : 0.f, ain = rin ? bcast(cur.ca[n], r + 1) : 0.f;
                         float a[CPL], bu[CPL], y[CPL], h[CPL], s[CPL];
 #pragma unroll
                         for (int k = 0; k < CPL; ++k) {
@@ -416,11 +423,6 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                         }
                         hdiag[n] = hin;
                     }
-                } else {
-#pragma unroll
-                    for (int n = 0; n < NS; ++n)
-#pragma unroll
-                        for (int t = 0; t < CPL; ++t) { hT[r][n][t] = 0.f; sT[r][n][t] = 0.f; aT[r][n][t] = 0.f; }
                 }
             }
         }
@@ -437,17 +439,20 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
         // (column groups) what the group on the right left for this band goes where a wave on the right would have put
         // it: the group's last wave fills its own neighbour slot, one word per lane, and the rows below read it as ever
         if (EXT && !SPL && ext_in && lane < kExtLanes) ((float *)&sHO[(step + 1) & 1][kc][nseg][er][(el / R) % NS])[eq] = cur.e;
-        const int rows = EVEN ? R : min(R, H - i0);  // rows of this band inside the plane
-        const int mlast = mad24(i0 + rows - 1, rs, r0m);
+        // (from the band's last row up, rows past the plane's last included: their offsets are never used)
+        const int mlast = mad24(i0 + R - 1, rs, r0m);
         uint32_t og = mad24(mlast, WB * rs, colG), o4 = mad24(mlast, W4 * rs, col4);   // du / ddelta and dB / dC offsets of the row
 #pragma unroll
         for (int r = R - 1; r >= 0; --r) {
-            if (EVEN || i0 + r < H) {
+            {
+                // whether this lane's cells of the row are inside the plane: outside, dout counts as zero - which makes
+                // every adjoint there exactly zero - and nothing is stored or added
+                const bool in_plane = jin && (EVEN || i0 + r < H);
                 float dov[CPL], dlu[CPL], qsum[CPL], psum[CPL];
                 unpack(cur.o[r], dov);
 #pragma unroll
                 for (int t = 0; t < CPL; ++t) {
-                    dov[t] = jin ? wm * dov[t] : 0.f;
+                    dov[t] = in_plane ? wm * dov[t] : 0.f;
                     dlu[t] = dl[r][t] * uu[r][t];
                     qsum[t] = 0.f;
                     psum[t] = 0.f;
@@ -456,7 +461,7 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                 for (int n = 0; n < NS; ++n) {
                     // what the segment on the right left for this row: G, Gs, a at column S*(w+1)
                     const float4 in = (PK > 1 && NS <= 2) ? make_float4(0.f, 0.f, 0.f, 0.f) : sHO[(step + 1) & 1][kc][w + 1][r][n];   // (packed planes have no neighbour)
-                    const float hin = bcast(cur.ch[n], r + 1);                 // h[i, S*w-1]
+                    const float hin = (EVEN || i0 + r < H) ? bcast(cur.ch[n], r + 1) : 0.f;   // h[i, S*w-1]
                     float Bv[CPL], Cv[CPL], a[CPL], bu[CPL], dyC[CPL], z[CPL], ya[CPL], ys[CPL], Gt[CPL], Gst[CPL];
                     unpack(cur.b[r][n], Bv);
                     unpack(cur.c[r][n], Cv);
@@ -500,13 +505,14 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                     if (CHB > 1) {
                         sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2][lane] = active ? ya[0] : 0.f;
                         sX[kXBuf == 2 ? step & 1 : 0][wi][(r * NS + n) * 2 + 1][lane] = active ? ys[0] : 0.f;
-                    } else if (jin && (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f)) {
+                    } else if (!(SND_WAVE_ABLATE & 64) || ya[0] == 1234.5f) {
 #pragma unroll
                         for (int e = 0; e < CPL; ++e) {                                // memory order
                             const int t = fh ? e : CPL - 1 - e;
                             const float vb = (CPL == 2 && t == 1) ? ya[CPL - 1] : ya[0], vc = (CPL == 2 && t == 1) ? ys[CPL - 1] : ys[0];
-                            wave_glb_add((float *)((char *)dBg + n * HW4 + o4) + e, vb);
-                            wave_glb_add((float *)((char *)dCg + n * HW4 + o4) + e, vc);
+                            const uint32_t off = in_plane ? o4 + 4u * e : kBufOOB;
+                            buf_add_f32(rdB, off, (uint32_t)(n * HW4), vb);
+                            buf_add_f32(rdC, off, (uint32_t)(n * HW4), vc);
                         }
                     }
                     GdEdge[n] = in.x;
@@ -527,7 +533,7 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                         st2_coherent(d + 4 * R, a[CPL - 1], tg);
                     }
                 }
-                if (jin) {
+                {
                     float duv[CPL], ddl[CPL];
 #pragma unroll
                     for (int t = 0; t < CPL; ++t) {
@@ -542,8 +548,8 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                         t_ = ddl[0]; ddl[0] = ddl[CPL - 1]; ddl[CPL - 1] = t_;
                     }
                     if (!(SND_WAVE_ABLATE & 128) || duv[0] == 1234.5f) {
-                        wave_st<T, CPL, VEC>(dub, og, duv);
-                        wave_st<T, CPL, VEC>(ddb, og, ddl);
+                        wave_st_buf<T, CPL, VEC>(rdu, in_plane ? og : kBufOOB, duv);
+                        wave_st_buf<T, CPL, VEC>(rdd, in_plane ? og : kBufOOB, ddl);
                     }
                 }
                 og -= WB;
@@ -563,8 +569,9 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
                 for (int q = 0; q < CHB; ++q)
 #pragma unroll
                     for (int k = 0; k < PK; ++k) v += sX[kXBuf == 2 ? step & 1 : 0][w + q * nseg][it][PK > 1 ? sl + k * S : lane];
-                float *dst = (float *)((char *)((it & 1) ? dCg : dBg) + n * HW4 + (int64_t)mad24(mad24(i0 + r, rs, r0m), W * 4, (int)col4));
-                if (jin && (PK == 1 || lane < S) && (EVEN || i0 + r < H)) wave_glb_add(dst, v);
+                const uint32_t off = mad24(mad24(i0 + r, rs, r0m), W * 4, (int)col4);
+                const bool in_plane = jin && (PK == 1 || lane < S) && (EVEN || i0 + r < H);
+                buf_add_f32(buf_rsrc((it & 1) ? dCg : dBg), in_plane ? off : kBufOOB, (uint32_t)(n * HW4), v);
             }
             if (kXBuf == 1) lds_barrier();
             ++step;
@@ -574,7 +581,7 @@ __global__ __launch_bounds__(64 * (XW + (SPL ? 1 : 0))) void wave_bwd_kernel(con
     In sA;
     if (PF) load_band(sA, wg.nBands - 1);
     // (nothing in flight on the way into the band loop: its first waits then follow the loop's own path as well)
-    if (PF && EVEN) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    if (PF) __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
     lds_barrier();                                   // the zeroed slot
     if (SPL) lds_barrier();                          // (and what the block's extra wave has fetched for the first band)
     if (multi)
