@@ -35,6 +35,11 @@ def draw(seed):
         c.update(W=int(r.randint(513, 1501)), H=int(r.randint(1, 13)), Bt=int(r.randint(1, 3)), Dm=K * min(rg, 4),
                  sched=int(r.choice([capi.SCHED_AUTO, capi.SCHED_WAVEFRONT])))
         c["Dd"] = c["Dm"] // 2 if (c["share_delta"] and c["Dm"] % 2 == 0) else c["Dm"]
+    if c["N"] <= 2 and seed % 8 == 1:
+        # 128 to 256 planes of eight row segments: the backward cuts them in two halves that run side by side
+        c.update(W=int(r.randint(449, 513)), H=int(r.randint(1, 13)), Bt=1, K=4, sched=int(r.choice([capi.SCHED_AUTO, capi.SCHED_WAVEFRONT])))
+        c["Dm"] = 4 * int(r.randint(32, 65))
+        c["Dd"] = c["Dm"] // 2 if c["share_delta"] else c["Dm"]
     if c["N"] >= 9 and seed % 4 == 3:
         # the 16-lane backward with its strips cut into column segments (forced: the model only cuts large launches)
         c.update(sched=capi.SCHED_STRIPS, segments=int(r.choice([2, 3, 4])), W=max(c["W"], 20))
