@@ -435,9 +435,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     float dw_acc = 0.f;
 
     // dB, dC of a tile leave the block (summed over its channels) one tile late, from the partial sums that stay
-    // in LDS until the next sweep: after the next tile's inputs have arrived, so that the wait for those inputs
-    // does not also cover the acknowledgement of these atomics, which then complete under the sweep
-    // (4 % of the backward at B=2, D=192, 200x336 under the strip pipeline; nothing at B=64, 56x56).
+    // in LDS until the next sweep: between the requests for the next tile's inputs and the wait for them, so that the
+    // LDS reads and the address arithmetic of the flush fall under the latency of those loads (B=64, D=192, 56x56:
+    // 1.279 -> 1.245 ms against the flush behind the wait; with the sums in front of the wait and the atomics behind it
+    // the eight values kept across the wait are spilled and nothing more is gained, and the per-pixel epilogue moved
+    // to the same place gains nothing either).
     int pI = -1, pJ = 0;                            // the tile whose partial sums are still in LDS
     auto flush_bc = [&](int I_, int J_) __attribute__((always_inline)) {
         SND_THREAD_MAPS(NP);
@@ -478,7 +480,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             }
             __syncthreads();
             const float *src = colstate + (tid << 1);
-            const bool bad = *(volatile int *)&sDead != 0;   // the wait timed out: poison everything downstream
+            const bool bad = lds_peek(&sDead) != 0;   // the wait timed out: poison everything downstream
 #pragma unroll
             for (int r = 0; r < kRows; r += 2) {
                 ld2_coherent(src + (r >> 1) * 512, GR[r], GR[r + 1]);
@@ -527,7 +529,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             // pipelined band - by another block.  It is requested here if it is known to be there (own
             // rows; rows whose hand-over an earlier poll has already seen), else after the wait below.
             const bool handed = PIPE && I == I_hi && I + 1 < geo.nCY;
-            const bool late = handed && __builtin_amdgcn_readfirstlane(*(volatile int *)&sSeen) < geo.nCX - J;
+            const bool late = handed && __builtin_amdgcn_readfirstlane(lds_peek(&sSeen)) < geo.nCX - J;
             if (!late) {
                 if (I + 1 < geo.nCY && lvalid) {
                     const float *src = gdown + (int64_t)J * DN8;
@@ -545,8 +547,8 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
             }
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
+            if (pI >= 0) flush_bc(pI, pJ);          // the previous tile's dB, dC, under the latency of the loads just requested
             commit(I, J);
-            if (pI >= 0) flush_bc(pI, pJ);          // the previous tile's dB, dC
             pI = I; pJ = J;
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                     for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
                 }
             }
-            if (handed && *(volatile int *)&sDead) {   // the wait timed out: poison everything downstream
+            if (handed && lds_peek(&sDead)) {   // the wait timed out: poison everything downstream
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) Gd[j] = __builtin_nanf("");
             }

@@ -147,6 +147,12 @@ __device__ __forceinline__ void st_f32_b(void *base, uint32_t off, int dt, float
     else if (dt == SND_BF16) *(uint16_t *)q = f32_to_bf16(v);
     else *(f16_t *)q = (f16_t)v;
 }
+// A word of LDS that another wave of the block may have written since the last barrier: a plain LDS load.  (Read
+// through a volatile generic pointer it becomes a flat load, and the wait for a flat load also covers every global
+// load the wave has in flight.)
+__device__ __forceinline__ int lds_peek(const int *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
 // float add to global memory, no value returned (one L2 atomic)
 __device__ __forceinline__ void glb_add(float *p, float v) {
     __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -373,7 +373,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
             float corner = 0.f;                     // h[r0-1][j0-1]
             if (handed) {
                 fetch_row_above(J, hup);
-                if (*(volatile int *)&sDead) {      // the wait timed out: poison everything downstream
+                if (lds_peek(&sDead)) {      // the wait timed out: poison everything downstream
 #pragma unroll
                     for (int j = 0; j < kCkX; ++j) hup[j] = __builtin_nanf("");
                 }
