@@ -135,6 +135,10 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
     const uint32_t cUb = (uint32_t)(p.u_shared ? cc - g * rg : cc) * (uint32_t)p.u_d_stride * ESZ, cDb = (uint32_t)(cc / rd) * (uint32_t)p.delta_d_stride * ESZ;
     const int BhB = (int)p.B_h_stride * ESZ, ChB = (int)p.C_h_stride * ESZ, UhB = (int)p.u_h_stride * ESZ, DhB = (int)p.delta_h_stride * ESZ;
     const int OhB = (int)p.out_h_stride * esz_out;
+    // (VEC) the gathered rows of out leave four columns per access if every row of out starts on a four-element boundary
+    // (the fused merge adds with atomics, element by element)
+    const bool ovec = VEC && !merge && ((uintptr_t)p.out & (uintptr_t)(4 * esz_out - 1)) == 0 && p.out_batch_stride % 4 == 0 &&
+                      p.out_d_stride % 4 == 0 && p.out_h_stride % 4 == 0;
     const int64_t BsB = p.B_dstate_stride * ESZ, CsB = p.C_dstate_stride * ESZ;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);   // the wave index as a scalar
 
@@ -529,6 +533,24 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(NP >= 8
                 __syncthreads();
                 const int c0 = (J - jq) * TE, ncols = min((jq + 1) * TE, W - c0);
                 constexpr int PER_CH = kRows * QC;
+                if (VEC && ovec) {
+                    constexpr int Q4 = QC / 4;      // four-column groups per gathered row
+#pragma unroll 1
+                    for (int idx = tid; idx < CB * kRows * Q4; idx += 16 * NP) {
+                        const int ch = idx / (kRows * Q4), rr = (idx / Q4) & 7, c4 = (idx & (Q4 - 1)) * 4;
+                        const int row = r0 + rr;
+                        if (row < H && c4 < ncols && cbase + ch < cend && !(SND_TILE_ABLATE & 1)) {
+                            const float4 v = *(const float4 *)(sOut + ch * OCH + rr * OROW + c4);
+                            float a4[4] = {v.x, v.y, v.z, v.w};
+                            if (fh) { a4[0] = v.w; a4[1] = v.z; a4[2] = v.y; a4[3] = v.x; }   // scan order -> memory order
+                            const uint32_t o = (uint32_t)(cbase + ch) * (uint32_t)p.out_d_stride * esz_out +
+                                               mad24(mrow(row), OhB, mcol(c0 + c4 + (fh ? 3 : 0)) << sh_out);
+                            if (p.out_dtype == SND_F32) stg4_b((float *)outb, o, a4);
+                            else if (p.out_dtype == SND_BF16) stg4_b((bf16_t *)outb, o, a4);
+                            else stg4_b((f16_t *)outb, o, a4);
+                        }
+                    }
+                } else
 #pragma unroll 4
                 for (int idx = tid; idx < CB * PER_CH; idx += 16 * NP) {
                     const int ch = idx / PER_CH, rr = (idx / QC) & 7, c32 = idx & (QC - 1);

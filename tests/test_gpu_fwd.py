@@ -99,6 +99,35 @@ def test_fwd_half_inputs(gpu_device, dtype, out_float):
     assert relerr(o, ref_r) <= (1e-4 if out_float else tol16)
 
 
+@pytest.mark.parametrize("dtype,out_float", [(torch.float32, True), (torch.bfloat16, False), (torch.float16, False)])
+def test_fwd_gathered_out_rows_vector_and_element_stores(gpu_device, dtype, out_float):
+    """Planes of more than two column tiles gather out over four tiles and write whole rows: four columns per store
+    when the rows of out start on four-element boundaries, element by element otherwise, in memory order under a
+    mirrored column order (directions = corners) too.  Against the oracle through flips, and one against the other."""
+    from test_gpu_corners import flip_groups_np
+    Bt, Dm, H, W, N, K = 1, 32, 17, 40, 16, 4
+    d = O.make_inputs(Bt, Dm, H, W, N=N, K=K, seed=12, with_dout=False)
+    t = to_dev(d, gpu_device, dtype)
+    rd = {k: t[k].float().cpu().numpy() for k in ("u", "delta", "B", "C")}
+    f = capi.FwdCall(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["delta_bias"], True, out_float, None, True,
+                     capi.SCHED_AUTO, capi.DIR_CORNERS)
+    f.launch()
+    torch.cuda.synchronize()
+    fu, fd, fB, fC = (flip_groups_np(rd[k], K) for k in ("u", "delta", "B", "C"))
+    ref = flip_groups_np(O.selective_nd_scan_fwd(fu, fd, d["A"], fB, fC, d["D"], d["delta_bias"], True), K)
+    tol = 1e-4 if out_float else (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    assert relerr(f.out.float().cpu().numpy(), ref) <= tol
+    want = f.out.clone()
+    big = torch.zeros(Bt, Dm, H, W + 3, dtype=want.dtype, device=gpu_device)
+    o2 = big[..., 3:]                                   # rows three elements past a four-element boundary
+    f.params.out = o2.data_ptr()
+    f.params.out_batch_stride, f.params.out_d_stride, f.params.out_h_stride = o2.stride(0), o2.stride(1), o2.stride(2)
+    f.launch()
+    torch.cuda.synchronize()
+    assert torch.equal(o2, want)
+    assert not big[..., :3].any()
+
+
 def test_fwd_strided_inputs(gpu_device):
     """Only the last dimension has to be contiguous (selective_scan_oflex.cpp:203-204,227,229)."""
     d = O.make_inputs(2, 8, 9, 12, N=16, K=2, seed=8, with_dout=False)
