@@ -254,7 +254,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 const int row = min(r0 + (q >> 1), H - 1), col = min(j0 + (q & 1) * 4, W - 4);
                 return (uint32_t)mad24(mrow(row), hB, mcol(col + (fh ? 3 : 0)) * esz);
             };
-            {
+            uint32_t z_ = 0;                        // (timing studies) what a load that is switched off leaves in its registers
+            if (SND_TILE_ABLATE & 112) asm volatile("v_mov_b32 %0, 0x3e000000" : "=v"(z_));
+            if (SND_TILE_ABLATE & 16) {
+                for (int e = 0; e < (int)sizeof(T); ++e) { vb.w[e] = z_; vc.w[e] = z_; }
+            } else {
                 const int sn = min(t_ >> 4, N - 1), q = t_ & 15;
                 ldraw4_b(vb, (const T *)((const char *)Bb + sn * BsB), chunk_off(q, BhB, ESZ));
                 ldraw4_b(vc, (const T *)((const char *)Cb + sn * CsB), chunk_off(q, ChB, ESZ));
@@ -262,6 +266,11 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 #pragma unroll
             for (int k = 0; k < NCH; ++k) {
                 const int q = n + NP * k;
+                if (SND_TILE_ABLATE & 32) {
+                    for (int e = 0; e < (int)sizeof(T); ++e) { vdl[k].w[e] = z_; vu[k].w[e] = z_; }
+                    for (int e = 0; e < 4; ++e) vdo[k][e] = z_;
+                    continue;
+                }
                 ldraw4_b(vdl[k], db, cDb + chunk_off(q, DhB, ESZ));
                 ldraw4_b(vu[k], ub, cUb + chunk_off(q, UhB, ESZ));
                 const char *src = (const char *)dob + (cDob + chunk_off(q, DohB, esz_do));
@@ -278,6 +287,7 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 int rr, jj;
                 halo_cell(n + NP * k, rr, jj);
                 const int row = min(max(r0 + rr, 0), H - 1), col = min(max(j0 + jj, 0), W - 1);
+                if (SND_TILE_ABLATE & 64) { vh[k] = z_; continue; }
                 vh[k] = ldraw_b(db, cDb + mad24(mrow(row), DhB, mcol(col) * ESZ));
             }
             return;

@@ -289,16 +289,16 @@ constexpr int kErrorWord = 1, kTicketWord = 4, kSyncHeader = 12;
 constexpr int kSpinLimit = 1 << 21;                 // default polls (a memory round trip each) before giving up
 // The limit launches use: kSpinLimit unless snd_debug_set_spin_limit() lowered it (tests of the time-out path).
 int spin_limit();
-__host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips) {
 // Timing studies of the tile kernels only (-DSND_TILE_ABLATE=<bits>, results wrong, never shipped): one memory
 // stream of a kernel is switched off or pointed at one hot tile, and the time that goes away prices it.
 // Forward: 1 no out stores, 2 staging loads from tile (0,0), 4 no checkpoint stores, 8 row-above loads from one
 // tile.  Backward: 1 no dB/dC atomics, 2 staging loads from tile (0,0), 4 no du/ddelta stores, 8 checkpoint loads
-// from one tile.
+// from one tile; (vector staging) 16 no loads of B and C, 32 none of delta, u and dout, 64 none of the halo of
+// delta - their registers hold a constant instead.
 #ifndef SND_TILE_ABLATE
 #define SND_TILE_ABLATE 0
 #endif
-
+__host__ __device__ inline int64_t sync_words(int64_t nPlaneChunks, int nStrips) {
     // per (plane chunk, strip): tiles handed over, then column segments finished
 #ifdef SND_PIPE_TRACE   // timing study only: 4 extra words per job (start, end, time spent waiting, -)
     return (kSyncHeader + 6 * nPlaneChunks * nStrips + 3) / 4 * 4;
