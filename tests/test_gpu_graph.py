@@ -17,6 +17,8 @@ pytestmark = pytest.mark.gpu
                                         (capi.SCHED_WAVEFRONT, (4, 160, 14, 14, 1)), (capi.SCHED_WAVEFRONT, (2, 16, 40, 150, 2)),
                                         # a wide plane: three launches per kernel (column groups) handing over through memory
                                         (capi.SCHED_WAVEFRONT, (1, 8, 12, 1300, 2)),
+                                        # split planes: two halves of a plane side by side, tagged words between them (backward)
+                                        (capi.SCHED_WAVEFRONT, (1, 128, 9, 512, 1)),
                                         # strips of the 16-lane backward cut into three column segments (forced)
                                         (-3, (2, 16, 40, 100, 16))])
 def test_graph_replays_match_eager(gpu_device, sched, dims):
@@ -71,3 +73,5 @@ def _graph_replays(gpu_device, sched, dims):
             assert relerr(a.cpu().numpy(), w.cpu().numpy()) <= tol, (rep, i)
         if sched not in (capi.SCHED_PLANE, capi.SCHED_WAVEFRONT):
             assert int(f.ws.view(torch.int32)[1]) == 0 and int(b.ws.view(torch.int32)[1]) == 0
+        elif sched == capi.SCHED_WAVEFRONT and f.plan.wavefront_workspace:
+            assert int(b.ws.view(torch.int32)[1]) == 0   # no hand-over wait of a wide or split plane gave up
