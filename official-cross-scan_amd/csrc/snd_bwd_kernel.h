@@ -62,7 +62,7 @@ __device__ __forceinline__ void rows_scatter4x2(float &b0, float &b1, float &b2,
 #define SND_BWD_WAVES 2
 #endif
 #ifndef SND_KA8
-#define SND_KA8 2
+#define SND_KA8 3
 #endif
 // VEC: the tile's inputs are staged, and du / ddelta stored, four columns at a time with one 16-byte (fp32) or
 // 8-byte (16-bit) access per thread and tensor instead of one access per element - a quarter of the memory
@@ -212,14 +212,20 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     //   x_v [b][I][J][half][c][n][4 cols]   x, x_sd [b][J][I][half][c][n][4 rows]   scratch G row [b][J][half][c][n][4 cols]
     const int64_t DN8 = (int64_t)Dm * N * 8;
     const int64_t DN4 = DN8 / 2;
-    const int64_t lane_off = ((int64_t)cc * N + nn) * 4;
-    const float *xv = f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8 + lane_off;
-    const float *xh = f.x + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
-    const float *xs = f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8 + lane_off;
+    // Addressed as a wave-uniform base (batch image, tile) plus one 32-bit byte offset per lane, laneB: one register for
+    // all of them across the tile loop instead of a 64-bit pointer per array.
+    const uint32_t laneB = (uint32_t)(cc * N + nn) * 16u;              // the lane's four floats inside a half tile
+    const char *xv = (const char *)(f.x_v + (int64_t)b * geo.nCY * geo.nCX * DN8);
+    const char *xh = (const char *)(f.x + (int64_t)b * geo.nCX * geo.nCY * DN8);
+    const char *xs = (const char *)(f.x_sd + (int64_t)b * geo.nCX * geo.nCY * DN8);
+    auto ck4 = [&](const char *tile, int64_t floats) __attribute__((always_inline)) {   // 16 bytes of this lane, `floats` into the tile
+        return *(const float4 *)(tile + floats * 4 + laneB);
+    };
     // hand-over between blocks (pipelined schedules): [J][pair k][c][n][2], so that a wave's 8-byte
-    // coherent accesses cover whole lines too
+    // coherent accesses cover whole lines too (the lane's offset there is half of laneB)
     const int64_t DN2 = (int64_t)Dm * N * 2;
-    float *gdown = (float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8 + (PIPE ? ((int64_t)cc * N + nn) * 2 : lane_off);
+    char *gdown = (char *)((float *)p.workspace + nSync + (int64_t)b * geo.nCX * DN8);
+    const uint32_t laneG = PIPE ? laneB >> 1 : laneB;
 
     const float *myDl = sDl + cl * DLP;
     const float *myDu = sDu + cl * PCH;
@@ -513,20 +519,21 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             float hu[kCkX], hlft[kRows], slft[kRows], hc = 0.f;   // h row above, h/s column to the left
             float Gd[kCkX];                                        // G of the row below
             if (I > 0) {
-                const float *src = xv + ((SND_TILE_ABLATE & 8) ? 1 : ((int64_t)(I - 1) * geo.nCX + J)) * DN8;
-                const float4 v0 = *(const float4 *)src, v1 = *(const float4 *)(src + DN4);
+                const char *src = xv + ((SND_TILE_ABLATE & 8) ? 1 : ((int64_t)(I - 1) * geo.nCX + J)) * DN8 * 4;
+                const float4 v0 = ck4(src, 0), v1 = ck4(src, DN4);
                 hu[0] = v0.x; hu[1] = v0.y; hu[2] = v0.z; hu[3] = v0.w;
                 hu[4] = v1.x; hu[5] = v1.y; hu[6] = v1.z; hu[7] = v1.w;
-                if (J > 0) hc = src[((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8];   // last column of the tile on the left
+                if (J > 0)                          // last column of the tile on the left
+                    hc = *(const float *)(src + (((TE - 1) >> 2) * DN4 + ((TE - 1) & 3) - DN8) * 4 + laneB);
             } else {
 #pragma unroll
                 for (int j = 0; j < kCkX; ++j) hu[j] = 0.f;
             }
             if (J > 0) {
-                const float *sh_ = xh + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8;
-                const float *ss_ = xs + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8;
-                const float4 h0 = *(const float4 *)sh_, h1 = *(const float4 *)(sh_ + DN4);
-                const float4 s0 = *(const float4 *)ss_, s1 = *(const float4 *)(ss_ + DN4);
+                const char *sh_ = xh + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8 * 4;
+                const char *ss_ = xs + ((SND_TILE_ABLATE & 8) ? 0 : ((int64_t)(J - 1) * geo.nCY + I)) * DN8 * 4;
+                const float4 h0 = ck4(sh_, 0), h1 = ck4(sh_, DN4);
+                const float4 s0 = ck4(ss_, 0), s1 = ck4(ss_, DN4);
                 hlft[0] = h0.x; hlft[1] = h0.y; hlft[2] = h0.z; hlft[3] = h0.w;
                 hlft[4] = h1.x; hlft[5] = h1.y; hlft[6] = h1.z; hlft[7] = h1.w;
                 slft[0] = s0.x; slft[1] = s0.y; slft[2] = s0.z; slft[3] = s0.w;
@@ -542,12 +549,12 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             const bool late = handed && __builtin_amdgcn_readfirstlane(lds_peek(&sSeen)) < geo.nCX - J;
             if (!late) {
                 if (I + 1 < geo.nCY && lvalid) {
-                    const float *src = gdown + (int64_t)J * DN8;
+                    const char *src = gdown + (int64_t)J * DN8 * 4;
                     if (PIPE) {
 #pragma unroll
-                        for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
+                        for (int k = 0; k < kCkX; k += 2) ld2_coherent((const float *)(src + (k >> 1) * DN2 * 4 + laneG), Gd[k], Gd[k + 1]);
                     } else {
-                        const float4 v0 = *(const float4 *)src, v1 = *(const float4 *)(src + DN4);
+                        const float4 v0 = *(const float4 *)(src + laneG), v1 = *(const float4 *)(src + DN4 * 4 + laneG);
                         Gd[0] = v0.x; Gd[1] = v0.y; Gd[2] = v0.z; Gd[3] = v0.w;
                         Gd[4] = v1.x; Gd[5] = v1.y; Gd[6] = v1.z; Gd[7] = v1.w;
                     }
@@ -577,9 +584,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
 
             if (late) {                             // only after the wait above
                 if (I + 1 < geo.nCY && lvalid) {
-                    const float *src = gdown + (int64_t)J * DN8;
+                    const char *src = gdown + (int64_t)J * DN8 * 4;
 #pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) ld2_coherent(src + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
+                    for (int k = 0; k < kCkX; k += 2) ld2_coherent((const float *)(src + (k >> 1) * DN2 * 4 + laneG), Gd[k], Gd[k + 1]);
                 } else {
 #pragma unroll
                     for (int j = 0; j < kCkX; ++j) Gd[j] = 0.f;
@@ -782,13 +789,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
             GRc = gd_old0;
             const bool hands_over = PIPE && I == I_lo && I > 0;   // top strip of a band: another block takes the row
             if (I > 0 && lvalid) {                  // adjoint row for the strip above
-                float *dst = gdown + (int64_t)J * DN8;
+                char *dst = gdown + (int64_t)J * DN8 * 4;
                 if (PIPE) {
 #pragma unroll
-                    for (int k = 0; k < kCkX; k += 2) st2_coherent(dst + (k >> 1) * DN2, Gd[k], Gd[k + 1]);
+                    for (int k = 0; k < kCkX; k += 2) st2_coherent((float *)(dst + (k >> 1) * DN2 * 4 + laneG), Gd[k], Gd[k + 1]);
                 } else {
-                    *(float4 *)dst = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
-                    *(float4 *)(dst + DN4) = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
+                    *(float4 *)(dst + laneG) = make_float4(Gd[0], Gd[1], Gd[2], Gd[3]);
+                    *(float4 *)(dst + DN4 * 4 + laneG) = make_float4(Gd[4], Gd[5], Gd[6], Gd[7]);
                 }
             }
             __builtin_amdgcn_s_setprio(0);
