@@ -258,10 +258,13 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // not a multiple of 2 MiB apart); everywhere else it follows dB directly and nothing beyond the two is filled.
     const bool spread = c.plan.auto_schedule == SND_SCHED_WAVEFRONT && nBC * 4 >= (int64_t)(2 << 20);
     const int64_t oC = spread ? (round_2mib(nBC * 4) + c.plan.dC_skew_bytes) / 4 : round64(nBC);
-    at::Tensor accBC = spread ? torch::empty({oC + nBC}, f32) : torch::zeros({oC + nBC}, f32);
+    // one fill (and, for 16-bit inputs, one cast) over both where the gap between them is small beside them, else one
+    // per tensor
+    const bool whole = (oC - nBC) * 4 <= nBC;
+    at::Tensor accBC = whole ? torch::zeros({oC + nBC}, f32) : torch::empty({oC + nBC}, f32);
     at::Tensor dB = accBC.narrow(0, 0, nBC).view(B.sizes());
     at::Tensor dC = accBC.narrow(0, oC, nBC).view(C.sizes());
-    if (spread) { dB.zero_(); dC.zero_(); }         // (not the gap between them)
+    if (!whole) { dB.zero_(); dC.zero_(); }         // (not the gap between them)
     const int64_t oD = round64(nA), oBias = oD + round64(dim), oDec = oBias + round64(dim), oMerge = oDec + 64;
     at::Tensor accP = torch::zeros({oMerge + (merge ? round64(dim) : 0)}, f32);
     at::Tensor dA = accP.narrow(0, 0, nA).view({dim, dstate});
@@ -303,7 +306,7 @@ std::vector<at::Tensor> selective_scan_bwd(const at::Tensor &u, const at::Tensor
     // (16-bit inputs: one cast kernel for the two tensors, which share a buffer)
     at::Tensor dBo = dB, dCo = dC;
     if (B.scalar_type() != at::ScalarType::Float) {
-        if (spread) {                               // two casts of the live ranges, not one of the gap as well
+        if (!whole) {                               // two casts of the live ranges, not one of the gap as well
             dBo = dB.to(B.dtype());
             dCo = dC.to(C.dtype());
         } else {
