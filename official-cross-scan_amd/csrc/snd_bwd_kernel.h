@@ -453,9 +453,9 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
     // dB, dC of a tile leave the block (summed over its channels) one tile late, from the partial sums that stay
     // in LDS until the next sweep: between the requests for the next tile's inputs and the wait for them, so that the
     // LDS reads and the address arithmetic of the flush fall under the latency of those loads (B=64, D=192, 56x56:
-    // 1.279 -> 1.245 ms against the flush behind the wait; with the sums in front of the wait and the atomics behind it
-    // the eight values kept across the wait are spilled and nothing more is gained, and the per-pixel epilogue moved
-    // to the same place gains nothing either).
+    // 1.290 -> 1.258 ms against the flush behind the wait, which -DSND_BWD_FLUSH_LATE restores for timing; with the
+    // sums in front of the wait and the atomics behind it the eight values kept across the wait are spilled and
+    // nothing more is gained, and the per-pixel epilogue moved to the same place gains nothing either).
     int pI = -1, pJ = 0;                            // the tile whose partial sums are still in LDS
     auto flush_bc = [&](int I_, int J_) __attribute__((always_inline)) {
         SND_THREAD_MAPS(NP);
@@ -564,8 +564,13 @@ __global__ __launch_bounds__(16 * NP) __attribute__((amdgpu_waves_per_eu(SND_BWD
                 }
             }
             prefetch(I, J);                         // no loads in flight across the register-hungry sweep
+#ifndef SND_BWD_FLUSH_LATE
             if (pI >= 0) flush_bc(pI, pJ);          // the previous tile's dB, dC, under the latency of the loads just requested
             commit(I, J);
+#else                                               // (timing study: the flush behind the wait, as it was; same results)
+            commit(I, J);
+            if (pI >= 0) flush_bc(pI, pJ);
+#endif
             pI = I; pJ = J;
             // strip pipeline: the strip below must have handed over tile J.  One wave polls; the
             // others wait at the barrier.
