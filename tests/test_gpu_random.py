@@ -119,8 +119,10 @@ def test_random_case(gpu_device, seed):
             # per-lane partial sums and atomics.  The terms cancel (|sum| is a few percent of sum |term|),
             # so the fp32 rounding of the terms shows up amplified against the sum itself: seed 14
             # (2 x 8 planes of 22 x 10, N = 2) measures 1.0e-4 to 1.2e-4 depending on the order the atomics
-            # land in.  Every other gradient keeps 1e-4.
-            tol = 5e-4
+            # land in.  Every other gradient keeps 1e-4.  A lane's partial sum runs over its whole plane, so the noise
+            # grows with the square root of the plane's cells: the bound scales with it beyond the 44 x 44 of the
+            # default sweep (SND_RANDOM_MAX_HW=200, seed 420: 6.6e-4 at 3 x 160 planes of 82 x 177, N = 12).
+            tol = 5e-4 * max(1.0, (c["H"] * c["W"] / 2000.0) ** 0.5)
         if nm == "dA" and c["H"] == 1:
             # likewise dA of a single row is identically zero, a sum of terms that cancel: what comes back is the fp32
             # rounding noise of that sum on relerr's absolute scale of 1e-2, and it grows with the row (seed 1805:
